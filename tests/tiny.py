@@ -1,0 +1,101 @@
+"""Tiny Qwen2 configurations that differ in every size and option, and helpers that build
+their random model folders and the plain implementation's logits for them."""
+
+from __future__ import annotations
+
+import json
+import random
+from pathlib import Path
+
+import torch
+
+from plain import qwen2_plain as plain
+
+#: A: grouped heads (G=2), tied head, no window, page 16.
+CONFIG_A = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 64,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "intermediate_size": 128,
+    "vocab_size": 256,
+    "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": True,
+    "use_sliding_window": False,
+    "max_position_embeddings": 128,
+}
+PAGE_A = 16
+
+#: B: one KV head for three query heads, head size 32, sizes that are no power of two,
+#: untied head, window 16 from layer 1 on (layer 0 keeps all keys), page 8.
+CONFIG_B = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 96,
+    "num_hidden_layers": 3,
+    "num_attention_heads": 3,
+    "num_key_value_heads": 1,
+    "intermediate_size": 200,
+    "vocab_size": 320,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False,
+    "use_sliding_window": True,
+    "sliding_window": 16,
+    "max_window_layers": 1,
+    "max_position_embeddings": 256,
+}
+PAGE_B = 8
+
+#: C: as many KV heads as query heads, head size 48 with heads * head size != hidden,
+#: an odd vocabulary, linear position scaling, every layer windowed (window 40), page 32.
+CONFIG_C = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 80,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 5,
+    "num_key_value_heads": 5,
+    "head_dim": 48,
+    "intermediate_size": 72,
+    "vocab_size": 301,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "linear", "factor": 2.0},
+    "rms_norm_eps": 3e-6,
+    "tie_word_embeddings": False,
+    "use_sliding_window": True,
+    "sliding_window": 40,
+    "max_window_layers": 0,
+    "max_position_embeddings": 512,
+}
+PAGE_C = 32
+
+TINY = {"A": (CONFIG_A, 0, PAGE_A), "B": (CONFIG_B, 1, PAGE_B), "C": (CONFIG_C, 2, PAGE_C)}
+
+
+def make_model_dir(folder: Path, config: dict, seed: int, dtype: torch.dtype = torch.float32) -> Path:
+    from turboserve_amd.weights.random_init import write_random_model
+
+    return write_random_model(config, folder, seed=seed, dtype=dtype)
+
+
+def read_model_dir(folder: Path) -> tuple[dict, dict[str, torch.Tensor]]:
+    """``(config.json mapping, tensors as float32)`` read without any engine code."""
+    from safetensors.torch import load_file
+
+    config = json.loads((Path(folder) / "config.json").read_text())
+    tensors = load_file(str(Path(folder) / "model.safetensors"))
+    return config, plain.as_float32(tensors)
+
+
+def random_tokens(vocab: int, length: int, seed: int) -> list[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(length)]
+
+
+def plain_logits(folder: Path, tokens: list[int]) -> torch.Tensor:
+    config, tensors = read_model_dir(folder)
+    return plain.forward_logits(config, tensors, tokens)

@@ -1,0 +1,254 @@
+// Row-wise kernels of the decoder: embedding gather, RMSNorm (with the residual sum fused in),
+// SwiGLU, and rotary encoding fused with the scatter of keys and values into cache pages.
+//
+// Formulas restate src/turboserve/engine/model/layers.py:202-208 (RMSNorm), :214-222 and
+// :290-302 (rotary, half-split pairs), :437-440 (SwiGLU) and
+// src/turboserve/engine/core/kv_cache.py:601-631 (cache write at slot = block * BS + offset).
+// Reductions, the residual sum and the rotation are computed in 32-bit whatever T is.
+#include "common.hpp"
+
+// ---------------------------------------------------------------------------------------------
+// embedding: residual[t, :] = float(table[ids[t], :])
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ residual, const T* __restrict__ table,
+                             const int* __restrict__ ids, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  const bool valid = id >= 0 && id < vocab;
+  const T* row = table + (size_t)(valid ? id : 0) * hidden;
+  float* out = residual + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    // An id outside the table is a host error; it yields NaN instead of a read out of bounds.
+    out[i] = valid ? to_float(row[i]) : __uint_as_float(0x7fc00000u);
+  }
+}
+
+extern "C" int ts_embed(void* residual, const void* table, const int* ids, int tokens, int hidden,
+                        int vocab, int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!residual || !table || !ids || hidden < 1 || vocab < 1) return TS_ERR_ARG;
+  dim3 grid(tokens), block(256);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (float*)residual, (const float*)table, ids, hidden, vocab);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (float*)residual, (const bf16_t*)table, ids, hidden, vocab);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// RMSNorm.  y = w * round_T(x * rsqrt(mean(x^2) + eps)): the normalised value is rounded to the
+// storage type before the gain, as the reference does (layers.py:208).
+//
+// add_rmsnorm: s = residual + pending (32-bit); residual = s; y = norm(s).  With `rows` the
+// kernel reads rows[i] and writes y[i] only (residual untouched): the final norm at the wanted
+// positions.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x, const T* __restrict__ w,
+                               float eps, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = to_float(x[base + i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float n = round_to<T>(to_float(x[base + i]) * rstd);
+    y[base + i] = from_float<T>(to_float(w[i]) * n);
+  }
+}
+
+template <typename T>
+__global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residual,
+                                   const T* __restrict__ pending, const T* __restrict__ w,
+                                   const int* __restrict__ rows, float eps, int hidden) {
+  __shared__ float scratch[16];
+  const int src = rows ? rows[blockIdx.x] : blockIdx.x;
+  const size_t in_base = (size_t)src * hidden;
+  const size_t out_base = (size_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  if (rows) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float s = residual[in_base + i];
+      if (pending) s += to_float(pending[in_base + i]);
+      ss += s * s;
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float s = residual[in_base + i];
+      if (pending) {
+        s += to_float(pending[in_base + i]);
+        residual[in_base + i] = s;  // re-read below by this same thread
+      }
+      ss += s * s;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float s = residual[in_base + i];
+    if (rows && pending) s += to_float(pending[in_base + i]);
+    const float n = round_to<T>(s * rstd);
+    y[out_base + i] = from_float<T>(to_float(w[i]) * n);
+  }
+}
+
+extern "C" int ts_rmsnorm(void* y, const void* x, const void* w, float eps, int tokens, int hidden,
+                          int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!y || !x || !w || hidden < 1) return TS_ERR_ARG;
+  dim3 grid(tokens), block(hidden <= 1024 ? 256 : 1024);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, (float*)y, (const float*)x, (const float*)w, eps, hidden);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, eps, hidden);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// `out_rows` = rows of y written: the number of entries of `rows` if given, else the tokens.
+extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, const void* w,
+                              const int* rows, float eps, int out_rows, int hidden, int dtype,
+                              hipStream_t stream) {
+  if (out_rows == 0) return TS_OK;
+  if (!y || !residual || !w || hidden < 1) return TS_ERR_ARG;
+  dim3 grid(out_rows), block(hidden <= 1024 ? 256 : 1024);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, (float*)y, residual, (const float*)pending, (const float*)w, rows, eps, hidden);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, residual, (const bf16_t*)pending, (const bf16_t*)w, rows, eps, hidden);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// SwiGLU over the fused gate|up projection: out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int inter,
+                              size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / inter;
+  const int i = (int)(idx - t * inter);
+  const float g = to_float(gate_up[t * 2 * inter + i]);
+  const float u = to_float(gate_up[t * 2 * inter + inter + i]);
+  const float act = g / (1.f + expf(-g));
+  out[idx] = from_float<T>(act * u);
+}
+
+extern "C" int ts_swiglu(void* out, const void* gate_up, int tokens, int inter, int dtype,
+                         hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!out || !gate_up || inter < 1) return TS_ERR_ARG;
+  const size_t total = (size_t)tokens * inter;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)gate_up, inter, total);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)gate_up, inter, total);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rotary encoding + cache write.  qkv is [T, (Hq + 2 Hkv) * D]: q heads, then k heads, then v
+// heads.  One block per (token, head).  q and k are rotated in place by the angles of the
+// token's position (cos/sin tables are 32-bit, [capacity, D/2]; pair (i, i + D/2)); k (rotated)
+// and v go to the pages at slot = block * BS + offset, page layout [NB, Hkv, BS, D].
+// rotate == 0 skips the rotation (a position encoding that only stores).
+// slots == nullptr or a negative slot: nothing is stored for that token.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, T* __restrict__ k_pages,
+                                  T* __restrict__ v_pages, const float* __restrict__ cos_table,
+                                  const float* __restrict__ sin_table,
+                                  const int* __restrict__ positions, const int* __restrict__ slots,
+                                  int heads, int kv_heads, int dim, int block_size, int rotate) {
+  const int t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int half = dim / 2;
+  const int width = (heads + 2 * kv_heads) * dim;
+  T* row = qkv + (size_t)t * width + (size_t)h * dim;
+  const int pos = positions[t];
+  const int slot = slots ? slots[t] : -1;
+  T* page = nullptr;
+  if (h >= heads && slot >= 0) {
+    const int kvh = (h - heads) % kv_heads;
+    T* pages = (h < heads + kv_heads) ? k_pages : v_pages;
+    const size_t blk = (size_t)(slot / block_size);
+    const int off = slot % block_size;
+    page = pages + ((blk * kv_heads + kvh) * block_size + off) * (size_t)dim;
+  }
+  if (h < heads + kv_heads && rotate) {
+    const float* c = cos_table + (size_t)pos * half;
+    const float* s = sin_table + (size_t)pos * half;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      const float x1 = to_float(row[i]);
+      const float x2 = to_float(row[i + half]);
+      const T o1 = from_float<T>(x1 * c[i] - x2 * s[i]);
+      const T o2 = from_float<T>(x2 * c[i] + x1 * s[i]);
+      row[i] = o1;
+      row[i + half] = o2;
+      if (page) {
+        page[i] = o1;
+        page[i + half] = o2;
+      }
+    }
+  } else if (page) {
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) page[i] = row[i];
+  }
+}
+
+extern "C" int ts_rope_store(void* qkv, void* k_pages, void* v_pages, const float* cos_table,
+                             const float* sin_table, const int* positions, const int* slots,
+                             int tokens, int heads, int kv_heads, int dim, int block_size,
+                             int rotate, int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!qkv || !positions || heads < 1 || kv_heads < 1 || dim < 2 || (dim & 1) || block_size < 1)
+    return TS_ERR_ARG;
+  if (rotate && (!cos_table || !sin_table)) return TS_ERR_ARG;
+  if (slots && (!k_pages || !v_pages)) return TS_ERR_ARG;
+  dim3 grid(tokens, heads + 2 * kv_heads), block(64);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, (float*)k_pages, (float*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// gather rows: out[i, :] = x[rows[i], :]
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                   const int* __restrict__ rows, int width) {
+  const size_t src = (size_t)rows[blockIdx.x] * width;
+  const size_t dst = (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = x[src + i];
+}
+
+extern "C" int ts_gather_rows(void* out, const void* x, const int* rows, int n, int width,
+                              int dtype, hipStream_t stream) {
+  if (n == 0) return TS_OK;
+  if (!out || !x || !rows || width < 1) return TS_ERR_ARG;
+  dim3 grid(n), block(256);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(gather_rows_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)x, rows, width);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(gather_rows_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)x, rows, width);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}

@@ -1,0 +1,144 @@
+"""The batch of one step: host entries in, one packed device buffer out.
+
+A step holds, for each request in it, that request's next tokens — a whole prompt, a portion
+of one, or a single decoded token — concatenated without padding.  The reference describes
+the same batch with ``AttnMetadata`` (src/turboserve/engine/core/types.py:244-398) built from
+Python lists by four ``torch.tensor`` calls (src/turboserve/engine/runtime/worker.py:190-194);
+here all integer inputs travel in one int32 buffer and the context keeps the host's copies of
+the lengths, so nothing is read back.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Hashable, Sequence
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from turboserve_amd.cache.manager import PAD_PAGE
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step."""
+
+    request: Hashable
+    tokens: Sequence[int]  # its next tokens
+    start: int  # position of tokens[0] = tokens of the request already in the cache
+    tables: Sequence[Sequence[int]]  # per cache group: the request's block table
+    slots: Sequence[Sequence[int]]  # per cache group: one slot per token
+    state_slot: int = 0
+    want: Sequence[int] = ()  # places among `tokens` whose logits are wanted
+
+
+@dataclass
+class StepContext:
+    """What parts see of a step.  Device tensors are int32 views into one buffer."""
+
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor  # [T]
+    positions: torch.Tensor  # [T] absolute position of each token in its request
+    token_seq: torch.Tensor  # [T] index of each token's request in this step
+    query_start_loc: torch.Tensor  # [S + 1] row range of each request
+    context_lens: torch.Tensor  # [S] tokens of each request in the cache after this step
+    state_slots: torch.Tensor  # [S]
+    logit_rows: torch.Tensor  # [n] rows whose logits are wanted
+    slot_mapping: list[torch.Tensor]  # per group [T]
+    block_tables: list[torch.Tensor]  # per group [S, MB], PAD_PAGE beyond a request's pages
+    # host copies
+    query_lens: list[int] = field(default_factory=list)
+    context_lens_host: list[int] = field(default_factory=list)
+    max_query_len: int = 0
+    max_context_len: int = 0
+    num_logit_rows: int = 0
+
+
+def validate_entries(entries: Sequence[StepEntry], num_groups: int, page_size: int) -> None:
+    """Host checks of a step (types.py:335-398, scheduler.py:270-274): every request once,
+    at least one token each, one slot per token, tables that cover the context."""
+    seen: set[Hashable] = set()
+    for entry in entries:
+        if entry.request in seen:
+            raise ValueError(f"request {entry.request!r} appears twice in one step")
+        seen.add(entry.request)
+        count = len(entry.tokens)
+        if count < 1:
+            raise ValueError(f"request {entry.request!r} brings no token")
+        if entry.start < 0:
+            raise ValueError(f"request {entry.request!r} starts at {entry.start}")
+        if len(entry.tables) != num_groups or len(entry.slots) != num_groups:
+            raise ValueError(f"request {entry.request!r}: expected tables and slots for {num_groups} cache groups")
+        context = entry.start + count
+        for group in range(num_groups):
+            if len(entry.slots[group]) != count:
+                raise ValueError(f"request {entry.request!r}: {len(entry.slots[group])} slots for {count} tokens")
+            if len(entry.tables[group]) * page_size < context:
+                raise ValueError(
+                    f"request {entry.request!r}: block table of {len(entry.tables[group])} pages "
+                    f"does not cover {context} tokens"
+                )
+        for place in entry.want:
+            if not 0 <= place < count:
+                raise ValueError(f"request {entry.request!r}: wanted place {place} is outside its {count} tokens")
+
+
+def build_context(
+    entries: Sequence[StepEntry],
+    *,
+    num_groups: int,
+    page_size: int,
+    device: torch.device | str,
+    check: bool = True,
+) -> StepContext:
+    """Pack a step's entries, in the order given, into device tensors with one copy."""
+    if check:
+        validate_entries(entries, num_groups, page_size)
+    num_seqs = len(entries)
+    query_lens = [len(e.tokens) for e in entries]
+    context_lens = [e.start + n for e, n in zip(entries, query_lens)]
+    num_tokens = sum(query_lens)
+    starts = np.zeros(num_seqs + 1, dtype=np.int32)
+    np.cumsum(query_lens, out=starts[1:])
+    widths = [max((len(e.tables[g]) for e in entries), default=1) or 1 for g in range(num_groups)]
+    logit_rows = [int(starts[i]) + place for i, e in enumerate(entries) for place in e.want]
+
+    pieces: list[np.ndarray] = [
+        np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=num_tokens),
+        np.concatenate([np.arange(e.start, e.start + n, dtype=np.int32) for e, n in zip(entries, query_lens)])
+        if num_seqs else np.zeros(0, dtype=np.int32),
+        np.repeat(np.arange(num_seqs, dtype=np.int32), query_lens),
+        starts,
+        np.asarray(context_lens, dtype=np.int32),
+        np.asarray([e.state_slot for e in entries], dtype=np.int32),
+        np.asarray(logit_rows, dtype=np.int32),
+    ]
+    for g in range(num_groups):
+        pieces.append(np.fromiter((s for e in entries for s in e.slots[g]), dtype=np.int32, count=num_tokens))
+        table = np.full((num_seqs, widths[g]), PAD_PAGE, dtype=np.int32)
+        for i, e in enumerate(entries):
+            row = e.tables[g]
+            table[i, : len(row)] = row
+        pieces.append(table.reshape(-1))
+    sizes = [p.size for p in pieces]
+    packed = torch.from_numpy(np.concatenate(pieces)).to(device)
+    views = list(torch.split(packed, sizes))
+    return StepContext(
+        num_tokens=num_tokens,
+        num_seqs=num_seqs,
+        token_ids=views[0],
+        positions=views[1],
+        token_seq=views[2],
+        query_start_loc=views[3],
+        context_lens=views[4],
+        state_slots=views[5],
+        logit_rows=views[6],
+        slot_mapping=[views[7 + 2 * g] for g in range(num_groups)],
+        block_tables=[views[8 + 2 * g].view(num_seqs, widths[g]) for g in range(num_groups)],
+        query_lens=query_lens,
+        context_lens_host=context_lens,
+        max_query_len=max(query_lens, default=0),
+        max_context_len=max(context_lens, default=0),
+        num_logit_rows=len(logit_rows),
+    )

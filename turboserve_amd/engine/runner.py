@@ -1,0 +1,62 @@
+"""The step function: a flat batch of (request, its next tokens) in, logits at the wanted
+places out.
+
+It runs only the tokens it is given, as one batch, against what earlier steps left in the
+cache; it samples nothing and owns no request state.  Generation, replay and measurement all
+go through it.  The reference's counterpart is ``ModelRunner.execute``
+(src/turboserve/engine/runtime/worker.py:237-266), which also samples; its separable phases
+(:180-233) are ``build_context`` / ``forward`` / ``logits`` here.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+
+import torch
+
+from turboserve_amd.cache.layout import CacheLayout
+from turboserve_amd.cache.storage import CacheStorage
+from turboserve_amd.engine.batch import StepContext, StepEntry, build_context
+from turboserve_amd.models.decoder import DecoderModel
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, storage: CacheStorage, *, check: bool = True) -> None:
+        self.model = model
+        self.storage = storage
+        self.layout: CacheLayout = storage.layout
+        self.check = check
+        self.views = storage.views()
+        self.vocab_size = model.plan.vocab_size
+        self.num_steps = 0
+
+    def context_for(self, entries: Sequence[StepEntry]) -> StepContext:
+        if self.check:
+            vocab = self.vocab_size
+            for entry in entries:
+                for token in entry.tokens:
+                    if not 0 <= token < vocab:
+                        raise ValueError(f"request {entry.request!r}: token id {token} is outside the vocabulary of {vocab}")
+        return build_context(
+            entries,
+            num_groups=len(self.layout.groups),
+            page_size=self.storage.page_size,
+            device=self.model.runtime.device,
+            check=self.check,
+        )
+
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry], *, fresh_state_slots: Sequence[int] = ()) -> torch.Tensor:
+        """Run one step and return 32-bit logits ``[wanted, V]`` on the device, in the order of
+        the entries and of each entry's ``want``.  A step that wants nothing still runs (it
+        fills the cache, worker.py:248-256) and returns ``[0, V]``."""
+        self.storage.zero_state_slots(fresh_state_slots)
+        device = self.model.runtime.device
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
+        ctx = self.context_for(entries)
+        stream = self.model.forward(ctx.token_ids, ctx, self.views)
+        self.num_steps += 1
+        if ctx.num_logit_rows == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
+        return self.model.logits(stream, ctx.logit_rows)

@@ -1,0 +1,371 @@
+"""Python face of the HIP kernels: shape checks on the host, then one C call per op.
+
+Every op runs on the current torch stream of the tensors' device.  There is no fallback: if
+the library cannot be built or loaded, or a tensor is not on a GPU, the op raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from turboserve_amd.kernels import build
+
+TS_F32 = 0
+TS_BF16 = 1
+
+_ERRORS = {
+    1: "unsupported dtype code",
+    2: "a size the kernel does not take",
+    3: "the kernel launch failed",
+    4: "null pointer or inconsistent arguments",
+}
+
+
+class KernelError(RuntimeError):
+    """A kernel refused its arguments or failed to launch."""
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return TS_F32
+    if dtype == torch.bfloat16:
+        return TS_BF16
+    raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+_SIGNATURES: dict[str, dict[str, list]] = {
+    "core": {
+        "ts_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
+        "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
+        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_rope_store": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
+                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                       c_float, c_int, c_int, c_void_p],
+        "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
+                          c_int, c_int, c_void_p],
+        "ts_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    },
+}
+
+_LIBRARIES: dict[str, ctypes.CDLL] = {}
+
+
+def load_module(module: str) -> ctypes.CDLL:
+    """The loaded library of a kernel module, compiled first if nothing is built."""
+    lib = _LIBRARIES.get(module)
+    if lib is not None:
+        return lib
+    path = build.ensure_module(module)
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as exc:  # pragma: no cover - depends on the machine
+        raise KernelError(f"cannot load the kernel library {path}: {exc}") from exc
+    for name, argtypes in _SIGNATURES.get(module, {}).items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    _LIBRARIES[module] = lib
+    return lib
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _check(status: int, name: str) -> None:
+    if status != 0:
+        raise KernelError(f"{name}: {_ERRORS.get(status, f'error {status}')}")
+
+
+def _need(cond: bool, message: str) -> None:
+    if not cond:
+        raise KernelError(message)
+
+
+def _gpu(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+def _i32(t: torch.Tensor | None, name: str) -> None:
+    if t is not None:
+        _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+
+
+class Ops:
+    """The kernel library bound to one device."""
+
+    def __init__(self, device: torch.device | str = "cuda:0", modules: tuple[str, ...] = ("core",)) -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"the kernels need a GPU device, not {self.device}")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to torch; this engine has no CPU path")
+        self.core = load_module("core")
+        for module in modules:
+            load_module(module)
+
+    def stream(self) -> int:
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    # -- rows ---------------------------------------------------------------------------------
+
+    def embed(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """``float32 [T, H]`` rows of ``table [V, H]`` at ``ids [T]`` (the start of the 32-bit
+        residual stream)."""
+        _gpu(table, ids)
+        _i32(ids, "ids")
+        _need(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [V, H]")
+        tokens, (vocab, hidden) = ids.numel(), table.shape
+        if out is None:
+            out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+        _need(out.shape == (tokens, hidden) and out.dtype == torch.float32 and out.is_contiguous(),
+              "out must be contiguous float32 [T, H]")
+        _check(self.core.ts_embed(_ptr(out), _ptr(table), _ptr(ids), tokens, hidden, vocab,
+                                  dtype_code(table.dtype), self.stream()), "ts_embed")
+        return out
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        _gpu(x, weight)
+        _need(x.dim() == 2 and x.is_contiguous(), "x must be contiguous [T, H]")
+        _need(weight.shape == (x.shape[1],) and weight.dtype == x.dtype and weight.is_contiguous(),
+              "weight must be [H] of x's dtype")
+        y = torch.empty_like(x)
+        _check(self.core.ts_rmsnorm(_ptr(y), _ptr(x), _ptr(weight), float(eps), x.shape[0], x.shape[1],
+                                    dtype_code(x.dtype), self.stream()), "ts_rmsnorm")
+        return y
+
+    def add_rmsnorm(
+        self,
+        residual: torch.Tensor,
+        pending: torch.Tensor | None,
+        weight: torch.Tensor,
+        eps: float,
+        rows: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """``residual += pending`` in 32-bit (in place) and the normalised sum in ``weight``'s
+        dtype; with ``rows`` only those rows, and ``residual`` is left alone."""
+        _gpu(residual, pending, weight, rows)
+        _i32(rows, "rows")
+        _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
+              "residual must be contiguous float32 [T, H]")
+        tokens, hidden = residual.shape
+        _need(weight.shape == (hidden,) and weight.is_contiguous(), "weight must be [H]")
+        if pending is not None:
+            _need(pending.shape == residual.shape and pending.dtype == weight.dtype and pending.is_contiguous(),
+                  "pending must be contiguous [T, H] of the weight's dtype")
+        out_rows = tokens if rows is None else rows.numel()
+        y = torch.empty((out_rows, hidden), dtype=weight.dtype, device=residual.device)
+        _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), _ptr(weight), _ptr(rows),
+                                        float(eps), out_rows, hidden, dtype_code(weight.dtype), self.stream()),
+               "ts_add_rmsnorm")
+        return y
+
+    def swiglu(self, gate_up: torch.Tensor) -> torch.Tensor:
+        """``silu(gate) * up`` of the fused ``[T, 2 I]`` projection -> ``[T, I]``."""
+        _gpu(gate_up)
+        _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
+              "gate_up must be contiguous [T, 2 I]")
+        tokens, inter = gate_up.shape[0], gate_up.shape[1] // 2
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+        _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), tokens, inter, dtype_code(gate_up.dtype),
+                                   self.stream()), "ts_swiglu")
+        return out
+
+    def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        _gpu(x, rows)
+        _i32(rows, "rows")
+        _need(x.dim() == 2 and x.is_contiguous(), "x must be contiguous [T, W]")
+        out = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+        _check(self.core.ts_gather_rows(_ptr(out), _ptr(x), _ptr(rows), rows.numel(), x.shape[1],
+                                        dtype_code(x.dtype), self.stream()), "ts_gather_rows")
+        return out
+
+    def rope_store(
+        self,
+        qkv: torch.Tensor,
+        k_pages: torch.Tensor | None,
+        v_pages: torch.Tensor | None,
+        cos: torch.Tensor | None,
+        sin: torch.Tensor | None,
+        positions: torch.Tensor,
+        slots: torch.Tensor | None,
+        heads: int,
+        kv_heads: int,
+        head_dim: int,
+        block_size: int,
+        max_position: int,
+    ) -> None:
+        """Rotate q and k of ``qkv [T, (Hq + 2 Hkv) D]`` in place (skipped when ``cos`` is
+        ``None``) and store k, v at ``slots`` into pages ``[NB, Hkv, BS, D]`` (skipped when
+        ``slots`` is ``None``).  ``max_position`` is the largest position of the step, known on
+        the host, and must lie inside the tables."""
+        _gpu(qkv, k_pages, v_pages, cos, sin, positions, slots)
+        _i32(positions, "positions")
+        _i32(slots, "slots")
+        tokens = positions.numel()
+        width = (heads + 2 * kv_heads) * head_dim
+        _need(qkv.shape == (tokens, width) and qkv.is_contiguous(), f"qkv must be contiguous [T, {width}]")
+        _need(head_dim % 2 == 0, "head_dim must be even")
+        if cos is not None:
+            half = head_dim // 2
+            _need(sin is not None and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == half
+                  and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                  and cos.is_contiguous() and sin.is_contiguous(), "cos/sin must be float32 [capacity, D/2]")
+            _need(max_position < cos.shape[0], f"position {max_position} is beyond the rotary tables ({cos.shape[0]})")
+        if slots is not None:
+            _need(slots.numel() == tokens, "one slot per token")
+            _need(k_pages is not None and v_pages is not None, "slots given without pages")
+            for pages in (k_pages, v_pages):
+                _need(pages.dim() == 4 and pages.shape[1:] == (kv_heads, block_size, head_dim)
+                      and pages.dtype == qkv.dtype and pages.is_contiguous(),
+                      "pages must be contiguous [NB, Hkv, BS, D] of qkv's dtype")
+        _check(self.core.ts_rope_store(_ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(cos), _ptr(sin),
+                                       _ptr(positions), _ptr(slots), tokens, heads, kv_heads, head_dim,
+                                       block_size, 0 if cos is None else 1, dtype_code(qkv.dtype), self.stream()),
+               "ts_rope_store")
+
+    # -- attention ----------------------------------------------------------------------------
+
+    def paged_attention_generic(
+        self,
+        q: torch.Tensor,
+        q_stride: int,
+        k_pages: torch.Tensor,
+        v_pages: torch.Tensor,
+        block_table: torch.Tensor,
+        token_seq: torch.Tensor,
+        positions: torch.Tensor,
+        heads: int,
+        scale: float,
+        window: int | None,
+    ) -> torch.Tensor:
+        """Attention of every token over the keys ``lo..position`` of its request.
+
+        ``q`` is the tensor whose first ``heads * D`` elements of each ``q_stride``-long row
+        are the (already encoded) queries.  Returns ``[T, heads * D]``."""
+        _gpu(q, k_pages, v_pages, block_table, token_seq, positions)
+        _i32(block_table, "block_table")
+        _i32(token_seq, "token_seq")
+        _i32(positions, "positions")
+        _need(k_pages.dim() == 4 and k_pages.shape == v_pages.shape and k_pages.is_contiguous()
+              and v_pages.is_contiguous() and k_pages.dtype == q.dtype == v_pages.dtype,
+              "pages must be contiguous [NB, Hkv, BS, D] of q's dtype")
+        _, kv_heads, block_size, head_dim = k_pages.shape
+        tokens = positions.numel()
+        _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
+              "q does not hold [T, q_stride] rows")
+        _need(block_table.dim() == 2 and token_seq.numel() == tokens, "block_table [S, MB], token_seq [T]")
+        _need(heads % kv_heads == 0, "query heads must be a multiple of KV heads")
+        _need(head_dim <= 512, "head_dim above 512 is not supported by the attention kernel")
+        out = torch.empty((tokens, heads * head_dim), dtype=q.dtype, device=q.device)
+        _check(self.core.ts_paged_attention_generic(
+            _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim,
+            block_size, float(scale), int(window or 0), dtype_code(q.dtype), self.stream()),
+            "ts_paged_attention_generic")
+        return out
+
+    # -- products -----------------------------------------------------------------------------
+
+    def gemm_plain(
+        self,
+        x: torch.Tensor,
+        weight: torch.Tensor,
+        bias: torch.Tensor | None = None,
+        *,
+        out_float32: bool = False,
+    ) -> torch.Tensor:
+        """``x [M, K] @ weight [N, K]^T (+ bias)`` by 32-bit fused multiply-adds."""
+        _gpu(x, weight, bias)
+        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous(),
+              "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
+        _need(x.shape[1] == weight.shape[1] and x.dtype == weight.dtype, "x and weight disagree on K or dtype")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            _need(bias.shape == (n,) and bias.dtype == x.dtype and bias.is_contiguous(), "bias must be [N]")
+        out_dtype = torch.float32 if out_float32 else x.dtype
+        y = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        _check(self.core.ts_gemm_plain(_ptr(y), _ptr(x), _ptr(weight), _ptr(bias), m, n, k,
+                                       x.stride(0) if m > 1 else max(k, x.stride(0)), n,
+                                       dtype_code(x.dtype), 1 if out_float32 else 0, self.stream()),
+               "ts_gemm_plain")
+        return y
+
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+        """The projection of the serving path: 32-bit runs use :meth:`gemm_plain` (no reduced
+        matrix mode); bfloat16 runs use the BLAS library behind torch, as the reference does
+        for every linear layer (src/turboserve/engine/model/layers.py:142)."""
+        if x.dtype == torch.float32:
+            return self.gemm_plain(x, weight, bias)
+        _gpu(x, weight, bias)
+        if bias is None:
+            return torch.mm(x, weight.t())
+        return torch.addmm(bias, x, weight.t())
+
+    def linear_float32_out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """``x @ weight^T`` with a 32-bit result (the head: logits are 32-bit,
+        src/turboserve/engine/model/model.py:244)."""
+        if x.dtype == torch.float32:
+            return self.gemm_plain(x, weight)
+        _gpu(x, weight)
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+
+    # -- sampling -----------------------------------------------------------------------------
+
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        _gpu(logits)
+        _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(),
+              "logits must be contiguous float32 [n, V]")
+        tokens = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+        _check(self.core.ts_argmax(_ptr(tokens), _ptr(logits), logits.shape[0], logits.shape[1], self.stream()),
+               "ts_argmax")
+        return tokens
+
+    def sample(
+        self,
+        logits: torch.Tensor,
+        temperature: torch.Tensor,
+        top_k: torch.Tensor,
+        top_p: torch.Tensor,
+        penalty: torch.Tensor,
+        seed_lo: torch.Tensor,
+        seed_hi: torch.Tensor,
+        draw_index: torch.Tensor,
+        history: torch.Tensor,
+        history_start: torch.Tensor,
+        want_logprobs: bool,
+    ) -> tuple[torch.Tensor, torch.Tensor | None]:
+        """One token per row of ``logits [n, V]``; parameter tensors are per row (see
+        ``csrc/sampling.hip``).  Returns ``(tokens int32 [n], logprobs float32 [n] | None)``."""
+        _gpu(logits, temperature, top_k, top_p, penalty, seed_lo, seed_hi, draw_index, history, history_start)
+        _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(),
+              "logits must be contiguous float32 [n, V]")
+        rows, vocab = logits.shape
+        for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                            ("top_p", top_p, torch.float32), ("penalty", penalty, torch.float32),
+                            ("seed_lo", seed_lo, torch.int32), ("seed_hi", seed_hi, torch.int32),
+                            ("draw_index", draw_index, torch.int32)):
+            _need(t.shape == (rows,) and t.dtype == dt and t.is_contiguous(), f"{name} must be {dt} [n]")
+        _i32(history, "history")
+        _i32(history_start, "history_start")
+        _need(history_start.numel() == rows + 1, "history_start must have n + 1 entries")
+        tokens = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        logprobs = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_logprobs else None
+        work = torch.empty_like(logits)
+        _check(self.core.ts_sample(_ptr(tokens), _ptr(logprobs), _ptr(logits), _ptr(work), rows, vocab,
+                                   _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(penalty), _ptr(seed_lo),
+                                   _ptr(seed_hi), _ptr(draw_index), _ptr(history), _ptr(history_start),
+                                   self.stream()), "ts_sample")
+        return tokens, logprobs

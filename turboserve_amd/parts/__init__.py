@@ -1,0 +1,28 @@
+"""The parts a model is assembled from; importing this package registers the built-in kinds."""
+
+from turboserve_amd.parts import attention, block, mlp, norm, rope  # noqa: F401  (registration)
+from turboserve_amd.parts.base import (  # noqa: F401
+    Block,
+    CacheNeed,
+    FeedForward,
+    FixedState,
+    FixedStateView,
+    Mixer,
+    Norm,
+    PagedKV,
+    PagedKVView,
+    Part,
+    PartSpec,
+    PositionEncoding,
+    ResidualStream,
+    Runtime,
+    TensorSpec,
+)
+from turboserve_amd.parts.registry import (  # noqa: F401
+    build_part,
+    register_block,
+    register_feed_forward,
+    register_mixer,
+    register_norm,
+    register_position_encoding,
+)

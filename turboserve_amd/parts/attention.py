@@ -1,0 +1,98 @@
+"""Grouped-query attention over the paged cache (src/turboserve/engine/model/layers.py:311-391,
+src/turboserve/engine/model/attention.py:213-295)."""
+
+from __future__ import annotations
+
+from collections.abc import Mapping
+
+import torch
+
+from turboserve_amd.parts.base import CacheNeed, Mixer, PagedKV, PagedKVView, PartSpec, Runtime, TensorSpec
+from turboserve_amd.parts.registry import build_part, register_mixer
+
+
+@register_mixer("gqa_attention")
+class GroupedQueryAttention(Mixer):
+    """q/k/v projections (optionally biased), position encoding, cache write, attention of every
+    token over its request's keys up to itself (optionally only the last ``window``), output
+    projection.
+
+    The three projections are held as one ``[(Hq + 2 Hkv) D, H]`` matrix (the checkpoint keeps
+    them apart; ``load`` concatenates), so a step does one product for them.  Scale is a
+    parameter (``head_dim ** -0.5`` for Qwen2, model_config.py:224-227)."""
+
+    def __init__(
+        self,
+        prefix: str,
+        runtime: Runtime,
+        *,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        scale: float,
+        qkv_bias: bool,
+        out_bias: bool,
+        window: int | None,
+        position: PartSpec,
+    ) -> None:
+        super().__init__(prefix, runtime)
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"{num_heads} query heads is not a multiple of {num_kv_heads} KV heads")
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.num_kv_heads = int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.scale = float(scale)
+        self.qkv_bias = bool(qkv_bias)
+        self.out_bias = bool(out_bias)
+        self.window = None if window is None else int(window)
+        self.position = build_part("position_encoding", position, prefix, runtime)
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.qkv_weight: torch.Tensor | None = None
+        self.qkv_bias_tensor: torch.Tensor | None = None
+        self.o_weight: torch.Tensor | None = None
+        self.o_bias_tensor: torch.Tensor | None = None
+
+    def cache_need(self) -> CacheNeed:
+        return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        specs = {
+            self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden_size)),
+            self.name("k_proj.weight"): TensorSpec((self.kv_size, self.hidden_size)),
+            self.name("v_proj.weight"): TensorSpec((self.kv_size, self.hidden_size)),
+            self.name("o_proj.weight"): TensorSpec((self.hidden_size, self.q_size)),
+        }
+        if self.qkv_bias:
+            specs[self.name("q_proj.bias")] = TensorSpec((self.q_size,))
+            specs[self.name("k_proj.bias")] = TensorSpec((self.kv_size,))
+            specs[self.name("v_proj.bias")] = TensorSpec((self.kv_size,))
+        if self.out_bias:
+            specs[self.name("o_proj.bias")] = TensorSpec((self.hidden_size,))
+        specs.update(self.position.tensor_specs())
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.qkv_weight = torch.cat(
+            [tensors[self.name(f"{p}_proj.weight")] for p in ("q", "k", "v")], dim=0
+        ).contiguous()
+        if self.qkv_bias:
+            self.qkv_bias_tensor = torch.cat(
+                [tensors[self.name(f"{p}_proj.bias")] for p in ("q", "k", "v")], dim=0
+            ).contiguous()
+        self.o_weight = tensors[self.name("o_proj.weight")].contiguous()
+        if self.out_bias:
+            self.o_bias_tensor = tensors[self.name("o_proj.bias")].contiguous()
+        self.position.load(tensors)
+
+    def forward(self, x: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
+        ops = self.runtime.ops
+        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_tensor)
+        self.position.encode_and_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache)
+        attended = ops.paged_attention_generic(
+            qkv, qkv.shape[1], cache.k, cache.v, ctx.block_tables[cache.group], ctx.token_seq,
+            ctx.positions, self.num_heads, self.scale, self.window,
+        )
+        return ops.linear(attended, self.o_weight, self.o_bias_tensor)

@@ -1,0 +1,214 @@
+"""Interfaces of the parts a model is put together from.
+
+A model is data: an embedding, a list of layers, the order in which the layers run, a final
+norm and a head.  Each layer names a block arrangement and, inside it, a mixer, a feed-forward
+and norms, every one a :class:`PartSpec` (a registered kind plus its sizes and constants).
+No part knows which architecture it serves; what a part needs it gets as constructor
+parameters, as tensors by name, and as the :class:`StepContext` of the running step.
+
+The reference hard-wires one block (src/turboserve/engine/model/layers.py:443-487) and one
+cache kind (src/turboserve/engine/core/kv_cache.py:372-386); the split below is this engine's.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Mapping
+from dataclasses import dataclass, field
+from typing import TYPE_CHECKING, Any
+
+import torch
+
+if TYPE_CHECKING:  # pragma: no cover
+    from turboserve_amd.engine.batch import StepContext
+
+
+# ---------------------------------------------------------------------------------------------
+# plain-data descriptions
+# ---------------------------------------------------------------------------------------------
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A registered part ``kind`` and the keyword parameters it is built with."""
+
+    kind: str
+    params: Mapping[str, Any] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """What a part expects under one checkpoint tensor name.
+
+    ``kind`` is ``"float"`` (converted to the run's dtype), ``"float_keep32"`` (a tensor the
+    file stores in 32-bit stays 32-bit, anything else is converted to the run's dtype) or
+    ``"int"`` (kept as int32).  ``init`` says how the random-weights mode fills it:
+    ``"normal"`` (N(0, std)), ``"ones"`` or ``"zeros"``.
+    """
+
+    shape: tuple[int, ...]
+    kind: str = "float"
+    init: str = "normal"
+
+
+@dataclass(frozen=True)
+class PagedKV:
+    """A mixer's need for per-token cache pages: ``num_kv_heads x head_dim`` keys and values
+    per token; ``window`` keys are ever read again (``None``: all of them)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class FixedState:
+    """A mixer's need for per-request state of fixed size (``shape`` elements of ``dtype``
+    per request), zeroed when a request takes its slot."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+CacheNeed = PagedKV | FixedState | None
+
+
+@dataclass
+class PagedKVView:
+    """One cache unit's pages: ``k`` and ``v`` are ``[num_blocks, kv_heads, block_size,
+    head_dim]``; ``group`` indexes the step's per-group block tables and slot mappings;
+    ``writable`` is false when the layer reads another layer's cache."""
+
+    k: torch.Tensor
+    v: torch.Tensor
+    group: int
+    block_size: int
+    window: int | None
+    writable: bool = True
+
+
+@dataclass
+class FixedStateView:
+    """One cache unit's per-request state: ``[num_slots, *shape]``; the rows of this step's
+    requests are ``ctx.state_slots``."""
+
+    state: torch.Tensor
+    writable: bool = True
+
+
+CacheView = PagedKVView | FixedStateView | None
+
+
+@dataclass
+class Runtime:
+    """What every part is built with: the device, the run's dtype and the kernel library.
+
+    ``shared`` holds parts without weights that several layers may use as one object (the
+    rotary tables: one per distinct set of constants, not one per layer)."""
+
+    device: torch.device
+    dtype: torch.dtype
+    ops: Any  # turboserve_amd.kernels.ops.Ops
+    shared: dict = field(default_factory=dict)
+
+
+@dataclass
+class ResidualStream:
+    """The hidden state between blocks: a 32-bit running sum ``residual [T, H]`` and the last
+    part's output ``pending [T, H]`` (run dtype) that has not been added to it yet."""
+
+    residual: torch.Tensor
+    pending: torch.Tensor | None = None
+
+
+# ---------------------------------------------------------------------------------------------
+# interfaces
+# ---------------------------------------------------------------------------------------------
+
+
+class Part:
+    """Base of everything that holds weights.
+
+    ``prefix`` is the checkpoint name prefix of the part (``"model.layers.3.self_attn"``).
+    ``tensor_specs`` maps full checkpoint names to what is expected there; ``load`` receives
+    exactly those tensors, on the device, already converted, and may fuse or re-lay them.
+    """
+
+    #: A part without weights whose instances with equal parameters may be one object.
+    shareable = False
+
+    def __init__(self, prefix: str, runtime: Runtime) -> None:
+        self.prefix = prefix
+        self.runtime = runtime
+
+    def name(self, suffix: str) -> str:
+        return f"{self.prefix}.{suffix}" if self.prefix else suffix
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        return {}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:  # pragma: no cover - default
+        return None
+
+
+class Norm(Part):
+    """Normalisation over the last dimension."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """``[T, H]`` run dtype -> ``[T, H]`` run dtype."""
+        raise NotImplementedError
+
+    def forward_residual(self, stream: ResidualStream, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """Add ``stream.pending`` into ``stream.residual`` (32-bit) and return the normalised
+        sum in the run dtype.  With ``rows`` only those rows are read and returned, and the
+        stream is left as it is."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into the queries and keys of an attention mixer and stores the
+    step's keys and values into the cache pages (one pass over the projection output)."""
+
+    def encode_and_store(
+        self,
+        qkv: torch.Tensor,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        ctx: "StepContext",
+        cache: PagedKVView,
+    ) -> None:
+        """``qkv [T, (Hq + 2 Hkv) D]``: encode q and k in place; write k, v at the step's slots
+        of ``cache.group`` unless the cache is not writable."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request (attention, or anything with state)."""
+
+    def cache_need(self) -> CacheNeed:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext", cache: CacheView) -> torch.Tensor:
+        """``x [T, H]`` (normalised) -> ``[T, H]``.  The rows of request ``s`` are
+        ``ctx.query_start_loc[s]:ctx.query_start_loc[s+1]``, in position order, continuing
+        whatever earlier steps left in ``cache``."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Acts on each token alone."""
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norms, a mixer and a feed-forward around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, stream: ResidualStream, ctx: "StepContext", cache: CacheView) -> ResidualStream:
+        raise NotImplementedError
+
+    def parts(self) -> list[Part]:
+        raise NotImplementedError

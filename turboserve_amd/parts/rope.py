@@ -1,0 +1,90 @@
+"""Rotary position encoding (src/turboserve/engine/model/layers.py:214-308)."""
+
+from __future__ import annotations
+
+import torch
+
+from turboserve_amd.parts.base import PagedKVView, PositionEncoding, Runtime
+from turboserve_amd.parts.registry import register_position_encoding
+
+
+def rotary_tables(capacity: int, head_dim: int, theta: float, factor: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """32-bit ``cos, sin [capacity, D/2]`` of the angles ``(pos / factor) * theta^(-2i/D)``.
+
+    Computed on the CPU with the reference's expressions (layers.py:258-262 for the inverse
+    frequencies, :281-286 for the outer product; its tables repeat the ``D/2`` columns twice,
+    which is not stored here)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    positions = torch.arange(capacity, dtype=torch.float32)
+    if factor != 1.0:
+        positions = positions / factor
+    angles = torch.outer(positions, inv_freq)
+    return angles.cos().contiguous(), angles.sin().contiguous()
+
+
+@register_position_encoding("rope")
+class RotaryEncoding(PositionEncoding):
+    """Half-split rotary encoding: the pair ``(i, i + D/2)`` of every query and key head is
+    turned by the angle of the token's position (layers.py:214-222, 298-302).  The rotation is
+    computed in 32-bit from 32-bit tables and rounded once.  Tables grow by doubling, driven
+    by the host-known largest position of a step (layers.py:272-288).  It has no weights, so
+    layers with the same constants share one instance and one pair of tables."""
+
+    shareable = True
+
+    def __init__(
+        self,
+        prefix: str,
+        runtime: Runtime,
+        *,
+        head_dim: int,
+        theta: float,
+        scaling_factor: float = 1.0,
+        max_positions: int = 2048,
+    ) -> None:
+        super().__init__(prefix, runtime)
+        if head_dim % 2 != 0:
+            raise ValueError(f"head_dim must be even for rotary encoding, got {head_dim}")
+        self.head_dim = int(head_dim)
+        self.theta = float(theta)
+        self.scaling_factor = float(scaling_factor)
+        self.cos: torch.Tensor | None = None
+        self.sin: torch.Tensor | None = None
+        self.capacity = 0
+        #: First table size; the tables themselves are made at the first step (layers.py:265).
+        self.initial_capacity = min(int(max_positions), 1024)
+
+    def ensure_capacity(self, num_positions: int) -> None:
+        if num_positions <= self.capacity:
+            return
+        target = max(num_positions, 2 * self.capacity, self.initial_capacity, 16)
+        cos, sin = rotary_tables(target, self.head_dim, self.theta, self.scaling_factor)
+        self.cos = cos.to(self.runtime.device)
+        self.sin = sin.to(self.runtime.device)
+        self.capacity = target
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView) -> None:
+        self.ensure_capacity(ctx.max_context_len)
+        slots = ctx.slot_mapping[cache.group] if cache.writable else None
+        self.runtime.ops.rope_store(
+            qkv, cache.k, cache.v, self.cos, self.sin, ctx.positions, slots,
+            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1,
+        )
+
+
+@register_position_encoding("none")
+class NoPositionEncoding(PositionEncoding):
+    """No encoding: queries and keys stay as projected; keys and values are stored."""
+
+    shareable = True
+
+    def __init__(self, prefix: str, runtime: Runtime) -> None:
+        super().__init__(prefix, runtime)
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView) -> None:
+        if not cache.writable:
+            return
+        self.runtime.ops.rope_store(
+            qkv, cache.k, cache.v, None, None, ctx.positions, ctx.slot_mapping[cache.group],
+            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1,
+        )

@@ -1,0 +1,127 @@
+"""The engine's entry point on the GPU: greedy generation equals the plain implementation,
+whatever the token budget and however few pages there are; sampling follows the stated rule."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import tiny
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def make_engine(folder, dtype, page, *, num_blocks, budget=2048, max_num_seqs=8, seed=None):
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+
+    return LLMEngine(EngineConfig(
+        model=str(folder), dtype=dtype, seed=seed,
+        scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget, block_size=page,
+                                  num_blocks=num_blocks),
+    ))
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def model(request, tmp_path_factory):
+    config, seed, page = tiny.TINY[request.param]
+    folder = tiny.make_model_dir(tmp_path_factory.mktemp(f"engine{request.param}"), config, seed, torch.float32)
+    raw, tensors = tiny.read_model_dir(folder)
+    lengths = [5, 17, 33] if request.param == "A" else [1, 9, 24, 40]
+    prompts = [tiny.random_tokens(config["vocab_size"], n, 50 + n) for n in lengths]
+    return {"name": request.param, "folder": folder, "page": page, "raw": raw, "tensors": tensors, "prompts": prompts,
+            "vocab": config["vocab_size"]}
+
+
+def test_greedy_generation_equals_plain(model):
+    """Mixed-length prompts in one continuous batch, token for token
+    (tests/unit/test_engine_e2e.py:103-116 in the reference)."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 8 if model["name"] == "A" else 12
+    want = [plain.greedy_generate(model["raw"], model["tensors"], p, new) for p in model["prompts"]]
+    for budget, blocks in ((2048, 64), (16, 64), (7 if model["page"] <= 7 else model["page"], 64)):
+        with make_engine(model["folder"], "float32", model["page"], num_blocks=blocks, budget=budget) as engine:
+            outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+            assert [o.new_token_ids for o in outputs] == want, f"budget {budget}"
+            assert all(o.finish_reason == "length" and o.output_tokens == new for o in outputs)
+            engine.scheduler.check_invariants()
+            assert all(pool.num_in_use == 0 for pool in engine.scheduler.cache.pools)
+
+
+def test_preemption_keeps_the_tokens(model):
+    """So few pages that running requests are preempted and recomputed: same tokens
+    (tests/unit/test_engine_e2e.py:149-165)."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 10
+    want = [plain.greedy_generate(model["raw"], model["tensors"], p, new) for p in model["prompts"]]
+    longest = max(len(p) for p in model["prompts"]) + new
+    blocks = -(-longest // model["page"]) + 1  # one request fits, all of them do not
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=blocks, budget=64) as engine:
+        outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+        assert [o.new_token_ids for o in outputs] == want
+        assert engine.stats()["num_preemptions"] > 0
+        engine.scheduler.check_invariants()
+
+
+def test_temperature_sampling_follows_the_rule(model):
+    """Seeded temperature sampling: each token is the first whose cumulative probability
+    (plain implementation, 64-bit) exceeds the request's Philox uniform for that draw."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 12
+    params = [SamplingParams(max_tokens=new, temperature=0.8, seed=1000 + i, ignore_eos=True, logprobs=True)
+              for i in range(len(model["prompts"]))]
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=64, budget=7 if model["page"] <= 7 else 16) as engine:
+        outputs = engine.generate(model["prompts"], params)
+    for i, (prompt, output) in enumerate(zip(model["prompts"], outputs)):
+        tokens = list(prompt)
+        assert len(output.new_token_ids) == new
+        for draw, token in enumerate(output.new_token_ids):
+            logits = plain.forward_logits(model["raw"], model["tensors"], tokens)[-1]
+            _, cdf = plain.sample_token(logits, temperature=0.8, seed=1000 + i, draw_index=draw)
+            u = plain.philox_uniform(1000 + i, draw)
+            low = float(cdf[token - 1]) if token > 0 else 0.0
+            assert low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"request {i} draw {draw}: token {token}"
+            assert abs(output.logprobs[draw] - plain.log_softmax_at(logits, token)) < 1e-4
+            tokens.append(token)
+
+
+def test_seeded_request_does_not_depend_on_its_neighbours(model):
+    """A seeded request alone and in a batch draws the same tokens (tests/unit/test_sampler.py:131-149)."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    params = SamplingParams(max_tokens=6, temperature=1.0, seed=77, ignore_eos=True)
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=64) as engine:
+        alone = engine.generate([model["prompts"][-1]], params)[0].new_token_ids
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=64, seed=5) as engine:
+        others = SamplingParams(max_tokens=6, temperature=1.0, ignore_eos=True)
+        batch = engine.generate([*model["prompts"][:-1], model["prompts"][-1]],
+                                [*[others] * (len(model["prompts"]) - 1), params])
+    assert batch[-1].new_token_ids == alone
+
+
+def test_stop_ids_and_length(model):
+    """A stop id ends the request and stays in the output (tests/unit/test_engine_e2e.py:296-313)."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    prompt = model["prompts"][1]
+    free = plain.greedy_generate(model["raw"], model["tensors"], prompt, 6)
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=64) as engine:
+        out = engine.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0, stop_token_ids=[free[2]]))[0]
+    cut = free.index(free[2]) + 1
+    assert out.new_token_ids == free[:cut] and out.finish_reason == "stop"
+
+
+def test_too_large_prompt_is_refused(model):
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=2) as engine:
+        with pytest.raises(ValueError, match="cache pages"):
+            engine.add_request("big", tiny.random_tokens(model["vocab"], 5 * model["page"], 1))
+
+
+def test_smoke_entry_point():
+    import __graft_entry__
+
+    __graft_entry__.smoke()

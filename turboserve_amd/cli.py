@@ -1,0 +1,181 @@
+"""Command line in the reference's manner (src/turboserve/cli.py:43-95,
+src/turboserve/engine/runtime/engine.py:515-641)::
+
+    turboserve [--log-level L] engine generate PROMPT... --model DIR [options]
+    turboserve engine kv-size --model DIR [options]
+    turboserve engine random-model --config FILE --out DIR --seed N
+    turboserve version | hwinfo [--indent N]
+
+Option names, defaults and meanings are the reference's where it has them (``--max-tokens 64``,
+``--temperature 0`` = greedy, ``--max-num-seqs 8`` for ``generate`` and 64 for ``kv-size``,
+...).  Added here: ``--prompt-ids`` (prompts as comma-separated token ids, so no tokenizer is
+needed), ``--top-k``, ``--repetition-penalty`` and the ``random-model`` command.  Not here:
+``--prefix-caching`` and ``--offline`` (there is no prefix cache and no download).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import logging
+import os
+import sys
+import time
+
+
+def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> None:
+    p.add_argument("--model", "-m", default=os.environ.get("TURBOSERVE_MODEL", ""), help="model folder (config.json + safetensors)")
+    p.add_argument("--device", default="auto", help="auto or cuda[:N]")
+    p.add_argument("--dtype", default="auto", help="auto, bfloat16 or float32")
+    p.add_argument("--block-size", type=int, default=16)
+    p.add_argument("--max-num-seqs", type=int, default=max_num_seqs)
+    p.add_argument("--max-num-batched-tokens", type=int, default=2048)
+
+
+def build_parser() -> argparse.ArgumentParser:
+    parser = argparse.ArgumentParser(prog="turboserve", description="Qwen2 inference engine for one MI355X.")
+    parser.add_argument("--log-level", default=os.environ.get("TURBOSERVE_LOG_LEVEL", "INFO"))
+    top = parser.add_subparsers(dest="command", required=True)
+    top.add_parser("version", help="print the version")
+    hw = top.add_parser("hwinfo", help="print the hardware and software record")
+    hw.add_argument("--indent", type=int, default=2)
+
+    engine = top.add_parser("engine", help="run the engine directly").add_subparsers(dest="engine_command", required=True)
+    gen = engine.add_parser("generate", help="complete one or more prompts and print the results")
+    gen.add_argument("prompt", nargs="*", help="text prompts (need a tokenizer.json in the model folder)")
+    gen.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids; repeatable")
+    _add_engine_options(gen, max_num_seqs=8)
+    gen.add_argument("--max-tokens", type=int, default=64)
+    gen.add_argument("--temperature", type=float, default=0.0)
+    gen.add_argument("--top-p", type=float, default=1.0)
+    gen.add_argument("--top-k", type=int, default=0)
+    gen.add_argument("--repetition-penalty", type=float, default=1.0)
+    gen.add_argument("--seed", type=int, default=None, help="seed for stochastic sampling")
+    gen.add_argument("--num-blocks", type=int, default=None, help="explicit cache pool size; skips memory sizing")
+    gen.add_argument("--ignore-eos", action="store_true")
+    gen.add_argument("--stats", dest="stats", action="store_true")
+    gen.add_argument("--no-stats", dest="stats", action="store_false")
+    gen.set_defaults(stats=False)
+
+    kv = engine.add_parser("kv-size", help="report how many cache blocks a configuration would get, and why")
+    _add_engine_options(kv, max_num_seqs=64)
+    kv.add_argument("--gpu-memory-utilization", type=float, default=0.9)
+    kv.add_argument("--max-model-len", type=int, default=None)
+
+    rnd = engine.add_parser("random-model", help="write a model folder with random weights from a config.json")
+    rnd.add_argument("--config", required=True, help="a config.json")
+    rnd.add_argument("--out", required=True)
+    rnd.add_argument("--seed", type=int, default=0)
+    rnd.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    return parser
+
+
+def _generate(args: argparse.Namespace) -> int:
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    prompts: list = list(args.prompt) + [[int(t) for t in ids.split(",") if t.strip()] for ids in args.prompt_ids]
+    if not prompts:
+        print("no prompt given", file=sys.stderr)
+        return 2
+    if not args.model:
+        print("--model is required", file=sys.stderr)
+        return 2
+    config = EngineConfig(
+        model=args.model, device=args.device, dtype=args.dtype, seed=args.seed,
+        scheduler=SchedulerConfig(
+            max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
+            block_size=args.block_size, num_blocks=args.num_blocks,
+        ),
+    )
+    sampling = SamplingParams(
+        max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
+        repetition_penalty=args.repetition_penalty, seed=args.seed, ignore_eos=args.ignore_eos,
+    )
+    with LLMEngine(config) as engine:
+        started = time.perf_counter()
+        outputs = engine.generate(prompts, sampling)
+        elapsed = time.perf_counter() - started
+        for index, output in enumerate(outputs):
+            print(f"prompt {index}: {prompts[index]}")
+            shown = output.text_delta if engine.tokenizer is not None else output.new_token_ids
+            print(f"output {index}: {shown}")
+            print(f"  {output.output_tokens} tokens, finish_reason={output.finish_reason}")
+        print(f"{len(outputs)} completions in {elapsed:.2f}s")
+        if args.stats:
+            print(json.dumps(engine.stats(), indent=2))
+    return 0
+
+
+def _kv_size(args: argparse.Namespace) -> int:
+    import torch
+
+    from turboserve_amd.cache.layout import CacheLayout
+    from turboserve_amd.cache.sizing import activation_headroom_bytes, size_cache
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.config.model_config import read_config_json
+    from turboserve_amd.weights.random_init import describe_model
+
+    config = EngineConfig(
+        model=args.model, device=args.device, dtype=args.dtype,
+        gpu_memory_utilization=args.gpu_memory_utilization, max_model_len=args.max_model_len,
+        scheduler=SchedulerConfig(
+            max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
+            block_size=args.block_size,
+        ),
+    )
+    model_config, model = describe_model(read_config_json(config.model))
+    itemsize = 2 if config.resolved_dtype() == "bfloat16" else 4
+    activation = activation_headroom_bytes(
+        config.scheduler, hidden=model_config.hidden_size, intermediate=model_config.intermediate_size,
+        qkv_width=model_config.q_proj_size + 2 * model_config.kv_proj_size, vocab=model_config.vocab_size,
+        itemsize=itemsize,
+    )
+    if not torch.cuda.is_available():
+        print("no GPU is visible: the sizing needs the device's memory", file=sys.stderr)
+        return 1
+    sizing = size_cache(
+        CacheLayout.from_model(model), config.scheduler, itemsize=itemsize, activation_bytes=activation,
+        gpu_memory_utilization=config.gpu_memory_utilization, max_model_len=config.max_model_len,
+        device=config.resolved_device(),
+    )
+    print(json.dumps(sizing.to_dict(), indent=2))
+    return 0
+
+
+def _random_model(args: argparse.Namespace) -> int:
+    import torch
+
+    from turboserve_amd.weights.random_init import write_random_model
+
+    with open(args.config, encoding="utf-8") as handle:
+        data = json.load(handle)
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    print(write_random_model(data, args.out, seed=args.seed, dtype=dtype))
+    return 0
+
+
+def main(argv: list[str] | None = None) -> int:
+    args = build_parser().parse_args(argv)
+    logging.basicConfig(level=getattr(logging, str(args.log_level).upper(), logging.INFO),
+                        format="%(asctime)s %(levelname)s %(name)s: %(message)s")
+    if args.command == "version":
+        from turboserve_amd import __version__
+
+        print(f"turboserve_amd {__version__}")
+        return 0
+    if args.command == "hwinfo":
+        from turboserve_amd.hwinfo import collect
+
+        print(json.dumps(collect(), indent=args.indent or None, sort_keys=True))
+        return 0
+    if args.engine_command == "generate":
+        return _generate(args)
+    if args.engine_command == "kv-size":
+        return _kv_size(args)
+    return _random_model(args)
+
+
+if __name__ == "__main__":  # pragma: no cover
+    sys.exit(main())

@@ -1,0 +1,75 @@
+"""Options of the scheduler and of the engine (src/turboserve/engine/core/types.py:484-593).
+
+Names and defaults are the reference's where it has them; what it has and this engine does
+not (prefix caching, tenant policy, speculative and LoRA blocks) is absent.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+
+@dataclass
+class SchedulerConfig:
+    """Limits of one step (types.py:484-518)."""
+
+    max_num_seqs: int = 64
+    max_num_batched_tokens: int = 2048
+    block_size: int = 16
+    num_blocks: int | None = None
+    enable_chunked_prefill: bool = True
+
+    def __post_init__(self) -> None:
+        for name in ("max_num_seqs", "max_num_batched_tokens", "block_size"):
+            value = getattr(self, name)
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be an int >= 1, got {value!r}")
+        if self.num_blocks is not None and (not isinstance(self.num_blocks, int) or self.num_blocks < 1):
+            raise ValueError(f"num_blocks must be an int >= 1 or None, got {self.num_blocks!r}")
+        if self.block_size & (self.block_size - 1):
+            raise ValueError(f"block_size must be a power of two, got {self.block_size}")
+        if self.max_num_batched_tokens < self.block_size:
+            raise ValueError(
+                f"max_num_batched_tokens ({self.max_num_batched_tokens}) must be at least one block "
+                f"({self.block_size})"
+            )
+
+
+@dataclass
+class EngineConfig:
+    """Everything needed to build an engine (types.py:521-593)."""
+
+    model: str
+    tokenizer: str | None = None
+    dtype: str = "auto"  # auto | bfloat16 | float32
+    device: str = "auto"  # auto | cuda | cuda:N
+    gpu_memory_utilization: float = 0.9
+    max_model_len: int | None = None
+    seed: int | None = None
+    scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
+
+    def __post_init__(self) -> None:
+        if self.dtype not in ("auto", "bfloat16", "float32"):
+            raise ValueError(f"unsupported dtype {self.dtype!r}; expected auto, bfloat16 or float32")
+        if self.device != "auto" and not self.device.startswith("cuda"):
+            raise ValueError(f"unsupported device {self.device!r}: this engine runs on the GPU only")
+        if not 0.0 < self.gpu_memory_utilization <= 1.0:
+            raise ValueError(f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization!r}")
+        if self.max_model_len is not None and self.max_model_len < 1:
+            raise ValueError(f"max_model_len must be >= 1, got {self.max_model_len!r}")
+
+    @property
+    def block_size(self) -> int:
+        return self.scheduler.block_size
+
+    @property
+    def num_blocks(self) -> int | None:
+        return self.scheduler.num_blocks
+
+    def resolved_device(self) -> str:
+        return "cuda:0" if self.device in ("auto", "cuda") else self.device
+
+    def resolved_dtype(self) -> str:
+        """``auto`` is bfloat16: the matrix cores' native serving precision here (the
+        reference's ``auto`` picks float16 on a GPU, types.py:566-574)."""
+        return "bfloat16" if self.dtype == "auto" else self.dtype

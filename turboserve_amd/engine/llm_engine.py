@@ -1,0 +1,285 @@
+"""The engine loop: requests in, tokens out, one forward pass per ``step()``
+(src/turboserve/engine/runtime/engine.py:118-508).
+
+One process, one thread, one GPU.  ``step()`` = schedule, run the step function, sample, feed
+the tokens back.  Every collaborator can be passed in, so a test can build an engine around a
+tiny pool or a stand-in runner.
+"""
+
+from __future__ import annotations
+
+import logging
+import time
+from collections.abc import Sequence as SequenceABC
+from typing import Any
+
+import torch
+
+from turboserve_amd.cache.manager import CacheManager
+from turboserve_amd.cache.sizing import CacheSizing, activation_headroom_bytes, size_cache
+from turboserve_amd.config.engine_config import EngineConfig
+from turboserve_amd.engine.detokenizer import StreamingDecoder, get_tokenizer
+from turboserve_amd.engine.outputs import RequestOutput
+from turboserve_amd.engine.scheduler import Scheduler, SchedulerOutput
+from turboserve_amd.engine.sequence import Sequence
+from turboserve_amd.sampling.params import FinishReason, SamplingParams
+
+logger = logging.getLogger(__name__)
+
+
+class LLMEngine:
+    def __init__(
+        self,
+        config: EngineConfig,
+        *,
+        model: Any | None = None,
+        model_config: Any | None = None,
+        tokenizer: Any | None = None,
+        storage: Any | None = None,
+        scheduler: Scheduler | None = None,
+        runner: Any | None = None,
+        sampler: Any | None = None,
+    ) -> None:
+        from turboserve_amd.cache.layout import CacheLayout
+        from turboserve_amd.cache.storage import CacheStorage
+        from turboserve_amd.engine.loading import load_model
+        from turboserve_amd.engine.runner import ModelRunner
+        from turboserve_amd.sampling.sampler import Sampler
+
+        self.config = config
+        if model is None:
+            model_config, model, report = load_model(
+                config.model, dtype=config.resolved_dtype(), device=config.resolved_device()
+            )
+            logger.info("weights: %s", report.summary())
+        self.model = model
+        self.model_config = model_config
+        self.tokenizer = tokenizer if tokenizer is not None else get_tokenizer(config.tokenizer or config.model)
+        self._eos_token_ids = self._resolve_eos_token_ids()
+
+        self.sizing: CacheSizing | None = None
+        sched_cfg = config.scheduler
+        if storage is None and runner is None:
+            layout = CacheLayout.from_model(model)
+            runtime = model.runtime
+            itemsize = torch.empty((), dtype=runtime.dtype).element_size()
+            activation = 0
+            if model_config is not None and sched_cfg.num_blocks is None:
+                activation = activation_headroom_bytes(
+                    sched_cfg, hidden=model_config.hidden_size, intermediate=model_config.intermediate_size,
+                    qkv_width=model_config.q_proj_size + 2 * model_config.kv_proj_size,
+                    vocab=model_config.vocab_size, itemsize=itemsize,
+                )
+            self.sizing = size_cache(
+                layout, sched_cfg, itemsize=itemsize, activation_bytes=activation,
+                gpu_memory_utilization=config.gpu_memory_utilization, max_model_len=config.max_model_len,
+                device=runtime.device,
+            )
+            storage = CacheStorage(layout, self.sizing.num_blocks, sched_cfg.block_size, sched_cfg.max_num_seqs,
+                                   runtime.dtype, runtime.device)
+        self.storage = storage
+        if scheduler is None:
+            if storage is None:
+                raise ValueError("an engine built around a stand-in runner needs its scheduler passed in")
+            cache = CacheManager(storage.layout.windows(), storage.num_pages, sched_cfg.block_size, sched_cfg.max_num_seqs)
+            scheduler = Scheduler(sched_cfg, cache)
+        self.scheduler = scheduler
+        self.runner = runner if runner is not None else ModelRunner(model, storage)
+        self.sampler = sampler if sampler is not None else Sampler(model.runtime.ops)
+        self._decoders: dict[str, StreamingDecoder] = {}
+        self._seed = config.seed if config.seed is not None else time.time_ns() & 0xFFFFFFFF
+        self._num_generated_tokens = 0
+        self._num_prompt_tokens = 0
+        self._closed = False
+
+    # -- helpers --------------------------------------------------------------------------------
+
+    def _resolve_eos_token_ids(self) -> frozenset[int]:
+        """The checkpoint's end-of-sequence ids (engine.py:223-237)."""
+        ids = getattr(self.model_config, "eos_token_ids", ()) or ()
+        return frozenset(int(i) for i in ids)
+
+    @property
+    def eos_token_ids(self) -> frozenset[int]:
+        return self._eos_token_ids
+
+    def encode(self, prompt: str) -> list[int]:
+        if self.tokenizer is None:
+            raise TypeError("no tokenizer is configured: pass prompts as token ids")
+        return [int(t) for t in self.tokenizer.encode(prompt, add_special_tokens=False)]
+
+    def _request_seed(self, sampling: SamplingParams, seq_index: int) -> int:
+        """A request's own seed, or one derived from the engine's seed and its arrival number."""
+        if sampling.seed is not None:
+            return int(sampling.seed) & 0xFFFFFFFFFFFFFFFF
+        return ((self._seed & 0xFFFFFFFF) << 32 | (seq_index & 0xFFFFFFFF)) ^ 0x9E3779B97F4A7C15
+
+    # -- requests -------------------------------------------------------------------------------
+
+    def add_request(
+        self,
+        request_id: str,
+        prompt: str | SequenceABC[int],
+        sampling: SamplingParams | None = None,
+        *,
+        priority: int = 0,
+        arrival: float | None = None,
+    ) -> Sequence:
+        """Queue a request given as text or as token ids (engine.py:283-323)."""
+        if self._closed:
+            raise RuntimeError("engine is closed")
+        token_ids = self.encode(prompt) if isinstance(prompt, str) else [int(t) for t in prompt]
+        if not token_ids:
+            raise ValueError(f"request {request_id!r} has an empty prompt")
+        vocab = getattr(self.model_config, "vocab_size", None)
+        if vocab is not None and any(not 0 <= t < vocab for t in token_ids):
+            raise ValueError(f"request {request_id!r} has a token id outside the vocabulary of {vocab}")
+        sampling = sampling or SamplingParams()
+        seq = self.scheduler.add_request(
+            request_id, token_ids, sampling, priority=priority, arrival=arrival,
+            sample_seed=self._request_seed(sampling, self.scheduler._next_seq_id),
+        )
+        self._decoders[request_id] = StreamingDecoder(self.tokenizer, sampling.stop)
+        self._num_prompt_tokens += len(token_ids)
+        return seq
+
+    def abort(self, request_id: str, *, now: float | None = None) -> bool:
+        self._decoders.pop(request_id, None)
+        return self.scheduler.abort(request_id, now=now)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    # -- the step -------------------------------------------------------------------------------
+
+    def step(self, *, now: float | None = None) -> list[RequestOutput]:
+        """Advance every scheduled request.  An empty list is normal: nothing queued, only
+        unfinished portions of prompts ran, or everything scheduled was preempted
+        (engine.py:340-356)."""
+        if self._closed:
+            raise RuntimeError("engine is closed")
+        timestamp = time.perf_counter() if now is None else now
+        scheduled = self.scheduler.schedule(now=timestamp)
+        outputs = [self._output_for_dropped(seq) for seq in scheduled.dropped]
+        if scheduled.is_empty:
+            return outputs
+        tokens, logprobs = self._execute(scheduled)
+        outputs.extend(self._process(scheduled, tokens, logprobs, now=timestamp))
+        return outputs
+
+    def _execute(self, scheduled: SchedulerOutput) -> tuple[list[int], list[float] | None]:
+        logits = self.runner.step(scheduled.entries(), fresh_state_slots=scheduled.fresh_state_slots)
+        sampled = scheduled.sampled()
+        if not sampled:
+            return [], None
+        result = self.sampler.sample_sequences(logits, [item.seq for item in sampled])
+        return result.token_ids, result.logprobs
+
+    def _process(self, scheduled, tokens, logprobs, *, now: float) -> list[RequestOutput]:
+        """Feed sampled tokens back: stop checks, text, per-request deltas (engine.py:366-410)."""
+        outputs = []
+        for index, (item, token) in enumerate(zip(scheduled.sampled(), tokens)):
+            seq = item.seq
+            if seq.is_finished:
+                continue
+            logprob = None
+            if logprobs is not None and seq.sampling.logprobs:
+                logprob = logprobs[index]
+            reason = self.scheduler.append_token(seq, token, eos_token_ids=self._eos_token_ids, logprob=logprob, now=now)
+            outputs.append(self._emit(seq, token, reason, logprob, now=now))
+        self._num_generated_tokens += len(outputs)
+        return outputs
+
+    def _emit(self, seq: Sequence, token: int, reason, logprob, *, now: float) -> RequestOutput:
+        decoder = self._decoders.get(seq.request_id)
+        if decoder is None:
+            decoder = self._decoders[seq.request_id] = StreamingDecoder(self.tokenizer, seq.sampling.stop)
+        delta = decoder.feed((token,))
+        text = delta.text
+        if delta.stopped and reason is None:
+            self.scheduler.finish(seq, FinishReason.STOP, now=now)
+            reason = FinishReason.STOP
+        elif reason is not None and not delta.stopped:
+            text += decoder.finish()
+        if reason is not None:
+            self._decoders.pop(seq.request_id, None)
+        return RequestOutput(
+            request_id=seq.request_id, new_token_ids=[token], text_delta=text, finished=reason is not None,
+            finish_reason=reason, timing=seq.timing, prompt_tokens=seq.num_prompt_tokens,
+            output_tokens=seq.num_output_tokens, logprobs=[] if logprob is None else [logprob],
+        )
+
+    def _output_for_dropped(self, seq: Sequence) -> RequestOutput:
+        self._decoders.pop(seq.request_id, None)
+        return RequestOutput(
+            request_id=seq.request_id, finished=True, finish_reason=seq.finish_reason, timing=seq.timing,
+            prompt_tokens=seq.num_prompt_tokens, output_tokens=seq.num_output_tokens,
+        )
+
+    # -- convenience ----------------------------------------------------------------------------
+
+    def generate(
+        self,
+        prompts: SequenceABC[str | SequenceABC[int]],
+        sampling: SamplingParams | SequenceABC[SamplingParams] | None = None,
+        *,
+        request_id_prefix: str = "gen",
+    ) -> list[RequestOutput]:
+        """Run prompts to completion; one aggregate result each, in input order (engine.py:414-448)."""
+        order = []
+        for index, prompt in enumerate(prompts):
+            request_id = f"{request_id_prefix}-{index}"
+            params = sampling[index] if isinstance(sampling, (list, tuple)) else sampling
+            self.add_request(request_id, prompt, params)
+            order.append(request_id)
+        merged: dict[str, RequestOutput] = {}
+        while self.has_unfinished():
+            for output in self.step():
+                current = merged.get(output.request_id)
+                if current is None:
+                    merged[output.request_id] = output
+                    continue
+                current.new_token_ids.extend(output.new_token_ids)
+                current.logprobs.extend(output.logprobs)
+                current.text_delta += output.text_delta
+                current.finished = output.finished
+                current.finish_reason = output.finish_reason
+                current.output_tokens = output.output_tokens
+                current.timing = output.timing
+        return [merged[request_id] for request_id in order if request_id in merged]
+
+    # -- observability --------------------------------------------------------------------------
+
+    def stats(self) -> dict[str, int | float | str]:
+        """Flat, JSON-safe counters (engine.py:452-484)."""
+        out: dict[str, int | float | str] = dict(self.scheduler.stats())
+        out["num_prompt_tokens"] = self._num_prompt_tokens
+        out["num_generated_tokens"] = self._num_generated_tokens
+        out["model"] = self.config.model
+        runtime = getattr(self.model, "runtime", None)
+        if runtime is not None:
+            out["device"] = str(runtime.device)
+            out["dtype"] = str(runtime.dtype).removeprefix("torch.")
+        if self.storage is not None:
+            out["block_size"] = self.storage.page_size
+            out["num_kv_blocks"] = min(self.storage.num_pages) if self.storage.num_pages else 0
+            out["kv_bytes"] = self.storage.num_bytes()
+        return out
+
+    def close(self) -> None:
+        if self._closed:
+            return
+        self._closed = True
+        self.scheduler.reset()
+        self._decoders.clear()
+        self.storage = None
+        if self.runner is not None and hasattr(self.runner, "release"):
+            self.runner.release()
+        if torch.cuda.is_available():
+            torch.cuda.empty_cache()
+
+    def __enter__(self) -> "LLMEngine":
+        return self
+
+    def __exit__(self, *exc: object) -> None:
+        self.close()

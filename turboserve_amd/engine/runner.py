@@ -30,6 +30,11 @@ class ModelRunner:
         self.vocab_size = model.plan.vocab_size
         self.num_steps = 0
 
+    def release(self) -> None:
+        """Drop the cache tensors (the engine is closing)."""
+        self.views = []
+        self.storage = None
+
     def context_for(self, entries: Sequence[StepEntry]) -> StepContext:
         if self.check:
             vocab = self.vocab_size

@@ -1,0 +1,101 @@
+"""Batched sampling with per-request options (src/turboserve/engine/core/sampler.py:171-297).
+
+The stages and their order are the reference's (penalty, log-probabilities, temperature,
+top-k, top-p, draw); they run in one HIP kernel launch for the whole batch, one block per row.
+A request's randomness is its own: the draw for its n-th token uses a counter-based generator
+keyed by the request's seed with counter n, so a row does not depend on its batch neighbours
+or on any global generator state (the property the reference gets from per-request
+``torch.Generator`` objects, sampler.py:258-297), and a request that was preempted and
+recomputed continues with the same numbers.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence as SequenceABC
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from turboserve_amd.engine.sequence import Sequence
+from turboserve_amd.sampling.params import SamplingParams
+
+
+@dataclass
+class SamplerOutput:
+    token_ids: list[int]
+    logprobs: list[float] | None = None  # nan for rows that did not ask (sampler.py:66-74)
+
+
+class Sampler:
+    def __init__(self, ops) -> None:
+        self.ops = ops
+
+    def sample(
+        self,
+        logits: torch.Tensor,
+        params: SequenceABC[SamplingParams],
+        seeds: SequenceABC[int],
+        draw_indices: SequenceABC[int],
+        histories: SequenceABC[SequenceABC[int]] | None = None,
+    ) -> SamplerOutput:
+        """One token per row of ``logits [n, V]`` (32-bit, left untouched).
+
+        ``seeds[i]`` / ``draw_indices[i]``: key and counter of row ``i``'s draw.
+        ``histories[i]``: prompt + output tokens, read only when the row has a repetition
+        penalty other than 1."""
+        rows = int(logits.shape[0])
+        if len(params) != rows or len(seeds) != rows or len(draw_indices) != rows:
+            raise ValueError(f"{len(params)} params / {len(seeds)} seeds / {len(draw_indices)} counters for {rows} rows")
+        if histories is not None and len(histories) != rows:
+            raise ValueError(f"{len(histories)} histories for {rows} rows of logits")
+        if rows == 0:
+            return SamplerOutput(token_ids=[])
+        if all(p.is_plain_greedy for p in params):
+            return SamplerOutput(token_ids=self.ops.argmax(logits).tolist())
+
+        want_logprobs = any(p.logprobs for p in params)
+        history_start = [0]
+        flat_history: list[int] = []
+        for i, p in enumerate(params):
+            if p.repetition_penalty != 1.0 and histories is not None:
+                flat_history.extend(int(t) for t in histories[i])
+            history_start.append(len(flat_history))
+        floats = np.asarray(
+            [[p.temperature for p in params], [p.top_p for p in params], [p.repetition_penalty for p in params]],
+            dtype=np.float32,
+        )
+        seeds64 = np.asarray([int(s) & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64)
+        ints = np.concatenate([
+            np.asarray([p.top_k for p in params], dtype=np.int32),
+            (seeds64 & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32),
+            (seeds64 >> np.uint64(32)).astype(np.uint32).view(np.int32),
+            np.asarray([int(d) & 0xFFFFFFFF for d in draw_indices], dtype=np.uint32).view(np.int32),
+            np.asarray(history_start, dtype=np.int32),
+            np.asarray(flat_history, dtype=np.int32),
+        ])
+        device = logits.device
+        fdev = torch.from_numpy(floats).to(device)
+        idev = torch.from_numpy(ints).to(device)
+        top_k, seed_lo, seed_hi, draw, hstart, hist = torch.split(
+            idev, [rows, rows, rows, rows, rows + 1, len(flat_history)]
+        )
+        tokens, logprobs = self.ops.sample(
+            logits, fdev[0], top_k, fdev[1], fdev[2], seed_lo, seed_hi, draw, hist, hstart, want_logprobs
+        )
+        out = SamplerOutput(token_ids=tokens.tolist())
+        if logprobs is not None:
+            values = logprobs.tolist()
+            out.logprobs = [v if p.logprobs else float("nan") for v, p in zip(values, params)]
+        return out
+
+    def sample_sequences(self, logits: torch.Tensor, sequences: SequenceABC[Sequence]) -> SamplerOutput:
+        """Sample for requests: options, seed, draw counter (= tokens produced so far) and,
+        only if a penalty is set, the token history of each (sampler.py:240-256)."""
+        return self.sample(
+            logits,
+            [seq.sampling for seq in sequences],
+            [seq.sample_seed for seq in sequences],
+            [seq.num_output_tokens for seq in sequences],
+            [seq.token_ids if seq.sampling.repetition_penalty != 1.0 else () for seq in sequences],
+        )

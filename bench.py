@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at the Qwen2.5-7B layer sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one decode step of the whole engine path: the step function over a batch of
+single tokens against the paged cache, logits, greedy sampling, tokens back on the host.
+The default run has the 7B shape of BASELINE.json's configs[2], random weights
+(N(0, 0.02), norm gains 1), a batch of 8 requests each holding a context of 8,192 tokens
+(cache filled with random keys and values; what is timed is real decode steps on top of it).
+One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times one
+2,048-token prompt; ``roofline`` prices the decode step against HBM bandwidth; ``points``
+holds decode at batch 1 and 64.  Peaks are the published MI355X figures: HBM 8 TB/s, dense
+bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+#: BASELINE.json configs[2]: Qwen2.5-7B shape.
+SHAPE_7B = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 3584,
+    "num_hidden_layers": 28,
+    "num_attention_heads": 28,
+    "num_key_value_heads": 4,
+    "head_dim": 128,
+    "intermediate_size": 18944,
+    "vocab_size": 152064,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False,
+    "use_sliding_window": False,
+    "max_position_embeddings": 32768,
+}
+CONTEXT = 8192
+PREFILL_TOKENS = 2048
+PAGE = 16
+
+
+def parse_args() -> argparse.Namespace:
+    p = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=64)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=CONTEXT)
+    p.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    p.add_argument("--no-prefill", action="store_true")
+    return p.parse_args()
+
+
+class DecodeBench:
+    """Requests with a given context already in the cache, decoded one token per step through
+    the engine's own cache manager, step function and sampler."""
+
+    def __init__(self, model, config, batch: int, context: int, steps_total: int) -> None:
+        import torch
+
+        from turboserve_amd.cache.manager import CacheManager
+        from turboserve_amd.engine.loading import build_storage
+        from turboserve_amd.engine.runner import ModelRunner
+        from turboserve_amd.sampling.sampler import Sampler
+
+        self.torch = torch
+        self.batch = batch
+        self.context = context
+        pages_per_request = -(-(context + steps_total + 1) // PAGE)
+        num_pages = batch * pages_per_request
+        self.storage = build_storage(model, num_pages, PAGE, batch)
+        for pages in self.storage.pages:
+            pages.normal_(0.0, 0.5)
+        self.manager = CacheManager(self.storage.layout.windows(), num_pages, PAGE, batch)
+        self.runner = ModelRunner(model, self.storage, check=False)
+        self.sampler = Sampler(model.runtime.ops)
+        generator = torch.Generator().manual_seed(1234)
+        self.tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
+        for request in range(batch):
+            self.manager.admit(request)
+            self.manager.append(request, context - 1)  # the context's last token is decoded below
+
+    def step(self) -> None:
+        from turboserve_amd.engine.batch import StepEntry
+        from turboserve_amd.sampling.params import SamplingParams
+
+        entries = []
+        for request in range(self.batch):
+            held = self.manager.get(request)
+            start = held.num_tokens
+            slots = self.manager.append(request, 1)
+            entries.append(StepEntry(request=request, tokens=[self.tokens[request]], start=start,
+                                     tables=held.tables, slots=slots, state_slot=held.state_slot, want=[0]))
+        logits = self.runner.step(entries)
+        greedy = SamplingParams(temperature=0.0)
+        out = self.sampler.sample(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
+        self.tokens = out.token_ids
+
+    def run(self, steps: int, warmup: int) -> float:
+        """Seconds for ``steps`` decode steps after ``warmup`` untimed ones."""
+        torch = self.torch
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for _ in range(steps):
+            self.step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - started
+
+    def close(self) -> None:
+        self.runner.release()
+        self.storage = None
+        self.torch.cuda.empty_cache()
+
+
+def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
+    """Bytes a decode step has to read: every weight it uses once (all but the embedding
+    table, of which it reads one row per request) and the cache of the live requests."""
+    h, i, v = config.hidden_size, config.intermediate_size, config.vocab_size
+    qkv = config.q_proj_size + 2 * config.kv_proj_size
+    per_layer = h * qkv + qkv + config.q_proj_size * h + 3 * h * i + 2 * h
+    weights = (layers * per_layer + h + v * h + batch * h) * itemsize
+    cache = batch * context * 2 * layers * config.kv_proj_size * itemsize
+    return float(weights + cache)
+
+
+def prefill_flops(config, layers: int, tokens: int) -> float:
+    """Flops of one whole-prompt step: the projections (2 flops per weight per token), causal
+    attention (4 * Hq * D * T^2 / 2 per layer) and one head row."""
+    h, i = config.hidden_size, config.intermediate_size
+    qkv = config.q_proj_size + 2 * config.kv_proj_size
+    linear = layers * (h * qkv + config.q_proj_size * h + 3 * h * i)
+    attention = layers * 4 * config.q_proj_size * tokens * tokens / 2
+    return 2.0 * tokens * linear + attention + 2.0 * config.vocab_size * h
+
+
+def run_prefill(model, config, tokens: int, repeats: int = 3) -> float:
+    """Seconds (best of ``repeats``) for one step over a ``tokens``-long prompt, to its last
+    position's logits on the host."""
+    import torch
+
+    from turboserve_amd.cache.manager import CacheManager
+    from turboserve_amd.engine.batch import StepEntry
+    from turboserve_amd.engine.loading import build_storage
+    from turboserve_amd.engine.runner import ModelRunner
+
+    num_pages = -(-tokens // PAGE)
+    storage = build_storage(model, num_pages, PAGE, 1)
+    manager = CacheManager(storage.layout.windows(), num_pages, PAGE, 1)
+    runner = ModelRunner(model, storage, check=False)
+    generator = torch.Generator().manual_seed(4321)
+    prompt = torch.randint(0, config.vocab_size, (tokens,), generator=generator).tolist()
+    best = float("inf")
+    for _ in range(repeats + 1):
+        held = manager.admit("p")
+        slots = manager.append("p", tokens)
+        entry = StepEntry(request="p", tokens=prompt, start=0, tables=held.tables, slots=slots,
+                          state_slot=held.state_slot, want=[tokens - 1])
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        logits = runner.step([entry])
+        logits.argmax(dim=-1).tolist()
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - started)
+        manager.free("p")
+    runner.release()
+    del storage
+    torch.cuda.empty_cache()
+    return best
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU by design)")
+        return 2
+    import torch
+
+    from turboserve_amd.engine.loading import build_model, make_runtime, resolve_run_dtype
+    from turboserve_amd.hwinfo import collect
+    from turboserve_amd.weights.random_init import random_tensors_on_device
+
+    shape = dict(SHAPE_7B)
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is not None:
+        shape["num_hidden_layers"] = args.layers
+    dtype = resolve_run_dtype(args.dtype)
+    runtime = make_runtime(dtype, "cuda:0")
+    config, model = build_model(shape, runtime)
+    random_tensors_on_device(model, seed=0)
+    layers = config.num_hidden_layers
+    itemsize = 2 if dtype == torch.bfloat16 else 4
+    dtype_key = "bf16" if dtype == torch.bfloat16 else "fp32"
+
+    def decode_rate(batch: int, steps: int, warmup: int) -> tuple[float, float]:
+        bench = DecodeBench(model, config, batch, args.context, steps + warmup)
+        seconds = bench.run(steps, warmup)
+        bench.close()
+        return batch * steps / seconds, seconds / steps
+
+    value, step_seconds = decode_rate(args.batch, args.steps, args.warmup)
+    mean_context = args.context + args.warmup + args.steps / 2
+    read = decode_bytes(config, layers, args.batch, mean_context, itemsize)
+    achieved = read / step_seconds / 1e9
+    result = {
+        "metric": "decode tok/s (Qwen2.5-7B shape, paged cache, one MI355X)",
+        "value": round(value, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_seconds * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype_key,
+        "data": "synthetic: random weights N(0,0.02), uniform-random token ids, cache pre-filled with random keys/values",
+        "config": {
+            "model": "Qwen2.5-7B shape (Qwen2ForCausalLM)",
+            "global_batch": args.batch,
+            "seq_len": args.context,
+            "parallelism": "single GPU",
+            "layers": layers,
+            "layers_of_shape": full_layers,
+            "hidden_size": config.hidden_size,
+            "num_attention_heads": config.num_attention_heads,
+            "num_key_value_heads": config.num_key_value_heads,
+            "head_dim": config.head_dim,
+            "intermediate_size": config.intermediate_size,
+            "vocab_size": config.vocab_size,
+            "rope_theta": config.rope_theta,
+            "rms_norm_eps": config.rms_norm_eps,
+            "tie_word_embeddings": config.tie_word_embeddings,
+            "page_size": PAGE,
+            "prefill_tokens": PREFILL_TOKENS,
+            "sampling": "greedy",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+        },
+    }
+    if not args.no_prefill:
+        seconds = run_prefill(model, config, PREFILL_TOKENS)
+        flops = prefill_flops(config, layers, PREFILL_TOKENS)
+        result["prefill"] = {
+            "value": round(PREFILL_TOKENS / seconds, 1),
+            "tokens": PREFILL_TOKENS,
+            "ms": round(seconds * 1e3, 3),
+            "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4),
+        }
+    if not args.no_points:
+        points = {}
+        for batch in (1, 64):
+            rate, _ = decode_rate(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{batch}"] = round(rate, 2)
+        result["points"] = points
+    info = collect()
+    result["hw"] = {"gpu": info["gpu_name"], "torch": info["torch"]["version"], "hip": info["torch"]["hip_version"],
+                    "git": (info["git"]["sha"] or "")[:12]}
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

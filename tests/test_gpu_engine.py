@@ -55,10 +55,10 @@ def test_preemption_keeps_the_tokens(model):
     (tests/unit/test_engine_e2e.py:149-165)."""
     from turboserve_amd.sampling.params import SamplingParams
 
-    new = 10
+    new = 20
     want = [plain.greedy_generate(model["raw"], model["tensors"], p, new) for p in model["prompts"]]
     longest = max(len(p) for p in model["prompts"]) + new
-    blocks = -(-longest // model["page"]) + 1  # one request fits, all of them do not
+    blocks = -(-longest // model["page"])  # the longest request just fits alone; together they do not
     with make_engine(model["folder"], "float32", model["page"], num_blocks=blocks, budget=64) as engine:
         outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
         assert [o.new_token_ids for o in outputs] == want

@@ -1,0 +1,378 @@
+"""Each kernel alone against its plain reference, at sizes other than the tiny engines': widths
+and vocabularies that are no power of two, several head sizes and group sizes, scrambled
+pages, windows, long contexts with one far key made to stand out."""
+
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from turboserve_amd.kernels.ops import Ops
+
+    return Ops(DEV)
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+# -- rows -------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tokens,hidden", [(1, 72), (5, 3584), (3, 1100), (2, 4100)])
+def test_rmsnorm_and_fused_residual(ops, dtype, tokens, hidden):
+    g = torch.Generator().manual_seed(hidden)
+    x = (torch.randn(tokens, hidden, generator=g) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    eps = 1e-5
+    want = plain.rms_norm(x.float(), w.float(), eps)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps).float().cpu()
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+    residual = torch.randn(tokens, hidden, generator=g)
+    total = residual + x.float()
+    res_dev = residual.to(DEV)
+    got = ops.add_rmsnorm(res_dev, x.to(DEV), w.to(DEV), eps).float().cpu()
+    torch.testing.assert_close(res_dev.cpu(), total, rtol=0, atol=1e-6)  # the sum is kept in 32-bit
+    torch.testing.assert_close(got, plain.rms_norm(total, w.float(), eps), **tol(dtype))
+
+    rows = torch.tensor([tokens - 1, 0], dtype=torch.int32, device=DEV)
+    res_dev = residual.to(DEV)
+    got = ops.add_rmsnorm(res_dev, x.to(DEV), w.to(DEV), eps, rows).float().cpu()
+    torch.testing.assert_close(res_dev.cpu(), residual, rtol=0, atol=0)  # untouched with rows
+    torch.testing.assert_close(got, plain.rms_norm(total, w.float(), eps)[[tokens - 1, 0]], **tol(dtype))
+
+
+def test_rmsnorm_rounds_before_the_gain(ops):
+    """bfloat16: the normalised value is rounded to bfloat16 before the gain multiplies it
+    (src/turboserve/engine/model/layers.py:208); a single rounding of the product differs."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 512, generator=g).bfloat16()
+    w = (1 + 0.3 * torch.randn(512, generator=g)).bfloat16()
+    want = plain.rms_norm(x, w, 1e-6)  # bfloat16 in, reference order of roundings
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-6).cpu()
+    assert (got != want).float().mean() < 0.01  # rsqrt may differ in the last bit now and then
+    single = (w.float() * (x.float() * torch.rsqrt((x.float() ** 2).mean(-1, keepdim=True) + 1e-6))).bfloat16()
+    assert (single != want).float().mean() > 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_swiglu_gather(ops, dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(301, 72, generator=g).to(dtype)
+    ids = torch.tensor([5, 300, 0, 5], dtype=torch.int32)
+    got = ops.embed(table.to(DEV), ids.to(DEV)).cpu()
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got, table.float()[ids.long()], rtol=0, atol=0)
+
+    gu = torch.randn(7, 2 * 200, generator=g).to(dtype)
+    want = torch.nn.functional.silu(gu.float()[:, :200]) * gu.float()[:, 200:]
+    torch.testing.assert_close(ops.swiglu(gu.to(DEV)).float().cpu(), want, **tol(dtype))
+    zero_up = gu.clone()
+    zero_up[:, 200:] = 0
+    assert float(ops.swiglu(zero_up.to(DEV)).abs().max()) == 0.0
+
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32)
+    torch.testing.assert_close(ops.gather_rows(gu.to(DEV), rows.to(DEV)).cpu(), gu[rows.long()], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 100), (70, 65, 33), (130, 320, 96)])
+def test_gemm_plain(ops, dtype, m, n, k):
+    g = torch.Generator().manual_seed(m * n)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    w = torch.randn(n, k, generator=g).to(dtype)
+    b = torch.randn(n, generator=g).to(dtype)
+    want = x.double() @ w.double().T + b.double()
+    got = ops.gemm_plain(x.to(DEV), w.to(DEV), b.to(DEV)).double().cpu()
+    bound = 1e-5 if dtype == torch.float32 else 2e-2
+    assert float((got - want).abs().max()) <= bound * math.sqrt(k) * 4
+    got32 = ops.gemm_plain(x.to(DEV), w.to(DEV), out_float32=True)
+    assert got32.dtype == torch.float32
+    assert float((got32.double().cpu() - x.double() @ w.double().T).abs().max()) <= 1e-5 * math.sqrt(k) * 4
+    zero = ops.gemm_plain(x.to(DEV), torch.zeros_like(w).to(DEV), b.to(DEV)).float().cpu()
+    torch.testing.assert_close(zero, b.float().expand(m, n), rtol=0, atol=0)  # a dropped bias would show
+
+
+def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(77, 200, generator=g)
+    w = torch.randn(150, 200, generator=g)
+    full = ops.gemm_plain(x.to(DEV), w.to(DEV)).cpu()
+    one = ops.gemm_plain(x[40:41].to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(full[40:41], one)
+
+
+# -- rotary + cache write ---------------------------------------------------------------------------
+
+
+def scatter_reference(k, v, slots, num_pages, kv_heads, page, dim):
+    """Key pages [NB, Hkv, BS, D] and transposed value pages [NB, Hkv, D, BS] after writing."""
+    kp = torch.zeros(num_pages, kv_heads, page, dim)
+    vp = torch.zeros(num_pages, kv_heads, dim, page)
+    for t, slot in enumerate(slots):
+        if slot < 0:
+            continue
+        kp[slot // page, :, slot % page, :] = k[t]
+        vp[slot // page, :, :, slot % page] = v[t]
+    return kp, vp
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,dim,page,theta,factor", [(4, 2, 16, 16, 1e4, 1.0), (3, 1, 32, 8, 1e6, 1.0),
+                                                                  (5, 5, 48, 32, 5e5, 2.0), (14, 2, 128, 16, 1e6, 1.0)])
+def test_rope_store(ops, dtype, heads, kv_heads, dim, page, theta, factor):
+    from turboserve_amd.parts.rope import rotary_tables
+
+    g = torch.Generator().manual_seed(dim)
+    tokens, num_pages = 9, 6
+    qkv = torch.randn(tokens, (heads + 2 * kv_heads) * dim, generator=g).to(dtype)
+    positions = torch.tensor([0, 1, 2, 40, 41, 7, 100, 3, 64], dtype=torch.int32)
+    slot_pool = list(range(num_pages * page))
+    random.Random(1).shuffle(slot_pool)
+    slots = slot_pool[:tokens]
+    slots[4] = -1  # no write for this token
+    cos, sin = rotary_tables(128, dim, theta, factor)
+    kp = torch.zeros(num_pages, kv_heads, page, dim, dtype=dtype, device=DEV)
+    vp = torch.zeros(num_pages, kv_heads, dim, page, dtype=dtype, device=DEV)
+    dev = qkv.to(DEV)
+    ops.rope_store(dev, kp, vp, cos.to(DEV), sin.to(DEV), positions.to(DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                   heads, kv_heads, dim, page, 100)
+    q = qkv.float()[:, : heads * dim].view(tokens, heads, dim)
+    k = qkv.float()[:, heads * dim:(heads + kv_heads) * dim].view(tokens, kv_heads, dim)
+    v = qkv.float()[:, (heads + kv_heads) * dim:].view(tokens, kv_heads, dim)
+    angles = plain.rope_angles(positions, dim, theta, factor)
+    q_want, k_want = plain.apply_rope(q, angles), plain.apply_rope(k, angles)
+    got = dev.float().cpu()
+    torch.testing.assert_close(got[:, : heads * dim].view(tokens, heads, dim), q_want, **tol(dtype))
+    torch.testing.assert_close(got[:, heads * dim:(heads + kv_heads) * dim].view(tokens, kv_heads, dim), k_want, **tol(dtype))
+    torch.testing.assert_close(got[:, (heads + kv_heads) * dim:], qkv.float()[:, (heads + kv_heads) * dim:], rtol=0, atol=0)
+    kp_want, vp_want = scatter_reference(k_want, v, slots, num_pages, kv_heads, page, dim)
+    torch.testing.assert_close(kp.float().cpu(), kp_want, **tol(dtype))
+    torch.testing.assert_close(vp.float().cpu(), vp_want, rtol=0, atol=0)
+    with pytest.raises(Exception, match="beyond the rotary tables"):
+        ops.rope_store(dev, kp, vp, cos.to(DEV), sin.to(DEV), positions.to(DEV), None, heads, kv_heads, dim, page, 128)
+
+
+# -- attention --------------------------------------------------------------------------------------
+
+
+class PagedCase:
+    """Requests with dense random keys/values scattered into scrambled pages, and the plain
+    attention of each request's last ``q_len`` positions."""
+
+    def __init__(self, dtype, heads, kv_heads, dim, page, seqs, window=None, seed=0, spike=None):
+        g = torch.Generator().manual_seed(seed)
+        self.heads, self.kv_heads, self.dim, self.page, self.window = heads, kv_heads, dim, page, window
+        self.seqs = seqs  # list of (context_len, query_len)
+        need = sum(-(-c // page) for c, _ in seqs)
+        num_pages = need + 3
+        order = list(range(num_pages))
+        random.Random(seed).shuffle(order)  # scrambled, interleaved block ids
+        width = max(-(-c // page) for c, _ in seqs)
+        self.table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+        self.kp = torch.randn(num_pages, kv_heads, page, dim, generator=g).to(dtype)  # stale data everywhere
+        self.vp = torch.randn(num_pages, kv_heads, dim, page, generator=g).to(dtype)
+        self.q, self.expected, self.positions, self.token_seq, self.qsl = [], [], [], [], [0]
+        used = 0
+        for s, (ctx, qlen) in enumerate(seqs):
+            k = torch.randn(ctx, kv_heads, dim, generator=g).to(dtype)
+            v = torch.randn(ctx, kv_heads, dim, generator=g).to(dtype)
+            q = torch.randn(qlen, heads, dim, generator=g).to(dtype)
+            if spike is not None and ctx > spike:
+                # One far key dominates every query's scores: a kernel that skips it fails.
+                k[spike] = 0
+                k[spike, :, 0] = 16.0
+                q[:] = 0
+                q[:, :, 0] = 16.0
+                v[spike] = 5.0
+            pages = order[used:used + -(-ctx // page)]
+            used += len(pages)
+            self.table[s, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
+            for pos in range(ctx):
+                self.kp[pages[pos // page], :, pos % page, :] = k[pos]
+                self.vp[pages[pos // page], :, :, pos % page] = v[pos]
+            qpos = torch.arange(ctx - qlen, ctx)
+            mask = plain.attention_mask(qpos, ctx, window)
+            self.expected.append(plain.attention(q.float(), k.float(), v.float(), mask, dim ** -0.5))
+            self.q.append(q)
+            self.positions.extend(qpos.tolist())
+            self.token_seq.extend([s] * qlen)
+            self.qsl.append(self.qsl[-1] + qlen)
+        self.q = torch.cat(self.q).reshape(-1, heads * dim)
+        self.expected = torch.cat(self.expected).reshape(-1, heads * dim)
+
+    def dev(self, t, dtype=None):
+        return (t if dtype is None else t.to(dtype)).to(DEV)
+
+    def ints(self, values):
+        return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+ATTENTION_GEOMETRIES = [
+    # heads, kv_heads, dim, page
+    (4, 2, 16, 16),
+    (3, 1, 32, 8),
+    (5, 5, 48, 32),
+    (14, 2, 128, 16),   # G = 7, as the 7B shape
+    (8, 1, 64, 16),
+    (40, 2, 80, 16),    # G = 20: more than one tile of heads per KV head
+    (2, 1, 256, 64),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_GEOMETRIES)
+@pytest.mark.parametrize("window", [None, 20])
+def test_attention_generic(ops, dtype, heads, kv_heads, dim, page, window):
+    case = PagedCase(dtype, heads, kv_heads, dim, page, [(70, 1), (33, 33), (90, 7), (1, 1), (129, 2)], window, seed=dim)
+    got = ops.paged_attention_generic(
+        case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.token_seq), case.ints(case.positions), heads, dim ** -0.5, window,
+    ).float().cpu()
+    torch.testing.assert_close(got, case.expected, **tol(dtype))
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_GEOMETRIES)
+@pytest.mark.parametrize("window", [None, 20, 300])
+def test_attention_decode_mfma(ops, heads, kv_heads, dim, page, window):
+    contexts = [70, 1, 33, 600, 129, 32, 31, 257]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, [(c, 1) for c in contexts], window, seed=dim + 1)
+    out = torch.zeros(len(contexts), heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints(contexts), 0, len(contexts), heads, dim ** -0.5, window, max(contexts),
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+
+
+def test_attention_decode_mfma_far_key_and_subrange(ops):
+    """A context of thousands of keys where one far key carries the result, split over many
+    wavefronts; and a launch over a sub-range of the step's requests (rows before it untouched)."""
+    heads, kv_heads, dim, page = 28, 4, 128, 16
+    contexts = [4100, 3000, 5, 2049]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, [(c, 1) for c in contexts], None, seed=5, spike=1234)
+    out = torch.full((len(contexts), heads * dim), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints(contexts), 1, 3, heads, dim ** -0.5, None, max(contexts),
+    )
+    got = out.float().cpu()
+    assert float((got[0] - 7.0).abs().max()) == 0.0
+    torch.testing.assert_close(got[1:], case.expected[1:], **tol(torch.bfloat16))
+    assert float(case.expected[1].abs().mean()) > 4.0  # the spike's value dominates
+
+
+# -- sampling ---------------------------------------------------------------------------------------
+
+
+def test_argmax_lowest_index_of_ties(ops):
+    logits = torch.zeros(3, 152064)
+    logits[0, 77] = 1.0
+    logits[0, 151000] = 1.0
+    logits[1, 152063] = 2.0
+    got = ops.argmax(logits.to(DEV)).cpu().tolist()
+    assert got == [77, 152063, 0]
+
+
+def sample_rows(ops, logits, params, seeds, draws, histories=None):
+    from turboserve_amd.sampling.sampler import Sampler
+
+    return Sampler(ops).sample(logits.to(DEV), params, seeds, draws, histories)
+
+
+@pytest.mark.parametrize("vocab", [320, 5003])
+def test_sampler_stages_against_plain(ops, vocab):
+    """Every stage alone and combined, row by row against the plain implementation: the chosen
+    token's cumulative interval (64-bit) contains the row's uniform number."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    g = torch.Generator().manual_seed(vocab)
+    settings = [
+        dict(temperature=0.0),
+        dict(temperature=0.0, repetition_penalty=1.7),
+        dict(temperature=0.7),
+        dict(temperature=1.3, top_k=5),
+        dict(temperature=1.0, top_p=0.6),
+        dict(temperature=0.9, top_k=40, top_p=0.8, repetition_penalty=1.3),
+        dict(temperature=1.0, top_k=1),
+        dict(temperature=1e-3),
+    ]
+    rows = len(settings) * 4
+    logits = torch.randn(rows, vocab, generator=g) * 3
+    params = [SamplingParams(logprobs=True, **settings[i % len(settings)]) for i in range(rows)]
+    seeds = [1000 + i * 7919 + (i << 40) for i in range(rows)]
+    draws = [i * 3 for i in range(rows)]
+    histories = [torch.randint(0, vocab, (20,), generator=g).tolist() for _ in range(rows)]
+    out = sample_rows(ops, logits, params, seeds, draws, histories)
+    for i, p in enumerate(params):
+        token = out.token_ids[i]
+        want, cdf = plain.sample_token(
+            logits[i], temperature=p.temperature, seed=seeds[i], draw_index=draws[i], top_k=p.top_k, top_p=p.top_p,
+            penalty=p.repetition_penalty, history=histories[i],
+        )
+        penalised = plain.repetition_penalty(logits[i], histories[i], p.repetition_penalty)
+        assert abs(out.logprobs[i] - plain.log_softmax_at(penalised, token)) < 1e-4, f"row {i} logprob"
+        if p.temperature == 0.0:
+            assert token == want, f"row {i} {settings[i % len(settings)]}"
+            continue
+        u = plain.philox_uniform(seeds[i], draws[i])
+        low = float(cdf[token - 1]) if token > 0 else 0.0
+        high = float(cdf[token])
+        assert high > low, f"row {i}: token {token} has no mass after {settings[i % len(settings)]}"
+        assert low - 1e-5 <= u <= high + 1e-5, f"row {i} {settings[i % len(settings)]}: u={u} not in [{low}, {high}]"
+
+
+def test_sampler_rows_are_independent(ops):
+    """A batch equals its rows one by one, and a row does not depend on its neighbours
+    (tests/unit/test_sampler.py:131-149, 198-215)."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(6, 777, generator=g)
+    params = [SamplingParams(temperature=t, top_k=k) for t, k in ((1.0, 0), (0.0, 0), (0.5, 10), (2.0, 0), (1.0, 3), (0.0, 5))]
+    seeds, draws = [5, 6, 7, 8, 9, 10], [0, 1, 2, 3, 4, 5]
+    batch = sample_rows(ops, logits, params, seeds, draws).token_ids
+    single = [sample_rows(ops, logits[i:i + 1], params[i:i + 1], seeds[i:i + 1], draws[i:i + 1]).token_ids[0] for i in range(6)]
+    assert batch == single
+    assert batch[1] == int(logits[1].argmax()) and batch[5] == int(logits[5].argmax())  # greedy ignores top-k
+
+
+def test_sampler_distribution(ops):
+    """Draws follow the softmax: 4000 counters of one seed against the probabilities."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    logits = torch.tensor([[2.0, 1.0, 0.0, -1.0, 0.5]]).repeat(4000, 1)
+    out = sample_rows(ops, logits, [SamplingParams(temperature=1.0)] * 4000, [42] * 4000, list(range(4000)))
+    counts = torch.bincount(torch.tensor(out.token_ids), minlength=5).float() / 4000
+    probs = torch.softmax(logits[0], -1)
+    assert float((counts - probs).abs().max()) < 0.03
+    top2 = sample_rows(ops, logits[:500], [SamplingParams(temperature=1.0, top_k=2)] * 500, [1] * 500, list(range(500)))
+    assert set(top2.token_ids) == {0, 1}  # the support of top-k (tests/unit/test_sampler.py:121-128)
+
+
+def test_philox_matches_plain(ops):
+    """The kernel's uniform numbers are the plain implementation's: with logits that make the
+    cumulative distribution a ruler, the drawn token reads off u."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    vocab = 4096
+    logits = torch.zeros(64, vocab)
+    seeds = [random.Random(i).getrandbits(64) for i in range(64)]
+    draws = [random.Random(100 + i).getrandbits(31) for i in range(64)]
+    out = sample_rows(ops, logits, [SamplingParams(temperature=1.0)] * 64, seeds, draws)
+    for token, seed, draw in zip(out.token_ids, seeds, draws):
+        assert abs(token - int(plain.philox_uniform(seed, draw) * vocab)) <= 1

@@ -1,8 +1,9 @@
 """Device side of the cache: the page tensors of every group and the state tensors.
 
-Per group one tensor ``[members, 2, num_pages, kv_heads, page_size, head_dim]`` (keys at index
-0, values at 1): a page of one member is ``kv_heads`` contiguous runs of ``page_size *
-head_dim`` elements, which is what the attention kernels stream.  The reference keeps
+Per group one tensor ``[members, 2, num_pages, kv_heads, page_size * head_dim]`` (keys at index
+0, values at 1).  A key page of one head is ``[page_size, head_dim]``; a value page is stored
+transposed, ``[head_dim, page_size]``, so that the attention kernels load eight consecutive
+keys' values of one head dimension at once.  The reference keeps
 ``[num_blocks, block_size, kv_heads, head_dim]`` per layer
 (src/turboserve/engine/core/kv_cache.py:372-400); the slot contract (``page * page_size +
 offset``) is the same.
@@ -36,7 +37,7 @@ class CacheStorage:
         self.dtype = dtype
         self.pages = [
             torch.zeros(
-                (len(group.entries), 2, count, group.num_kv_heads, page_size, group.head_dim),
+                (len(group.entries), 2, count, group.num_kv_heads, page_size * group.head_dim),
                 dtype=dtype,
                 device=device,
             )
@@ -59,8 +60,12 @@ class CacheStorage:
         if unit[0] == "pages":
             _, group, member = unit
             tensor = self.pages[group][member]
+            spec = self.layout.groups[group]
+            pages = tensor.shape[1]
             return PagedKVView(
-                k=tensor[0], v=tensor[1], group=group, block_size=self.page_size,
+                k=tensor[0].view(pages, spec.num_kv_heads, self.page_size, spec.head_dim),
+                v=tensor[1].view(pages, spec.num_kv_heads, spec.head_dim, self.page_size),
+                group=group, block_size=self.page_size,
                 window=self.layout.groups[group].window, writable=writable,
             )
         return FixedStateView(state=self.states[unit[1]], writable=writable)

@@ -5,7 +5,8 @@
 // the keys lo..p of that request, lo = max(0, p - window + 1) for a windowed layer and 0
 // otherwise (src/turboserve/engine/model/attention.py:139-148: keys <= ctx - q_len + j; the
 // window bound is this engine's).  Keys and values are read through the request's block table
-// from pages laid out [NB, Hkv, BS, D]; KV head j serves query heads j*G .. j*G+G-1
+// from key pages [NB, Hkv, BS, D] and transposed value pages [NB, Hkv, D, BS]; KV head j serves
+// query heads j*G .. j*G+G-1
 // (attention.py:196-199).  Online softmax over tiles of 64 keys, as the reference's decode
 // kernel does over blocks (src/turboserve/engine/model/triton_attention.py:127-166).
 //
@@ -27,7 +28,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                int window) {
   __shared__ float qs[ATTN_MAX_DIM];
   __shared__ float ps[ATTN_TILE];
-  __shared__ long long rows[ATTN_TILE];
+  __shared__ long long rows[ATTN_TILE];  // per key of the tile: offset of its value column
 
   const int t = blockIdx.x;
   const int h = blockIdx.y;
@@ -56,8 +57,9 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
     long long row = 0;
     if (valid) {
       const int blk = table[key / block_size];
-      row = ((long long)blk * kv_heads + kvh) * block_size + (key % block_size);
-      const T* krow = k_pages + row * dim;
+      const long long head_base = ((long long)blk * kv_heads + kvh) * block_size * dim;
+      row = head_base + (key % block_size);
+      const T* krow = k_pages + head_base + (long long)(key % block_size) * dim;
       float s = 0.f;
       for (int d = 0; d < dim; ++d) s = fmaf(qs[d], to_float(krow[d]), s);
       score = s;
@@ -77,7 +79,8 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       const int d = lane + c * ATTN_TILE;
       if (d < dim) {
         float a = acc[c] * alpha;
-        for (int j = 0; j < count; ++j) a = fmaf(ps[j], to_float(v_pages[rows[j] * dim + d]), a);
+        for (int j = 0; j < count; ++j)
+          a = fmaf(ps[j], to_float(v_pages[rows[j] + (long long)d * block_size]), a);
         acc[c] = a;
       }
     }

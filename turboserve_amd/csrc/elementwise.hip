@@ -164,7 +164,9 @@ extern "C" int ts_swiglu(void* out, const void* gate_up, int tokens, int inter, 
 // Rotary encoding + cache write.  qkv is [T, (Hq + 2 Hkv) * D]: q heads, then k heads, then v
 // heads.  One block per (token, head).  q and k are rotated in place by the angles of the
 // token's position (cos/sin tables are 32-bit, [capacity, D/2]; pair (i, i + D/2)); k (rotated)
-// and v go to the pages at slot = block * BS + offset, page layout [NB, Hkv, BS, D].
+// and v go to the pages at slot = block * BS + offset.  Key pages are [NB, Hkv, BS, D]; value
+// pages are transposed, [NB, Hkv, D, BS], so that the attention kernels read eight consecutive
+// keys' values of one head dimension with a single 16-byte load.
 // rotate == 0 skips the rotation (a position encoding that only stores).
 // slots == nullptr or a negative slot: nothing is stored for that token.
 // ---------------------------------------------------------------------------------------------
@@ -181,13 +183,17 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, T* __restrict__ k_pages,
   T* row = qkv + (size_t)t * width + (size_t)h * dim;
   const int pos = positions[t];
   const int slot = slots ? slots[t] : -1;
-  T* page = nullptr;
+  T* page = nullptr;   // this token's row of a key page
+  T* vpage = nullptr;  // this token's column of a value page (elements block_size apart)
   if (h >= heads && slot >= 0) {
     const int kvh = (h - heads) % kv_heads;
-    T* pages = (h < heads + kv_heads) ? k_pages : v_pages;
     const size_t blk = (size_t)(slot / block_size);
     const int off = slot % block_size;
-    page = pages + ((blk * kv_heads + kvh) * block_size + off) * (size_t)dim;
+    const size_t head_base = (blk * kv_heads + kvh) * (size_t)block_size * dim;
+    if (h < heads + kv_heads)
+      page = k_pages + head_base + (size_t)off * dim;
+    else
+      vpage = v_pages + head_base + off;
   }
   if (h < heads + kv_heads && rotate) {
     const float* c = cos_table + (size_t)pos * half;
@@ -204,8 +210,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, T* __restrict__ k_pages,
         page[i + half] = o2;
       }
     }
-  } else if (page) {
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) page[i] = row[i];
+  } else if (vpage) {
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) vpage[(size_t)i * block_size] = row[i];
   }
 }
 

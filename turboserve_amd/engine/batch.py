@@ -53,6 +53,13 @@ class StepContext:
     max_query_len: int = 0
     max_context_len: int = 0
     num_logit_rows: int = 0
+    # Requests that bring more than one token come first, single-token (decode) requests last,
+    # so a kernel specialised for either kind gets one contiguous range of requests and rows.
+    num_prefill_seqs: int = 0
+    num_decode_seqs: int = 0
+    num_prefill_tokens: int = 0
+    max_prefill_context_len: int = 0
+    max_decode_context_len: int = 0
 
 
 def validate_entries(entries: Sequence[StepEntry], num_groups: int, page_size: int) -> None:
@@ -92,9 +99,17 @@ def build_context(
     device: torch.device | str,
     check: bool = True,
 ) -> StepContext:
-    """Pack a step's entries, in the order given, into device tensors with one copy."""
+    """Pack a step's entries into device tensors with one copy.
+
+    Rows are ordered with multi-token entries first and single-token entries last (the
+    reference's scheduler emits prefills before decodes, src/turboserve/engine/core/scheduler.py:637;
+    here any order is accepted and arranged).  ``logit_rows`` keeps the order of the entries as
+    given and of each entry's ``want``."""
     if check:
         validate_entries(entries, num_groups, page_size)
+    given = list(entries)
+    entries = [e for e in given if len(e.tokens) > 1] + [e for e in given if len(e.tokens) <= 1]
+    num_prefill_seqs = sum(1 for e in given if len(e.tokens) > 1)
     num_seqs = len(entries)
     query_lens = [len(e.tokens) for e in entries]
     context_lens = [e.start + n for e, n in zip(entries, query_lens)]
@@ -102,7 +117,8 @@ def build_context(
     starts = np.zeros(num_seqs + 1, dtype=np.int32)
     np.cumsum(query_lens, out=starts[1:])
     widths = [max((len(e.tables[g]) for e in entries), default=1) or 1 for g in range(num_groups)]
-    logit_rows = [int(starts[i]) + place for i, e in enumerate(entries) for place in e.want]
+    row_of = {id(e): int(starts[i]) for i, e in enumerate(entries)}
+    logit_rows = [row_of[id(e)] + place for e in given for place in e.want]
 
     pieces: list[np.ndarray] = [
         np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=num_tokens),
@@ -141,4 +157,9 @@ def build_context(
         max_query_len=max(query_lens, default=0),
         max_context_len=max(context_lens, default=0),
         num_logit_rows=len(logit_rows),
+        num_prefill_seqs=num_prefill_seqs,
+        num_decode_seqs=num_seqs - num_prefill_seqs,
+        num_prefill_tokens=int(starts[num_prefill_seqs]),
+        max_prefill_context_len=max(context_lens[:num_prefill_seqs], default=0),
+        max_decode_context_len=max(context_lens[num_prefill_seqs:], default=0),
     )

@@ -8,7 +8,7 @@ library is current.
 
 The sources are grouped into modules, one library each, so that a run only compiles what it
 uses: ``core`` holds the kernels of every run (both dtypes, incl. the whole 32-bit path),
-``bf16`` the matrix-core kernels that only bfloat16 serving needs.
+``attn_d<N>`` the matrix-core attention kernels of bfloat16 serving for head size N.
 """
 
 from __future__ import annotations
@@ -20,6 +20,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from pathlib import Path
 
@@ -37,6 +38,33 @@ MODULES: dict[str, tuple[str, ...]] = {
         "sampling.hip",
     ),
 }
+
+#: Head sizes whose matrix-core attention module ``build_all`` compiles ahead of time: the
+#: common ones and those of the test configurations.  Any other multiple of 16 up to 256 is
+#: compiled when a model with that head size is first loaded.
+PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
+
+
+def attention_module(head_dim: int) -> str:
+    """Name of the bfloat16 matrix-core attention module for one head size."""
+    return f"attn_d{int(head_dim)}"
+
+
+def module_spec(module: str) -> tuple[tuple[str, ...], tuple[str, ...]]:
+    """``(sources, extra compiler flags)`` of a module; ``attn_d<N>`` modules are one source
+    compiled for head size N."""
+    if module in MODULES:
+        return MODULES[module], ()
+    if module.startswith("attn_d") and module[6:].isdigit():
+        head_dim = int(module[6:])
+        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
+            raise BuildError(f"the matrix-core attention kernels take head sizes 16..256 in steps of 16, not {head_dim}")
+        return ("attention_mfma.hip",), (f"-DTS_HEAD_DIM={head_dim}",)
+    raise BuildError(f"unknown kernel module {module!r}")
+
+
+def all_modules() -> list[str]:
+    return [*MODULES, *(attention_module(d) for d in PREBUILT_HEAD_DIMS)]
 
 HIPCC_FLAGS = (
     f"--offload-arch={ARCH}",
@@ -63,10 +91,11 @@ def find_hipcc() -> str:
 
 
 def source_hash(module: str) -> str:
+    sources, extra = module_spec(module)
     digest = hashlib.sha256()
-    digest.update(" ".join(HIPCC_FLAGS).encode())
+    digest.update(" ".join((*HIPCC_FLAGS, *extra)).encode())
     headers = sorted(CSRC.glob("*.hpp"))
-    for path in [*headers, *(CSRC / name for name in MODULES[module])]:
+    for path in [*headers, *(CSRC / name for name in sources)]:
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
     return digest.hexdigest()
@@ -75,7 +104,7 @@ def source_hash(module: str) -> str:
 def _writable(directory: Path) -> bool:
     try:
         directory.mkdir(parents=True, exist_ok=True)
-        probe = directory / f".probe-{os.getpid()}"
+        probe = directory / f".probe-{os.getpid()}-{threading.get_ident()}"
         probe.write_bytes(b"")
         probe.unlink()
         return True
@@ -121,21 +150,20 @@ def _run(cmd: list[str]) -> None:
 
 def build_module(module: str, *, directory: Path | None = None, verbose: bool = True) -> Path:
     """Compile one module from scratch and return the library's path."""
-    if module not in MODULES:
-        raise BuildError(f"unknown kernel module {module!r}; known: {sorted(MODULES)}")
+    source_names, extra_flags = module_spec(module)
     hipcc = find_hipcc()
     out_dir = directory or build_dir()
     out_dir.mkdir(parents=True, exist_ok=True)
     obj_dir = out_dir / f"obj_{module}"
     obj_dir.mkdir(exist_ok=True)
-    sources = [CSRC / name for name in MODULES[module]]
+    sources = [CSRC / name for name in source_names]
     started = time.time()
     if verbose:
         _say(f"compiling module {module!r}: {len(sources)} sources for {ARCH} into {out_dir}")
 
     def compile_one(src: Path) -> Path:
         obj = obj_dir / (src.stem + ".o")
-        _run([hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)])
+        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-I", str(CSRC), "-c", str(src), "-o", str(obj)])
         return obj
 
     objects: list[Path] = []
@@ -172,8 +200,13 @@ def ensure_module(module: str, *, verbose: bool = True) -> Path:
 
 
 def build_all(*, verbose: bool = True) -> list[Path]:
-    """Compile every module, whether or not a built library is there."""
-    return [build_module(module, verbose=verbose) for module in MODULES]
+    """Compile every module, whether or not a built library is there; modules are compiled
+    side by side."""
+    modules = all_modules()
+    directory = build_dir()
+    workers = max(1, min(len(modules), int(os.environ.get("MAX_JOBS", "8")), 16))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=workers) as pool:
+        return list(pool.map(lambda module: build_module(module, directory=directory, verbose=verbose), modules))
 
 
 if __name__ == "__main__":

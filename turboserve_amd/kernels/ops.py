@@ -56,6 +56,14 @@ _SIGNATURES: dict[str, dict[str, list]] = {
     },
 }
 
+def _attention_signatures(head_dim: int) -> dict[str, list]:
+    return {
+        f"ts_attention_decode_d{head_dim}": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+                                             c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                             c_int, c_float, c_int, c_int, c_int, c_void_p],
+    }
+
+
 _LIBRARIES: dict[str, ctypes.CDLL] = {}
 
 
@@ -69,7 +77,10 @@ def load_module(module: str) -> ctypes.CDLL:
         lib = ctypes.CDLL(str(path))
     except OSError as exc:  # pragma: no cover - depends on the machine
         raise KernelError(f"cannot load the kernel library {path}: {exc}") from exc
-    for name, argtypes in _SIGNATURES.get(module, {}).items():
+    signatures = _SIGNATURES.get(module, {})
+    if module.startswith("attn_d"):
+        signatures = _attention_signatures(int(module[6:]))
+    for name, argtypes in signatures.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = c_int
@@ -100,6 +111,16 @@ def _gpu(*tensors: torch.Tensor | None) -> None:
 def _i32(t: torch.Tensor | None, name: str) -> None:
     if t is not None:
         _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+
+
+def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtype) -> None:
+    """Key pages ``[NB, Hkv, BS, D]`` and transposed value pages ``[NB, Hkv, D, BS]``."""
+    _need(k_pages.dim() == 4 and v_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous()
+          and k_pages.dtype == dtype and v_pages.dtype == dtype,
+          "pages must be contiguous 4-d tensors of the queries' dtype")
+    nb, kv_heads, block_size, head_dim = k_pages.shape
+    _need(tuple(v_pages.shape) == (nb, kv_heads, head_dim, block_size),
+          "value pages must be [NB, Hkv, D, BS] for key pages [NB, Hkv, BS, D]")
 
 
 class Ops:
@@ -226,10 +247,8 @@ class Ops:
         if slots is not None:
             _need(slots.numel() == tokens, "one slot per token")
             _need(k_pages is not None and v_pages is not None, "slots given without pages")
-            for pages in (k_pages, v_pages):
-                _need(pages.dim() == 4 and pages.shape[1:] == (kv_heads, block_size, head_dim)
-                      and pages.dtype == qkv.dtype and pages.is_contiguous(),
-                      "pages must be contiguous [NB, Hkv, BS, D] of qkv's dtype")
+            _check_pages(k_pages, v_pages, qkv.dtype)
+            _need(k_pages.shape[1:] == (kv_heads, block_size, head_dim), "pages do not match the heads' geometry")
         _check(self.core.ts_rope_store(_ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(cos), _ptr(sin),
                                        _ptr(positions), _ptr(slots), tokens, heads, kv_heads, head_dim,
                                        block_size, 0 if cos is None else 1, dtype_code(qkv.dtype), self.stream()),
@@ -258,9 +277,7 @@ class Ops:
         _i32(block_table, "block_table")
         _i32(token_seq, "token_seq")
         _i32(positions, "positions")
-        _need(k_pages.dim() == 4 and k_pages.shape == v_pages.shape and k_pages.is_contiguous()
-              and v_pages.is_contiguous() and k_pages.dtype == q.dtype == v_pages.dtype,
-              "pages must be contiguous [NB, Hkv, BS, D] of q's dtype")
+        _check_pages(k_pages, v_pages, q.dtype)
         _, kv_heads, block_size, head_dim = k_pages.shape
         tokens = positions.numel()
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
@@ -275,6 +292,65 @@ class Ops:
             block_size, float(scale), int(window or 0), dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
+
+    @staticmethod
+    def mfma_attention_supported(dtype: torch.dtype, head_dim: int, block_size: int) -> bool:
+        """Whether the matrix-core attention kernels take this geometry (bfloat16, head sizes
+        16..256 in steps of 16, pages of at least 8 tokens); anything else runs the generic
+        kernel."""
+        return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 8
+
+    def attention_decode(
+        self,
+        out: torch.Tensor,
+        q: torch.Tensor,
+        q_stride: int,
+        k_pages: torch.Tensor,
+        v_pages: torch.Tensor,
+        block_table: torch.Tensor,
+        query_start_loc: torch.Tensor,
+        context_lens: torch.Tensor,
+        seq_begin: int,
+        requests: int,
+        heads: int,
+        scale: float,
+        window: int | None,
+        max_context: int,
+    ) -> None:
+        """Matrix-core attention for the single-token requests ``seq_begin .. seq_begin +
+        requests - 1`` of the step; writes their rows of ``out [T, heads * D]``.  ``max_context``
+        (host-known) bounds their context lengths and sizes the split of the keys."""
+        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens)
+        _i32(block_table, "block_table")
+        _i32(query_start_loc, "query_start_loc")
+        _i32(context_lens, "context_lens")
+        _check_pages(k_pages, v_pages, torch.bfloat16)
+        _, kv_heads, block_size, head_dim = k_pages.shape
+        _need(self.mfma_attention_supported(q.dtype, head_dim, block_size), "geometry not taken by the matrix-core kernels")
+        _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[1] == heads * head_dim,
+              "out must be contiguous bfloat16 [T, heads * D]")
+        _need(q.is_contiguous() and q_stride >= heads * head_dim, "q does not hold [T, q_stride] rows")
+        _need(heads % kv_heads == 0 and block_table.dim() == 2, "heads / block table do not fit")
+        _need(seq_begin >= 0 and seq_begin + requests <= context_lens.numel() and requests <= block_table.shape[0],
+              "request range outside the step")
+        _need(max_context <= block_table.shape[1] * block_size, "block table does not cover the context")
+        span = max_context if not window else min(max_context, window + 31)
+        head_tiles = -(-(heads // kv_heads) // 16)
+        pairs = requests * kv_heads * head_tiles
+        splits = max(1, min(-(-self.decode_target_waves // pairs), -(-span // 128)))
+        keys_per_split = -(-(-(-(span + 31) // splits)) // 32) * 32
+        splits = -(-(span + 31) // keys_per_split)
+        partial_acc = torch.empty((requests * heads * splits, head_dim), dtype=torch.float32, device=q.device)
+        partial_ml = torch.empty((requests * heads * splits, 2), dtype=torch.float32, device=q.device)
+        lib = load_module(build.attention_module(head_dim))
+        fn = getattr(lib, f"ts_attention_decode_d{head_dim}")
+        _check(fn(_ptr(out), _ptr(partial_acc), _ptr(partial_ml), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages),
+                  _ptr(block_table), block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), seq_begin,
+                  requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
+                  self.stream()), "ts_attention_decode")
+
+    #: Wavefronts a decode attention launch aims for (8 per compute unit of a 256-CU device).
+    decode_target_waves = 2048
 
     # -- products -----------------------------------------------------------------------------
 

@@ -91,8 +91,26 @@ class GroupedQueryAttention(Mixer):
         ops = self.runtime.ops
         qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_tensor)
         self.position.encode_and_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache)
-        attended = ops.paged_attention_generic(
-            qkv, qkv.shape[1], cache.k, cache.v, ctx.block_tables[cache.group], ctx.token_seq,
-            ctx.positions, self.num_heads, self.scale, self.window,
-        )
+        attended = self.attend(qkv, ctx, cache)
         return ops.linear(attended, self.o_weight, self.o_bias_tensor)
+
+    def attend(self, qkv: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
+        """``[T, Hq D]`` attention output for the step's (encoded) queries in ``qkv``.
+
+        bfloat16 runs use the matrix-core kernels where the geometry allows: one launch for the
+        single-token requests at the end of the batch; everything else (and every 32-bit run)
+        goes through the generic kernel."""
+        ops = self.runtime.ops
+        table = ctx.block_tables[cache.group]
+        fast = ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
+        if fast and ctx.num_prefill_seqs == 0 and ctx.num_decode_seqs > 0:
+            out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
+            ops.attention_decode(
+                out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
+                0, ctx.num_decode_seqs, self.num_heads, self.scale, self.window, ctx.max_decode_context_len,
+            )
+            return out
+        return ops.paged_attention_generic(
+            qkv, qkv.shape[1], cache.k, cache.v, table, ctx.token_seq, ctx.positions,
+            self.num_heads, self.scale, self.window,
+        )

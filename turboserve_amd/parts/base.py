@@ -74,8 +74,8 @@ CacheNeed = PagedKV | FixedState | None
 
 @dataclass
 class PagedKVView:
-    """One cache unit's pages: ``k`` and ``v`` are ``[num_blocks, kv_heads, block_size,
-    head_dim]``; ``group`` indexes the step's per-group block tables and slot mappings;
+    """One cache unit's pages: ``k`` is ``[num_blocks, kv_heads, block_size, head_dim]``, ``v`` is
+    stored transposed, ``[num_blocks, kv_heads, head_dim, block_size]``; ``group`` indexes the step's per-group block tables and slot mappings;
     ``writable`` is false when the layer reads another layer's cache."""
 
     k: torch.Tensor

@@ -276,6 +276,39 @@ def test_attention_decode_mfma_far_key_and_subrange(ops):
     assert float(case.expected[1].abs().mean()) > 4.0  # the spike's value dominates
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_GEOMETRIES)
+@pytest.mark.parametrize("window", [None, 20, 300])
+def test_attention_prefill_mfma(ops, heads, kv_heads, dim, page, window):
+    """Whole prompts, portions that continue a cached prefix, two-token portions; block edges at
+    every alignment against pages and 32-key windows."""
+    seqs = [(70, 70), (33, 2), (600, 77), (129, 16), (257, 17), (48, 48), (2, 2), (515, 33)]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, window, seed=dim + 2)
+    blocks = [(s, case.qsl[s] + off) for s, (_, qlen) in enumerate(seqs) for off in range(0, qlen, 16)]
+    random.Random(3).shuffle(blocks)
+    out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, window,
+        max(c for c, _ in seqs),
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+
+
+def test_attention_prefill_mfma_far_key(ops):
+    heads, kv_heads, dim, page = 28, 4, 128, 16
+    seqs = [(3000, 40), (2100, 2100)]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, None, seed=11, spike=77)
+    blocks = [(s, case.qsl[s] + off) for s, (_, qlen) in enumerate(seqs) for off in range(0, qlen, 16)]
+    out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, None, 3000,
+    )
+    got = out.float().cpu()
+    torch.testing.assert_close(got, case.expected, **tol(torch.bfloat16))
+    assert float(case.expected[:40].abs().mean()) > 4.0
+
+
 # -- sampling ---------------------------------------------------------------------------------------
 
 

@@ -30,6 +30,11 @@
 #endif
 static_assert(TS_HEAD_DIM % 16 == 0 && TS_HEAD_DIM >= 16 && TS_HEAD_DIM <= 256, "head size: 16..256 in steps of 16");
 
+// Query heads of one KV head that share each loaded window in the prefill kernel.
+#ifndef TS_PREFILL_HEADS
+#define TS_PREFILL_HEADS 2
+#endif
+
 #define TS_CAT2(a, b) a##b
 #define TS_CAT(a, b) TS_CAT2(a, b)
 #define TS_SYM(name) TS_CAT(name, TS_HEAD_DIM)
@@ -39,9 +44,10 @@ namespace {
 constexpr int D = TS_HEAD_DIM;
 constexpr int NT = D / 16;        // 16-wide tiles of the head dimension (second product)
 constexpr int KJ = D / 32;        // 32-deep steps of the first product
-constexpr bool KTAIL = (D % 32) != 0;  // one more 16-deep step
+constexpr bool KTAIL = (D % 32) != 0;  // one more step whose upper 16 of 32 are zero
 constexpr int WINDOW_KEYS = 32;   // keys per iteration
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr int DECODE_MAX_SPLITS = 256;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -49,56 +55,30 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-union Frag8 {
-  bf16x8 v;
-  u32x4 u;
-  uint16_t h[8];
-};
-union Frag4 {
-  s16x4 v;
-  u32x2 u;
-  uint16_t h[4];
-};
+// Matrix-core operands are kept as raw 32-bit words (two bfloat16 each) and reinterpreted with
+// __builtin_bit_cast where an instruction wants its own vector type; no unions, no aliasing.
+typedef u32x4 Frag8;  // 8 bfloat16
+typedef u32x2 Frag4;  // 4 bfloat16
 
-__device__ __forceinline__ uint16_t bf16_bits(float v) { return from_float<bf16_t>(v).bits; }
+__device__ __forceinline__ uint32_t bf16_bits(float v) { return from_float<bf16_t>(v).bits; }
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) { return bf16_bits(lo) | (bf16_bits(hi) << 16); }
+__device__ __forceinline__ bf16x8 as_bf16x8(Frag8 f) { return __builtin_bit_cast(bf16x8, f); }
+__device__ __forceinline__ Frag8 load8(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 
 // The queries of 16 columns as B operands of the first product: lane l holds, for column
-// l % 16, the head dimensions 32 j + 8 (l / 16) .. + 7.
+// l % 16, the head dimensions 32 j + 8 (l / 16) .. + 7.  Only v_mfma_f32_16x16x32_bf16 is
+// used: a 16-deep remainder of the head size is padded with zeros to 32 (feeding one accumulator
+// from this instruction and then from the 16-deep one, back to back, gave wrong sums in testing
+// on gfx950).
 struct QueryFrags {
   Frag8 main[KJ > 0 ? KJ : 1];
-  Frag4 tail;
+  Frag8 tail;  // head sizes that are no multiple of 32: the last 16 dimensions, upper half zero
 };
 
 __device__ __forceinline__ void load_query(QueryFrags& q, const uint16_t* row, int group) {
 #pragma unroll
-  for (int j = 0; j < KJ; ++j) {
-    if (row) q.main[j].u = *reinterpret_cast<const u32x4*>(row + 32 * j + 8 * group);
-    else q.main[j].u = u32x4{0u, 0u, 0u, 0u};
-  }
-  if (KTAIL) {
-    if (row) q.tail.u = *reinterpret_cast<const u32x2*>(row + 32 * KJ + 4 * group);
-    else q.tail.u = u32x2{0u, 0u};
-  }
-}
-
-// One 16-key score tile: S^T[m][col] = sum_d K[key(m)][d] Q[col][d].  `krow` is this lane's key
-// row (row m = lane % 16 of the tile) or null when that key is outside the request's range.
-__device__ __forceinline__ f32x4 score_tile(const uint16_t* krow, const QueryFrags& q, int group) {
-  f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int j = 0; j < KJ; ++j) {
-    Frag8 a;
-    if (krow) a.u = *reinterpret_cast<const u32x4*>(krow + 32 * j + 8 * group);
-    else a.u = u32x4{0u, 0u, 0u, 0u};
-    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, q.main[j].v, s, 0, 0, 0);
-  }
-  if (KTAIL) {
-    Frag4 a;
-    if (krow) a.u = *reinterpret_cast<const u32x2*>(krow + 32 * KJ + 4 * group);
-    else a.u = u32x2{0u, 0u};
-    s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, q.tail.v, s, 0, 0, 0);
-  }
-  return s;
+  for (int j = 0; j < KJ; ++j) q.main[j] = row ? load8(row + 32 * j + 8 * group) : Frag8{0u, 0u, 0u, 0u};
+  if (KTAIL) q.tail = (row && group < 2) ? load8(row + 32 * KJ + 8 * group) : Frag8{0u, 0u, 0u, 0u};
 }
 
 struct PageGeometry {
@@ -124,7 +104,66 @@ __device__ __forceinline__ const uint16_t* value_chunk(const PageGeometry& g, in
   return g.v_pages + ((blk * g.kv_heads + g.kvh) << g.block_shift) * D + (key & g.block_mask);
 }
 
-// Online-softmax state of the lane's column, and the window update shared by both kernels.
+// Everything one 32-key window contributes, as matrix-core operands: the lane's two key rows
+// (A operands of the score tiles) and its 8-key value chunk for every head-dimension tile.
+struct WindowFrags {
+  Frag8 k[2][KJ > 0 ? KJ : 1];
+  Frag8 ktail[2];
+  Frag8 v[NT];
+};
+
+// Issue the loads of window `w`.  A key or chunk outside lo..last is redirected to `safe_key`
+// (a key of the request that is certainly in a live page): the loads stay unconditional, so
+// they can be issued a whole window ahead; what they bring is masked in the softmax.
+__device__ __forceinline__ void load_window(WindowFrags& f, const PageGeometry& g, int w, int lo, int last,
+                                            int safe_key, int lane16, int group) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = w + 8 * (lane16 >> 2) + 4 * t + (lane16 & 3);
+    const uint16_t* row = key_row(g, (key >= lo && key <= last) ? key : safe_key);
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) f.k[t][j] = load8(row + 32 * j + 8 * group);
+    if (KTAIL) f.ktail[t] = group < 2 ? load8(row + 32 * KJ + 8 * group) : Frag8{0u, 0u, 0u, 0u};
+  }
+  const int chunk = w + 8 * group;
+  const uint16_t* vp = value_chunk(g, (chunk + 7 >= lo && chunk <= last) ? chunk : (safe_key & ~7));
+#pragma unroll
+  for (int n = 0; n < NT; ++n)
+    f.v[n] = load8(vp + ((long long)(16 * n + lane16) << g.block_shift));
+}
+
+// Values of keys beyond `last` are whatever an earlier owner of the page left: clear them, so
+// that a stale non-finite value cannot meet a zero probability.  Needed only for a window that
+// is not wholly inside lo..last.
+__device__ __forceinline__ void clear_stale_values(WindowFrags& f, int w, int lo, int last, int group) {
+  const int chunk = w + 8 * group;
+  const bool live = chunk + 7 >= lo && chunk <= last;
+  // Word i of a fragment holds keys chunk + 2 i (low half) and chunk + 2 i + 1 (high half).
+  uint32_t keep[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t low = (live && chunk + 2 * i <= last) ? 0x0000ffffu : 0u;
+    const uint32_t high = (live && chunk + 2 * i + 1 <= last) ? 0xffff0000u : 0u;
+    keep[i] = low | high;
+  }
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.v[n][i] &= keep[i];
+  }
+}
+
+// S^T tile t of the window for the 16 columns whose queries are in `q`.
+__device__ __forceinline__ f32x4 score_tile(const WindowFrags& f, int t, const QueryFrags& q) {
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < KJ; ++j)
+    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(f.k[t][j]), as_bf16x8(q.main[j]), s, 0, 0, 0);
+  if (KTAIL) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(f.ktail[t]), as_bf16x8(q.tail), s, 0, 0, 0);
+  return s;
+}
+
+// Online-softmax state of the lane's column.
 struct ColumnState {
   float m;  // running maximum of the scaled scores (log2 domain)
   float l;  // this lane's share of the running sum (summed over lane groups at the end)
@@ -138,64 +177,49 @@ __device__ __forceinline__ void init_state(ColumnState& st) {
   for (int n = 0; n < NT; ++n) st.acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-// s0 / s1: raw scores of tiles 0 and 1 (lane: column l % 16, keys window + 8 g + 4 t + i).
-// `first_valid` .. `last_valid` (inclusive) bound the keys this column may see.
-// Returns the probabilities as the B operand of the second product.
-__device__ __forceinline__ Frag8 softmax_window(ColumnState& st, f32x4 s0, f32x4 s1, int window_start,
-                                                int group, int first_valid, int last_valid,
-                                                float scale_log2) {
+// One window for one set of 16 columns: scores, masked online softmax, O^T += V^T P^T.
+// The lane's column sees the keys first_valid..last_valid (inclusive).
+__device__ __forceinline__ void attend_window(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w,
+                                              int group, int first_valid, int last_valid, float scale_log2) {
+  const f32x4 s0 = score_tile(f, 0, q);
+  const f32x4 s1 = score_tile(f, 1, q);
   float s[8];
   float mx = -INFINITY;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int key = window_start + 8 * group + e;  // e = 4 t + i
-    const float raw = (e < 4 ? s0[e] : s1[e - 4]) * scale_log2;
+    const int key = w + 8 * group + e;  // e = 4 t + i: row 4 g + i of tile t
+    const float raw = (e < 4 ? s0[e & 3] : s1[e & 3]) * scale_log2;
     s[e] = (key >= first_valid && key <= last_valid) ? raw : -INFINITY;
     mx = fmaxf(mx, s[e]);
   }
   mx = fmaxf(mx, __shfl_xor(mx, 16, TS_WAVE));
   mx = fmaxf(mx, __shfl_xor(mx, 32, TS_WAVE));
   const float m_new = fmaxf(st.m, mx);
-  Frag8 p;
-  if (m_new == -INFINITY) {  // nothing visible to this column so far
-    p.u = u32x4{0u, 0u, 0u, 0u};
-    return p;
-  }
-  const float alpha = exp2f(st.m - m_new);  // 0 when st.m is -inf
+  // Nothing visible to this column so far: keep the state, contribute zeros.
+  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+  const float alpha = exp2f(st.m - m_use);  // 0 when st.m is -inf
+  float pe[8];
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float pe = exp2f(s[e] - m_new);  // 0 for masked keys
-    sum += pe;
-    p.h[e] = bf16_bits(pe);
+    pe[e] = exp2f(s[e] - m_use);  // 0 for masked keys
+    sum += pe[e];
   }
+  const Frag8 p = {pack2(pe[0], pe[1]), pack2(pe[2], pe[3]), pack2(pe[4], pe[5]), pack2(pe[6], pe[7])};
   st.l = st.l * alpha + sum;
   st.m = m_new;
 #pragma unroll
-  for (int n = 0; n < NT; ++n) st.acc[n] *= alpha;
-  return p;
+  for (int n = 0; n < NT; ++n) {
+    st.acc[n] *= alpha;
+    st.acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(f.v[n]), as_bf16x8(p), st.acc[n], 0, 0, 0);
+  }
 }
 
-// O^T += V^T P^T for one window.  `vchunk` points at the lane group's 8 keys (dimension 0) or is
-// null when the chunk lies wholly outside the request's range; `keep` masks keys of the chunk
-// that lie beyond the context (their page bytes are stale).
-__device__ __forceinline__ void accumulate_window(ColumnState& st, const uint16_t* vchunk, const Frag8& p,
-                                                  int lane16, int block_shift, unsigned keep) {
-#pragma unroll
-  for (int n = 0; n < NT; ++n) {
-    Frag8 a;
-    if (vchunk) {
-      a.u = *reinterpret_cast<const u32x4*>(vchunk + ((long long)(16 * n + lane16) << block_shift));
-      if (keep != 0xffu) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (!((keep >> e) & 1u)) a.h[e] = 0;
-      }
-    } else {
-      a.u = u32x4{0u, 0u, 0u, 0u};
-    }
-    st.acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, st.acc[n], 0, 0, 0);
-  }
+// Sum of the lane's column over the four lane groups.
+__device__ __forceinline__ float column_sum(float l) {
+  l += __shfl_xor(l, 16, TS_WAVE);
+  l += __shfl_xor(l, 32, TS_WAVE);
+  return l;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -229,34 +253,36 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
 
   PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, kv_heads, kvh, block_shift,
                    (1 << block_shift) - 1};
-  QueryFrags qf;
-  load_query(qf, head_valid ? q + (size_t)token * q_stride + (size_t)head * D : nullptr, group);
   ColumnState st;
   init_state(st);
 
-  for (int w = begin; w < end; w += WINDOW_KEYS) {
-    const int row_key = w + 8 * (lane16 >> 2) + (lane16 & 3);
-    const int key0 = row_key, key1 = row_key + 4;
-    const f32x4 s0 = score_tile((key0 >= lo && key0 < ctx) ? key_row(geo, key0) : nullptr, qf, group);
-    const f32x4 s1 = score_tile((key1 >= lo && key1 < ctx) ? key_row(geo, key1) : nullptr, qf, group);
-    const Frag8 pr = softmax_window(st, s0, s1, w, group, lo, p, scale_log2);
-    const int chunk = w + 8 * group;
-    const bool chunk_live = chunk + 8 > lo && chunk < ctx;
-    unsigned keep = 0xffu;
-    if (chunk + 8 > ctx) keep = (chunk < ctx) ? ((1u << (ctx - chunk)) - 1u) : 0u;
-    accumulate_window(st, chunk_live ? value_chunk(geo, chunk) : nullptr, pr, lane16, block_shift, keep);
+  if (begin < end) {
+    QueryFrags qf;
+    load_query(qf, head_valid ? q + (size_t)token * q_stride + (size_t)head * D : nullptr, group);
+    WindowFrags fa, fb;
+    load_window(fa, geo, begin, lo, p, p, lane16, group);
+    int w = begin;
+    while (true) {
+      if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo, p, p, lane16, group);
+      if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fa, w, lo, p, group);
+      attend_window(st, fa, qf, w, group, lo, p, scale_log2);
+      w += WINDOW_KEYS;
+      if (w >= end) break;
+      if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo, p, p, lane16, group);
+      if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fb, w, lo, p, group);
+      attend_window(st, fb, qf, w, group, lo, p, scale_log2);
+      w += WINDOW_KEYS;
+      if (w >= end) break;
+    }
   }
 
-  // The lane's column sum lives in four lane groups.
-  float l_total = st.l + __shfl_xor(st.l, 16, TS_WAVE);
-  l_total += __shfl_xor(l_total, 32, TS_WAVE);
+  const float l_total = column_sum(st.l);
   if (head_valid) {
     const size_t slot = ((size_t)blockIdx.z * heads + head) * splits + split;
     float* acc_out = partial_acc + slot * D;
 #pragma unroll
     for (int n = 0; n < NT; ++n)
-      *reinterpret_cast<float4*>(acc_out + 16 * n + 4 * group) =
-          make_float4(st.acc[n][0], st.acc[n][1], st.acc[n][2], st.acc[n][3]);
+      *reinterpret_cast<f32x4*>(acc_out + 16 * n + 4 * group) = st.acc[n];
     if (group == 0) {
       partial_ml[slot * 2] = st.m;
       partial_ml[slot * 2 + 1] = l_total;
@@ -265,27 +291,118 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
 }
 
 // Combine the splits of one (request, head): out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
-// grid (requests, heads), D threads.
-__global__ void decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_acc,
-                                     const float* __restrict__ partial_ml,
-                                     const int* __restrict__ query_start_loc, int seq_begin, int heads,
-                                     int splits) {
+// grid (requests, heads), one wavefront: lanes first share the splits (weights), then the head
+// dimensions.
+__global__ void __launch_bounds__(64)
+decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_acc,
+                     const float* __restrict__ partial_ml, const int* __restrict__ query_start_loc,
+                     int seq_begin, int heads, int splits) {
+  __shared__ float weights[DECODE_MAX_SPLITS];
   const int seq = seq_begin + blockIdx.x;
   const int head = blockIdx.y;
-  const int d = threadIdx.x;
+  const int lane = threadIdx.x;
   const size_t base = ((size_t)blockIdx.x * heads + head) * splits;
   float m_max = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_max = fmaxf(m_max, partial_ml[(base + s) * 2]);
-  float num = 0.f, den = 0.f;
-  for (int s = 0; s < splits; ++s) {
+  for (int s = lane; s < splits; s += TS_WAVE) m_max = fmaxf(m_max, partial_ml[(base + s) * 2]);
+  m_max = wave_max(m_max);
+  float den = 0.f;
+  for (int s = lane; s < splits; s += TS_WAVE) {
     const float m = partial_ml[(base + s) * 2];
-    if (m == -INFINITY) continue;  // a split past the end of this request's keys
-    const float w = exp2f(m - m_max);
-    den += partial_ml[(base + s) * 2 + 1] * w;
-    num += partial_acc[(base + s) * D + d] * w;
+    const float wgt = (m == -INFINITY) ? 0.f : exp2f(m - m_max);  // a split past the request's keys
+    weights[s] = wgt;
+    den += partial_ml[(base + s) * 2 + 1] * wgt;
   }
+  den = wave_sum(den);
+  __syncthreads();
   const int token = query_start_loc[seq];
-  out[((size_t)token * heads + head) * D + d] = bf16_bits(num / den);
+  uint16_t* orow = out + ((size_t)token * heads + head) * D;
+  const float inv = 1.f / den;
+  for (int d = lane; d < D; d += TS_WAVE) {
+    float num = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) num = fmaf(partial_acc[(base + s) * D + d], weights[s], num);
+    orow[d] = (uint16_t)bf16_bits(num * inv);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// prefill: grid (query blocks, kv_heads * head_chunks); one wavefront handles 16 consecutive
+// tokens of one request's portion for up to CT query heads of one KV head.
+// blocks [n, 2]: (request index in the step, first row of the block in the step).
+// ---------------------------------------------------------------------------------------------
+template <int CT>
+__global__ void __launch_bounds__(64)
+prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
+               const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
+               const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
+               const int* __restrict__ context_lens, const int* __restrict__ blocks, int heads, int kv_heads,
+               int block_shift, float scale_log2, int window) {
+  const int lane = threadIdx.x;
+  const int lane16 = lane & 15;
+  const int group = lane >> 4;
+  const int gsize = heads / kv_heads;
+  const int head_chunks = (gsize + CT - 1) / CT;
+  const int kvh = blockIdx.y / head_chunks;
+  const int first_head = (blockIdx.y % head_chunks) * CT;  // within the KV head's group
+  const int seq = blocks[2 * blockIdx.x];
+  const int row0 = blocks[2 * blockIdx.x + 1];
+  const int row_end = query_start_loc[seq + 1];
+  const int ctx = context_lens[seq];
+  const int pos0 = ctx - (row_end - query_start_loc[seq]) + (row0 - query_start_loc[seq]);  // position of row0
+  const int cols = min(16, row_end - row0);
+  const bool col_valid = lane16 < cols;
+  // An invalid column sees nothing (empty range): its state stays empty and it is never stored.
+  const int p_col = col_valid ? pos0 + lane16 : -1;
+  const int lo_col = (window > 0 && p_col - window + 1 > 0) ? p_col - window + 1 : 0;
+  const int p_last = pos0 + cols - 1;
+  const int lo_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int begin = lo_first & ~(WINDOW_KEYS - 1);
+  const int end = p_last + 1;
+
+  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, kv_heads, kvh, block_shift,
+                   (1 << block_shift) - 1};
+  QueryFrags qf[CT];
+  ColumnState st[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int hg = first_head + c;
+    const bool live = col_valid && hg < gsize;
+    load_query(qf[c], live ? q + (size_t)(row0 + lane16) * q_stride + (size_t)(kvh * gsize + hg) * D : nullptr, group);
+    init_state(st[c]);
+  }
+
+  WindowFrags fa, fb;
+  load_window(fa, geo, begin, lo_first, p_last, p_last, lane16, group);
+  int w = begin;
+  while (true) {
+    if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo_first, p_last, p_last, lane16, group);
+    if (w < lo_first || w + WINDOW_KEYS > end) clear_stale_values(fa, w, lo_first, p_last, group);
+#pragma unroll
+    for (int c = 0; c < CT; ++c) attend_window(st[c], fa, qf[c], w, group, lo_col, p_col, scale_log2);
+    w += WINDOW_KEYS;
+    if (w >= end) break;
+    if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo_first, p_last, p_last, lane16, group);
+    if (w < lo_first || w + WINDOW_KEYS > end) clear_stale_values(fb, w, lo_first, p_last, group);
+#pragma unroll
+    for (int c = 0; c < CT; ++c) attend_window(st[c], fb, qf[c], w, group, lo_col, p_col, scale_log2);
+    w += WINDOW_KEYS;
+    if (w >= end) break;
+  }
+
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int hg = first_head + c;
+    const float l_total = column_sum(st[c].l);
+    if (col_valid && hg < gsize) {
+      const float inv = 1.f / l_total;
+      uint16_t* orow = out + ((size_t)(row0 + lane16) * heads + kvh * gsize + hg) * D;
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const f32x4 a = st[c].acc[n] * inv;
+        *reinterpret_cast<u32x2*>(orow + 16 * n + 4 * group) = Frag4{pack2(a[0], a[1]), pack2(a[2], a[3])};
+      }
+    }
+  }
 }
 
 }  // namespace
@@ -304,7 +421,8 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
     return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0) return TS_ERR_SHAPE;
   if (block_size < 8 || (block_size & (block_size - 1))) return TS_ERR_SHAPE;
-  if (keys_per_split < WINDOW_KEYS || keys_per_split % WINDOW_KEYS != 0 || splits < 1) return TS_ERR_SHAPE;
+  if (keys_per_split < WINDOW_KEYS || keys_per_split % WINDOW_KEYS != 0 || splits < 1 || splits > DECODE_MAX_SPLITS)
+    return TS_ERR_SHAPE;
   if (requests > 65535) return TS_ERR_SHAPE;
   int shift = 0;
   while ((1 << shift) < block_size) ++shift;
@@ -316,8 +434,33 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
                      block_table, table_width, query_start_loc, context_lens, seq_begin, heads, kv_heads,
                      shift, scale * LOG2E, window, keys_per_split, splits);
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
-  hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(D), 0, stream, (uint16_t*)out,
+  hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(64), 0, stream, (uint16_t*)out,
                      (const float*)partial_acc, (const float*)partial_ml, query_start_loc, seq_begin, heads,
                      splits);
+  return ts_launch_status();
+}
+
+// Prefill attention for `num_blocks` blocks of 16 consecutive rows; blocks [num_blocks, 2] holds
+// (request index, first row) of each, rows being token rows of the step.  Writes the rows of
+// `out [T, heads * D]` the blocks cover.
+extern "C" int TS_SYM(ts_attention_prefill_d)(
+    void* out, const void* q, long q_stride, const void* k_pages, const void* v_pages, const int* block_table,
+    int table_width, const int* query_start_loc, const int* context_lens, const int* blocks, int num_blocks,
+    int heads, int kv_heads, int block_size, float scale, int window, hipStream_t stream) {
+  if (num_blocks == 0) return TS_OK;
+  if (!out || !q || !k_pages || !v_pages || !block_table || !query_start_loc || !context_lens || !blocks)
+    return TS_ERR_ARG;
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0) return TS_ERR_SHAPE;
+  if (block_size < 8 || (block_size & (block_size - 1))) return TS_ERR_SHAPE;
+  int shift = 0;
+  while ((1 << shift) < block_size) ++shift;
+  const int gsize = heads / kv_heads;
+  constexpr int CT = TS_PREFILL_HEADS;
+  const int head_chunks = (gsize + CT - 1) / CT;
+  if (kv_heads * head_chunks > 65535) return TS_ERR_SHAPE;
+  dim3 grid(num_blocks, kv_heads * head_chunks);
+  hipLaunchKernelGGL(prefill_kernel<CT>, grid, dim3(64), 0, stream, (uint16_t*)out, (const uint16_t*)q, q_stride,
+                     (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table, table_width,
+                     query_start_loc, context_lens, blocks, heads, kv_heads, shift, scale * LOG2E, window);
   return ts_launch_status();
 }

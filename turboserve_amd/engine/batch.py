@@ -19,6 +19,10 @@ import torch
 from turboserve_amd.cache.manager import PAD_PAGE
 
 
+#: Rows of one request that the prefill attention kernel handles per wavefront.
+PREFILL_BLOCK_ROWS = 16
+
+
 @dataclass
 class StepEntry:
     """One request's share of a step."""
@@ -47,6 +51,7 @@ class StepContext:
     logit_rows: torch.Tensor  # [n] rows whose logits are wanted
     slot_mapping: list[torch.Tensor]  # per group [T]
     block_tables: list[torch.Tensor]  # per group [S, MB], PAD_PAGE beyond a request's pages
+    prefill_blocks: torch.Tensor  # [n, 2]: (request index, first row) of every 16 rows of multi-token requests
     # host copies
     query_lens: list[int] = field(default_factory=list)
     context_lens_host: list[int] = field(default_factory=list)
@@ -120,6 +125,16 @@ def build_context(
     row_of = {id(e): int(starts[i]) for i, e in enumerate(entries)}
     logit_rows = [row_of[id(e)] + place for e in given for place in e.want]
 
+    # 16-row blocks of the multi-token requests, those that see the most keys first, so the
+    # long ones start early and the short ones fill the tail of the launch.
+    blocks = [
+        (context_lens[i] - query_lens[i] + min(offset + PREFILL_BLOCK_ROWS, query_lens[i]), i, int(starts[i]) + offset)
+        for i in range(num_prefill_seqs)
+        for offset in range(0, query_lens[i], PREFILL_BLOCK_ROWS)
+    ]
+    blocks.sort(key=lambda b: -b[0])
+    block_array = np.asarray([[b[1], b[2]] for b in blocks], dtype=np.int32).reshape(-1)
+
     pieces: list[np.ndarray] = [
         np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=num_tokens),
         np.concatenate([np.arange(e.start, e.start + n, dtype=np.int32) for e, n in zip(entries, query_lens)])
@@ -129,6 +144,7 @@ def build_context(
         np.asarray(context_lens, dtype=np.int32),
         np.asarray([e.state_slot for e in entries], dtype=np.int32),
         np.asarray(logit_rows, dtype=np.int32),
+        block_array,
     ]
     for g in range(num_groups):
         pieces.append(np.fromiter((s for e in entries for s in e.slots[g]), dtype=np.int32, count=num_tokens))
@@ -150,8 +166,9 @@ def build_context(
         context_lens=views[4],
         state_slots=views[5],
         logit_rows=views[6],
-        slot_mapping=[views[7 + 2 * g] for g in range(num_groups)],
-        block_tables=[views[8 + 2 * g].view(num_seqs, widths[g]) for g in range(num_groups)],
+        prefill_blocks=views[7].view(-1, 2),
+        slot_mapping=[views[8 + 2 * g] for g in range(num_groups)],
+        block_tables=[views[9 + 2 * g].view(num_seqs, widths[g]) for g in range(num_groups)],
         query_lens=query_lens,
         context_lens_host=context_lens,
         max_query_len=max(query_lens, default=0),

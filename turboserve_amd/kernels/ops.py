@@ -61,6 +61,9 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
         f"ts_attention_decode_d{head_dim}": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
                                              c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                              c_int, c_float, c_int, c_int, c_int, c_void_p],
+        f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
+                                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float,
+                                              c_int, c_void_p],
     }
 
 
@@ -337,7 +340,7 @@ class Ops:
         span = max_context if not window else min(max_context, window + 31)
         head_tiles = -(-(heads // kv_heads) // 16)
         pairs = requests * kv_heads * head_tiles
-        splits = max(1, min(-(-self.decode_target_waves // pairs), -(-span // 128)))
+        splits = max(1, min(-(-self.decode_target_waves // pairs), -(-span // self.decode_min_keys), 256))
         keys_per_split = -(-(-(-(span + 31) // splits)) // 32) * 32
         splits = -(-(span + 31) // keys_per_split)
         partial_acc = torch.empty((requests * heads * splits, head_dim), dtype=torch.float32, device=q.device)
@@ -349,8 +352,50 @@ class Ops:
                   requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
                   self.stream()), "ts_attention_decode")
 
-    #: Wavefronts a decode attention launch aims for (8 per compute unit of a 256-CU device).
-    decode_target_waves = 2048
+    def attention_prefill(
+        self,
+        out: torch.Tensor,
+        q: torch.Tensor,
+        q_stride: int,
+        k_pages: torch.Tensor,
+        v_pages: torch.Tensor,
+        block_table: torch.Tensor,
+        query_start_loc: torch.Tensor,
+        context_lens: torch.Tensor,
+        blocks: torch.Tensor,
+        heads: int,
+        scale: float,
+        window: int | None,
+        max_context: int,
+    ) -> None:
+        """Matrix-core attention for blocks of 16 consecutive rows of multi-token requests:
+        ``blocks [n, 2]`` holds (request index, first row) of each; writes those rows of
+        ``out [T, heads * D]``."""
+        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens, blocks)
+        _i32(block_table, "block_table")
+        _i32(query_start_loc, "query_start_loc")
+        _i32(context_lens, "context_lens")
+        _i32(blocks, "blocks")
+        _check_pages(k_pages, v_pages, torch.bfloat16)
+        _, kv_heads, block_size, head_dim = k_pages.shape
+        _need(self.mfma_attention_supported(q.dtype, head_dim, block_size), "geometry not taken by the matrix-core kernels")
+        _need(out.dtype == torch.bfloat16 and out.is_contiguous() and out.shape[1] == heads * head_dim,
+              "out must be contiguous bfloat16 [T, heads * D]")
+        _need(q.is_contiguous() and q_stride >= heads * head_dim, "q does not hold [T, q_stride] rows")
+        _need(heads % kv_heads == 0 and block_table.dim() == 2, "heads / block table do not fit")
+        _need(blocks.dim() == 2 and blocks.shape[1] == 2, "blocks must be [n, 2]")
+        _need(max_context <= block_table.shape[1] * block_size, "block table does not cover the context")
+        lib = load_module(build.attention_module(head_dim))
+        fn = getattr(lib, f"ts_attention_prefill_d{head_dim}")
+        _check(fn(_ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                  block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), _ptr(blocks), blocks.shape[0],
+                  heads, kv_heads, block_size, float(scale), int(window or 0), self.stream()),
+               "ts_attention_prefill")
+
+    #: Wavefronts a decode attention launch aims for (one per SIMD of a 256-CU device; each keeps two windows of loads in flight).
+    decode_target_waves = 1024
+    #: Fewest keys worth a wavefront of its own.
+    decode_min_keys = 128
 
     # -- products -----------------------------------------------------------------------------
 

@@ -98,17 +98,24 @@ class GroupedQueryAttention(Mixer):
         """``[T, Hq D]`` attention output for the step's (encoded) queries in ``qkv``.
 
         bfloat16 runs use the matrix-core kernels where the geometry allows: one launch for the
-        single-token requests at the end of the batch; everything else (and every 32-bit run)
-        goes through the generic kernel."""
+        multi-token requests at the front of the batch, one for the single-token requests
+        behind them; every 32-bit run and any other geometry goes through the generic kernel."""
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
         fast = ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
-        if fast and ctx.num_prefill_seqs == 0 and ctx.num_decode_seqs > 0:
+        if fast:
             out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
-            ops.attention_decode(
-                out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
-                0, ctx.num_decode_seqs, self.num_heads, self.scale, self.window, ctx.max_decode_context_len,
-            )
+            if ctx.num_prefill_seqs > 0:
+                ops.attention_prefill(
+                    out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
+                    ctx.prefill_blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len,
+                )
+            if ctx.num_decode_seqs > 0:
+                ops.attention_decode(
+                    out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
+                    ctx.num_prefill_seqs, ctx.num_decode_seqs, self.num_heads, self.scale, self.window,
+                    ctx.max_decode_context_len,
+                )
             return out
         return ops.paged_attention_generic(
             qkv, qkv.shape[1], cache.k, cache.v, table, ctx.token_seq, ctx.positions,

@@ -57,6 +57,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     return p.parse_args()
 
 
@@ -207,6 +208,11 @@ def main() -> int:
         seconds = bench.run(steps, warmup)
         bench.close()
         return batch * steps / seconds, seconds / steps
+
+    if args.only_prefill:
+        seconds = run_prefill(model, config, PREFILL_TOKENS)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}))
+        return 0
 
     value, step_seconds = decode_rate(args.batch, args.steps, args.warmup)
     mean_context = args.context + args.warmup + args.steps / 2

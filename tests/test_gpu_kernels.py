@@ -116,6 +116,82 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
     assert torch.equal(full[40:41], one)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(7, 8), (130, 104), (320, 96), (3584, 1000), (301, 2056), (4608, 3584)])
+def test_gemm_skinny(ops, m, n, k):
+    """The decode-sized product: 32-bit partial sums over ranges of K whose sum is the product,
+    for row counts around the 16-row tiles, N that is no multiple of 64 or 4, K that is no
+    multiple of the 256-wide chunk, one split and many."""
+    g = torch.Generator().manual_seed(m * n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    b = torch.randn(n, generator=g).bfloat16()
+    want = x.double() @ w.double().T + b.double()
+    for max_splits in (None, 1):
+        partial = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV), max_splits=max_splits)
+        assert partial.dtype == torch.float32 and partial.shape[1:] == (m, n)
+        if max_splits == 1:
+            assert partial.shape[0] == 1
+        got = partial.double().sum(0).cpu()
+        assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1)
+    none = ops.gemm_skinny(x.to(DEV), torch.zeros_like(w).to(DEV), b.to(DEV)).sum(0).cpu()
+    torch.testing.assert_close(none, b.float().expand(m, n), rtol=0, atol=0)  # the bias, once
+
+
+def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(40, 1000, generator=g).bfloat16()
+    w = torch.randn(200, 1000, generator=g).bfloat16()
+    full = ops.gemm_skinny(x.to(DEV), w.to(DEV)).cpu()
+    one = ops.gemm_skinny(x[17:18].to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(full[:, 17:18], one)
+
+
+def test_consumers_add_up_partial_sums(ops):
+    """Norm, SwiGLU and rotary/cache write take the skinny product's 32-bit partial sums and
+    give what they give for the summed tensor."""
+    from turboserve_amd.parts.rope import rotary_tables
+
+    g = torch.Generator().manual_seed(8)
+    tokens, hidden, splits = 6, 200, 3
+    parts = torch.randn(splits, tokens, hidden, generator=g)
+    total = parts.sum(0)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).bfloat16()
+    residual = torch.randn(tokens, hidden, generator=g)
+    res_dev = residual.to(DEV)
+    got = ops.add_rmsnorm(res_dev, parts.to(DEV), w.to(DEV), 1e-6).float().cpu()
+    torch.testing.assert_close(res_dev.cpu(), residual + total, rtol=0, atol=1e-5)
+    torch.testing.assert_close(got, plain.rms_norm(residual + total, w.float(), 1e-6), **tol(torch.bfloat16))
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    got = ops.add_rmsnorm(residual.to(DEV), parts.to(DEV), w.to(DEV), 1e-6, rows).float().cpu()
+    torch.testing.assert_close(got, plain.rms_norm(residual + total, w.float(), 1e-6)[[4, 1]], **tol(torch.bfloat16))
+
+    gu = torch.randn(splits, tokens, 2 * 72, generator=g)
+    want = torch.nn.functional.silu(gu.sum(0)[:, :72]) * gu.sum(0)[:, 72:]
+    torch.testing.assert_close(ops.swiglu(gu.to(DEV), torch.bfloat16).float().cpu(), want, **tol(torch.bfloat16))
+
+    heads, kv_heads, dim, page = 3, 1, 32, 8
+    proj = torch.randn(splits, tokens, (heads + 2 * kv_heads) * dim, generator=g)
+    positions = torch.tensor([0, 5, 6, 30, 31, 2], dtype=torch.int32)
+    slots = [3, 17, 9, 0, 25, 31]
+    cos, sin = rotary_tables(64, dim, 1e4, 1.0)
+    kp = torch.zeros(4, kv_heads, page, dim, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(4, kv_heads, dim, page, dtype=torch.bfloat16, device=DEV)
+    q, q_stride = ops.rope_store(proj.to(DEV), kp, vp, cos.to(DEV), sin.to(DEV), positions.to(DEV),
+                                 torch.tensor(slots, dtype=torch.int32, device=DEV), heads, kv_heads, dim, page, 31,
+                                 torch.bfloat16)
+    assert q.shape == (tokens, heads * dim) and q_stride == heads * dim and q.dtype == torch.bfloat16
+    summed = proj.sum(0)
+    angles = plain.rope_angles(positions, dim, 1e4)
+    q_want = plain.apply_rope(summed[:, : heads * dim].view(tokens, heads, dim), angles)
+    k_want = plain.apply_rope(summed[:, heads * dim:(heads + kv_heads) * dim].view(tokens, kv_heads, dim), angles)
+    v = summed[:, (heads + kv_heads) * dim:].view(tokens, kv_heads, dim)
+    torch.testing.assert_close(q.float().cpu().view(tokens, heads, dim), q_want, **tol(torch.bfloat16))
+    kp_want, vp_want = scatter_reference(k_want, v, slots, 4, kv_heads, page, dim)
+    torch.testing.assert_close(kp.float().cpu(), kp_want, **tol(torch.bfloat16))
+    torch.testing.assert_close(vp.float().cpu(), vp_want, **tol(torch.bfloat16))
+
+
 # -- rotary + cache write ---------------------------------------------------------------------------
 
 
@@ -158,8 +234,8 @@ def test_rope_store(ops, dtype, heads, kv_heads, dim, page, theta, factor):
     q_want, k_want = plain.apply_rope(q, angles), plain.apply_rope(k, angles)
     got = dev.float().cpu()
     torch.testing.assert_close(got[:, : heads * dim].view(tokens, heads, dim), q_want, **tol(dtype))
-    torch.testing.assert_close(got[:, heads * dim:(heads + kv_heads) * dim].view(tokens, kv_heads, dim), k_want, **tol(dtype))
-    torch.testing.assert_close(got[:, (heads + kv_heads) * dim:], qkv.float()[:, (heads + kv_heads) * dim:], rtol=0, atol=0)
+    # Only the queries are rotated in place; keys and values leave through the pages.
+    torch.testing.assert_close(got[:, heads * dim:], qkv.float()[:, heads * dim:], rtol=0, atol=0)
     kp_want, vp_want = scatter_reference(k_want, v, slots, num_pages, kv_heads, page, dim)
     torch.testing.assert_close(kp.float().cpu(), kp_want, **tol(dtype))
     torch.testing.assert_close(vp.float().cpu(), vp_want, rtol=0, atol=0)

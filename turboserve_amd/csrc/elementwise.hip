@@ -64,36 +64,32 @@ __global__ void rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x, const
   }
 }
 
-template <typename T>
+// P is the type of `pending`: T, or float for `splits` partial sums of a product that are
+// `split_stride` elements apart and are added up here.
+template <typename T, typename P>
 __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residual,
-                                   const T* __restrict__ pending, const T* __restrict__ w,
-                                   const int* __restrict__ rows, float eps, int hidden) {
+                                   const P* __restrict__ pending, int splits, size_t split_stride,
+                                   const T* __restrict__ w, const int* __restrict__ rows, float eps,
+                                   int hidden) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
   const size_t out_base = (size_t)blockIdx.x * hidden;
   float ss = 0.f;
-  if (rows) {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      float s = residual[in_base + i];
-      if (pending) s += to_float(pending[in_base + i]);
-      ss += s * s;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float s = residual[in_base + i];
+    if (pending) {
+      for (int sp = 0; sp < splits; ++sp) s += to_float(pending[sp * split_stride + in_base + i]);
+      if (!rows) residual[in_base + i] = s;  // re-read below by this same thread
     }
-  } else {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      float s = residual[in_base + i];
-      if (pending) {
-        s += to_float(pending[in_base + i]);
-        residual[in_base + i] = s;  // re-read below by this same thread
-      }
-      ss += s * s;
-    }
+    ss += s * s;
   }
   ss = block_sum(ss, scratch);
   const float rstd = rsqrtf(ss / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
-    if (rows && pending) s += to_float(pending[in_base + i]);
+    if (rows && pending)
+      for (int sp = 0; sp < splits; ++sp) s += to_float(pending[sp * split_stride + in_base + i]);
     const float n = round_to<T>(s * rstd);
     y[out_base + i] = from_float<T>(to_float(w[i]) * n);
   }
@@ -114,16 +110,19 @@ extern "C" int ts_rmsnorm(void* y, const void* x, const void* w, float eps, int 
 }
 
 // `out_rows` = rows of y written: the number of entries of `rows` if given, else the tokens.
-extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, const void* w,
-                              const int* rows, float eps, int out_rows, int hidden, int dtype,
-                              hipStream_t stream) {
+// pending_f32 != 0: `pending` holds `splits` 32-bit partial sums, `split_stride` elements apart.
+extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int pending_f32, int splits,
+                              long split_stride, const void* w, const int* rows, float eps, int out_rows,
+                              int hidden, int dtype, hipStream_t stream) {
   if (out_rows == 0) return TS_OK;
-  if (!y || !residual || !w || hidden < 1) return TS_ERR_ARG;
+  if (!y || !residual || !w || hidden < 1 || splits < 1) return TS_ERR_ARG;
   dim3 grid(out_rows), block(hidden <= 1024 ? 256 : 1024);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, (float*)y, residual, (const float*)pending, (const float*)w, rows, eps, hidden);
+    hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), grid, block, 0, stream, (float*)y, residual, (const float*)pending, splits, (size_t)split_stride, (const float*)w, rows, eps, hidden);
+  else if (dtype == TS_BF16 && pending_f32)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)y, residual, (const float*)pending, splits, (size_t)split_stride, (const bf16_t*)w, rows, eps, hidden);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, residual, (const bf16_t*)pending, (const bf16_t*)w, rows, eps, hidden);
+    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)y, residual, (const bf16_t*)pending, splits, (size_t)split_stride, (const bf16_t*)w, rows, eps, hidden);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
@@ -132,55 +131,63 @@ extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, con
 // ---------------------------------------------------------------------------------------------
 // SwiGLU over the fused gate|up projection: out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 // ---------------------------------------------------------------------------------------------
-template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int inter,
-                              size_t total) {
+// P: type of the projection output: T, or float for `splits` partial sums to be added up.
+template <typename T, typename P>
+__global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
+                              size_t split_stride, int inter, size_t total) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t t = idx / inter;
   const int i = (int)(idx - t * inter);
-  const float g = to_float(gate_up[t * 2 * inter + i]);
-  const float u = to_float(gate_up[t * 2 * inter + inter + i]);
+  float g = 0.f, u = 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    g += to_float(gate_up[sp * split_stride + t * 2 * inter + i]);
+    u += to_float(gate_up[sp * split_stride + t * 2 * inter + inter + i]);
+  }
   const float act = g / (1.f + expf(-g));
   out[idx] = from_float<T>(act * u);
 }
 
-extern "C" int ts_swiglu(void* out, const void* gate_up, int tokens, int inter, int dtype,
-                         hipStream_t stream) {
+extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits, long split_stride,
+                         int tokens, int inter, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!out || !gate_up || inter < 1) return TS_ERR_ARG;
+  if (!out || !gate_up || inter < 1 || splits < 1) return TS_ERR_ARG;
   const size_t total = (size_t)tokens * inter;
   dim3 block(256), grid((unsigned)((total + 255) / 256));
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)gate_up, inter, total);
+    hipLaunchKernelGGL((swiglu_kernel<float, float>), grid, block, 0, stream, (float*)out, (const float*)gate_up, splits, (size_t)split_stride, inter, total);
+  else if (dtype == TS_BF16 && in_f32)
+    hipLaunchKernelGGL((swiglu_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)out, (const float*)gate_up, splits, (size_t)split_stride, inter, total);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)gate_up, inter, total);
+    hipLaunchKernelGGL((swiglu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)gate_up, splits, (size_t)split_stride, inter, total);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
 }
 
 // ---------------------------------------------------------------------------------------------
-// Rotary encoding + cache write.  qkv is [T, (Hq + 2 Hkv) * D]: q heads, then k heads, then v
-// heads.  One block per (token, head).  q and k are rotated in place by the angles of the
-// token's position (cos/sin tables are 32-bit, [capacity, D/2]; pair (i, i + D/2)); k (rotated)
-// and v go to the pages at slot = block * BS + offset.  Key pages are [NB, Hkv, BS, D]; value
-// pages are transposed, [NB, Hkv, D, BS], so that the attention kernels read eight consecutive
-// keys' values of one head dimension with a single 16-byte load.
-// rotate == 0 skips the rotation (a position encoding that only stores).
+// Rotary encoding + cache write.  The projection output is [T, (Hq + 2 Hkv) * D]: q heads, then
+// k heads, then v heads; it is either of type T, or `splits` 32-bit partial sums that are added
+// up here.  One block per (token, head).  q and k are rotated by the angles of the token's
+// position (cos/sin tables are 32-bit, [capacity, D/2]; pair (i, i + D/2)); the rotated q goes
+// to q_out (rows q_stride apart; with a projection of type T this may be the projection itself:
+// rotation in place); k (rotated) and v go to the pages at slot = block * BS + offset.  Key
+// pages are [NB, Hkv, BS, D]; value pages are transposed, [NB, Hkv, D, BS], so that the
+// attention kernels read eight consecutive keys' values of one head dimension with a single
+// 16-byte load.  rotate == 0 skips the rotation (a position encoding that only stores).
 // slots == nullptr or a negative slot: nothing is stored for that token.
 // ---------------------------------------------------------------------------------------------
-template <typename T>
-__global__ void rope_store_kernel(T* __restrict__ qkv, T* __restrict__ k_pages,
-                                  T* __restrict__ v_pages, const float* __restrict__ cos_table,
-                                  const float* __restrict__ sin_table,
+template <typename T, typename P>
+__global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int splits,
+                                  size_t split_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                  const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                                   const int* __restrict__ positions, const int* __restrict__ slots,
                                   int heads, int kv_heads, int dim, int block_size, int rotate) {
   const int t = blockIdx.x;
   const int h = blockIdx.y;
   const int half = dim / 2;
   const int width = (heads + 2 * kv_heads) * dim;
-  T* row = qkv + (size_t)t * width + (size_t)h * dim;
+  const P* row = proj + (size_t)t * width + (size_t)h * dim;
   const int pos = positions[t];
   const int slot = slots ? slots[t] : -1;
   T* page = nullptr;   // this token's row of a key page
@@ -195,40 +202,54 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, T* __restrict__ k_pages,
     else
       vpage = v_pages + head_base + off;
   }
-  if (h < heads + kv_heads && rotate) {
+  T* qrow = (h < heads) ? q_out + (size_t)t * q_stride + (size_t)h * dim : nullptr;
+  if (h < heads + kv_heads) {
     const float* c = cos_table + (size_t)pos * half;
     const float* s = sin_table + (size_t)pos * half;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      const float x1 = to_float(row[i]);
-      const float x2 = to_float(row[i + half]);
-      const T o1 = from_float<T>(x1 * c[i] - x2 * s[i]);
-      const T o2 = from_float<T>(x2 * c[i] + x1 * s[i]);
-      row[i] = o1;
-      row[i + half] = o2;
+      float x1 = 0.f, x2 = 0.f;
+      for (int sp = 0; sp < splits; ++sp) {
+        x1 += to_float(row[sp * split_stride + i]);
+        x2 += to_float(row[sp * split_stride + i + half]);
+      }
+      const T o1 = from_float<T>(rotate ? x1 * c[i] - x2 * s[i] : x1);
+      const T o2 = from_float<T>(rotate ? x2 * c[i] + x1 * s[i] : x2);
+      if (qrow) {
+        qrow[i] = o1;
+        qrow[i + half] = o2;
+      }
       if (page) {
         page[i] = o1;
         page[i + half] = o2;
       }
     }
   } else if (vpage) {
-    for (int i = threadIdx.x; i < dim; i += blockDim.x) vpage[(size_t)i * block_size] = row[i];
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+      float x = 0.f;
+      for (int sp = 0; sp < splits; ++sp) x += to_float(row[sp * split_stride + i]);
+      vpage[(size_t)i * block_size] = from_float<T>(x);
+    }
   }
 }
 
-extern "C" int ts_rope_store(void* qkv, void* k_pages, void* v_pages, const float* cos_table,
-                             const float* sin_table, const int* positions, const int* slots,
-                             int tokens, int heads, int kv_heads, int dim, int block_size,
-                             int rotate, int dtype, hipStream_t stream) {
+extern "C" int ts_rope_store(void* q_out, long q_stride, const void* proj, int in_f32, int splits,
+                             long split_stride, void* k_pages, void* v_pages, const float* cos_table,
+                             const float* sin_table, const int* positions, const int* slots, int tokens,
+                             int heads, int kv_heads, int dim, int block_size, int rotate, int dtype,
+                             hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!qkv || !positions || heads < 1 || kv_heads < 1 || dim < 2 || (dim & 1) || block_size < 1)
+  if (!q_out || !proj || !positions || heads < 1 || kv_heads < 1 || dim < 2 || (dim & 1) || block_size < 1 ||
+      splits < 1)
     return TS_ERR_ARG;
   if (rotate && (!cos_table || !sin_table)) return TS_ERR_ARG;
   if (slots && (!k_pages || !v_pages)) return TS_ERR_ARG;
   dim3 grid(tokens, heads + 2 * kv_heads), block(64);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, (float*)k_pages, (float*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
+    hipLaunchKernelGGL((rope_store_kernel<float, float>), grid, block, 0, stream, (float*)q_out, q_stride, (const float*)proj, splits, (size_t)split_stride, (float*)k_pages, (float*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
+  else if (dtype == TS_BF16 && in_f32)
+    hipLaunchKernelGGL((rope_store_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)q_out, q_stride, (const float*)proj, splits, (size_t)split_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
+    hipLaunchKernelGGL((rope_store_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)q_out, q_stride, (const bf16_t*)proj, splits, (size_t)split_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

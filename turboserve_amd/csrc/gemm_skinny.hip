@@ -1,0 +1,212 @@
+// Weight-streaming product for decode-sized batches:
+//   partial[s][m][n] = sum over the k-range of split s of  X[m][k] * W[n][k]   (+ bias[n] in split 0)
+// for M <= 64 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
+// them (F.linear's layout, src/turboserve/engine/model/layers.py:142), 32-bit accumulation on
+// the matrix cores and 32-bit partial sums out.  The consumer (norm, rotary/cache write,
+// SwiGLU, or nobody when splits == 1) adds the splits up, so no rounding happens between the
+// product and its consumer.
+//
+// At these batch sizes the product is bound by reading W once from HBM.  Layout of the work:
+//   * a workgroup of 4 wavefronts owns 64 consecutive weight rows (16 per wavefront) and one
+//     k-range; the grid is (row blocks, splits);
+//   * the k-range is walked in chunks of 256; a lane loads 128 contiguous bytes of its weight
+//     row per chunk (the four lane groups of a row cover 512 contiguous bytes), one chunk
+//     ahead of the matrix cores;
+//   * the chunk's activations are staged once per workgroup in LDS (rows padded against bank
+//     conflicts) and read as B operands by all four wavefronts; they are fetched from global
+//     memory into registers two chunks ahead and written to LDS one chunk ahead;
+//   * v_mfma_f32_16x16x32_bf16 with A = 16 weight rows, B = 16 activation rows; k index 8 g + e
+//     of step j stands for k = chunk + 64 g + 8 j + e on both operands, which is what makes the
+//     per-lane loads contiguous.
+#include "common.hpp"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int CHUNK = 256;          // k per iteration
+constexpr int STEPS = CHUNK / 32;   // matrix-core steps per chunk
+constexpr int ROWS_PER_WAVE = 16;
+constexpr int WAVES = 4;
+constexpr int ROWS_PER_BLOCK = ROWS_PER_WAVE * WAVES;
+constexpr int X_ROW = CHUNK + 8;    // LDS row stride in elements (16 bytes of padding)
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+struct WeightChunk {
+  u32x4 piece[STEPS];  // k = chunk + 64 g + 8 j .. + 7 of the lane's row, j = 0..7
+};
+
+// `row` points at the lane's weight row; k_limit = K: pieces at or beyond it read as zero
+// (K is a multiple of 8, so a piece is wholly inside or wholly outside).
+__device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row, int k0, int group, int k_limit) {
+  const int base = k0 + 64 * group;
+  if (k0 + CHUNK <= k_limit) {
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) w.piece[j] = *reinterpret_cast<const u32x4*>(row + base + 8 * j);
+  } else {
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+      const int k = base + 8 * j;
+      w.piece[j] = (k < k_limit) ? *reinterpret_cast<const u32x4*>(row + k) : u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+}
+
+// The activations of one chunk, X[0..m-1][k0 .. k0+255], travel in two hops: global memory to
+// registers (issued a whole iteration before they are needed), registers to LDS.  A thread
+// carries 2 MT pieces of 16 bytes; rows >= m and k >= K are zeros.
+template <int MT>
+struct ActivationRegs {
+  u32x4 piece[2 * MT];
+};
+
+template <int MT>
+__device__ __forceinline__ void fetch_activations(ActivationRegs<MT>& r, const uint16_t* __restrict__ x,
+                                                  long x_stride, int m, int k0, int k_limit) {
+#pragma unroll
+  for (int i = 0; i < 2 * MT; ++i) {
+    const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
+    const int row = idx / (CHUNK / 8);
+    const int k = k0 + 8 * (idx % (CHUNK / 8));
+    r.piece[i] = (row < m && k < k_limit) ? *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + k)
+                                          : u32x4{0u, 0u, 0u, 0u};
+  }
+}
+
+template <int MT>
+__device__ __forceinline__ void store_activations(uint16_t* lds, const ActivationRegs<MT>& r) {
+#pragma unroll
+  for (int i = 0; i < 2 * MT; ++i) {
+    const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
+    *reinterpret_cast<u32x4*>(lds + (idx / (CHUNK / 8)) * X_ROW + 8 * (idx % (CHUNK / 8))) = r.piece[i];
+  }
+}
+
+template <int MT>
+__device__ __forceinline__ void multiply_chunk(f32x4 (&acc)[MT], const WeightChunk& w, const uint16_t* xs,
+                                               int lane16, int group) {
+#pragma unroll
+  for (int j = 0; j < STEPS; ++j) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const u32x4 b = *reinterpret_cast<const u32x4*>(xs + (16 * t + lane16) * X_ROW + 64 * group + 8 * j);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w.piece[j]), as_bf16x8(b), acc[t], 0, 0, 0);
+    }
+  }
+}
+
+template <int MT>
+__global__ void __launch_bounds__(WAVES * TS_WAVE)
+gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
+                   const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
+                   int chunks_per_split) {
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16 * X_ROW];
+  const int lane = threadIdx.x & (TS_WAVE - 1);
+  const int wave = threadIdx.x / TS_WAVE;
+  const int lane16 = lane & 15;
+  const int group = lane >> 4;
+  const int split = blockIdx.y;
+  const int n0 = blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE;
+  const int total_chunks = (k + CHUNK - 1) / CHUNK;
+  const int first = split * chunks_per_split;
+  const int last = min(first + chunks_per_split, total_chunks);  // exclusive
+
+  // Rows beyond N repeat the last row; their sums are never stored.
+  const int row_index = min(n0 + lane16, n - 1);
+  const uint16_t* wrow = w + (size_t)row_index * k;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (first < last) {
+    // Invariant at the top of a round for chunk c: xs[buf] holds chunk c (complete, behind a
+    // barrier), `xr` holds chunk c + 1's activations (loads issued a round ago), and the
+    // weight registers of this round hold chunk c.
+    WeightChunk wa, wb;
+    ActivationRegs<MT> xr;
+    load_weights(wa, wrow, first * CHUNK, group, k);
+    fetch_activations<MT>(xr, x, x_stride, m, first * CHUNK, k);
+    store_activations<MT>(xs[0], xr);
+    if (first + 1 < last) fetch_activations<MT>(xr, x, x_stride, m, (first + 1) * CHUNK, k);
+    __syncthreads();
+    int c = first;
+    int buf = 0;
+    while (true) {
+      if (c + 1 < last) {
+        store_activations<MT>(xs[buf ^ 1], xr);  // free since the last barrier
+        load_weights(wb, wrow, (c + 1) * CHUNK, group, k);
+        if (c + 2 < last) fetch_activations<MT>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
+      }
+      multiply_chunk<MT>(acc, wa, xs[buf], lane16, group);
+      __syncthreads();
+      if (++c >= last) break;
+      buf ^= 1;
+      if (c + 1 < last) {
+        store_activations<MT>(xs[buf ^ 1], xr);
+        load_weights(wa, wrow, (c + 1) * CHUNK, group, k);
+        if (c + 2 < last) fetch_activations<MT>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
+      }
+      multiply_chunk<MT>(acc, wb, xs[buf], lane16, group);
+      __syncthreads();
+      if (++c >= last) break;
+      buf ^= 1;
+    }
+  }
+
+  // acc[t][i] = sum for weight row n0 + 4 g + i and activation row 16 t + lane16.
+  const int nrow = n0 + 4 * group;
+  if (nrow < n) {
+    f32x4 b = {0.f, 0.f, 0.f, 0.f};
+    if (bias && split == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nrow + i < n) b[i] = to_float(bf16_t{bias[nrow + i]});
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int row = 16 * t + lane16;
+      if (row >= m) continue;
+      float* dst = partial + ((size_t)split * m + row) * n + nrow;
+      const f32x4 v = acc[t] + b;
+      if (nrow + 3 < n && (n & 3) == 0) {
+        *reinterpret_cast<f32x4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nrow + i < n) dst[i] = v[i];
+      }
+    }
+  }
+}
+
+}  // namespace
+
+// partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
+// w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
+// chunks_per_split 256-wide chunks of k go to each of `splits` = ceil(ceil(k / 256) / chunks_per_split).
+extern "C" int ts_gemm_skinny(float* partial, const void* x, long x_stride, const void* w, const void* bias,
+                              int m, int n, int k, int chunks_per_split, int splits, hipStream_t stream) {
+  if (m == 0 || n == 0) return TS_OK;
+  if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
+  if (m > 64 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
+  const int total_chunks = (k + CHUNK - 1) / CHUNK;
+  if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
+  dim3 grid((n + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, splits), block(WAVES * TS_WAVE);
+  if (grid.y > 65535) return TS_ERR_SHAPE;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* bp = (const uint16_t*)bias;
+  if (m <= 16)
+    hipLaunchKernelGGL(gemm_skinny_kernel<1>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
+  else if (m <= 32)
+    hipLaunchKernelGGL(gemm_skinny_kernel<2>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
+  else if (m <= 48)
+    hipLaunchKernelGGL(gemm_skinny_kernel<3>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
+  else
+    hipLaunchKernelGGL(gemm_skinny_kernel<4>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
+  return ts_launch_status();
+}

@@ -35,6 +35,7 @@ MODULES: dict[str, tuple[str, ...]] = {
         "elementwise.hip",
         "attention_generic.hip",
         "gemm_plain.hip",
+        "gemm_skinny.hip",
         "sampling.hip",
     ),
 }

@@ -40,16 +40,18 @@ _SIGNATURES: dict[str, dict[str, list]] = {
     "core": {
         "ts_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
-        "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
-        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-        "ts_rope_store": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
+                           c_int, c_int, c_int, c_void_p],
+        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p],
+        "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_int, c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
+        "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -169,6 +171,24 @@ class Ops:
                                     dtype_code(x.dtype), self.stream()), "ts_rmsnorm")
         return y
 
+    @staticmethod
+    def _partials(t: torch.Tensor, rows: int, width: int, dtype: torch.dtype, what: str) -> tuple[int, int, int]:
+        """``(is_float32_partials, splits, split_stride)`` of a projection output: either
+        ``[rows, width]`` of the run dtype, or ``[S, rows, width]`` 32-bit partial sums (what the
+        skinny product leaves for its consumer to add up)."""
+        _need(t.is_contiguous(), f"{what} must be contiguous")
+        if t.dim() == 3:
+            _need(t.dtype == torch.float32 and t.shape[1:] == (rows, width),
+                  f"{what}: partial sums must be float32 [S, {rows}, {width}]")
+            return 1, t.shape[0], rows * width
+        _need(t.shape == (rows, width) and t.dtype == dtype, f"{what} must be [{rows}, {width}] of {dtype}")
+        return 0, 1, 0
+
+    def dense(self, t: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        """A projection output as one ``[rows, width]`` tensor of ``dtype`` (partial sums added
+        up), for consumers that have no fused form."""
+        return t.sum(dim=0).to(dtype) if t.dim() == 3 else t
+
     def add_rmsnorm(
         self,
         residual: torch.Tensor,
@@ -178,32 +198,38 @@ class Ops:
         rows: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """``residual += pending`` in 32-bit (in place) and the normalised sum in ``weight``'s
-        dtype; with ``rows`` only those rows, and ``residual`` is left alone."""
+        dtype; with ``rows`` only those rows, and ``residual`` is left alone.  ``pending`` is a
+        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums."""
         _gpu(residual, pending, weight, rows)
         _i32(rows, "rows")
         _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
               "residual must be contiguous float32 [T, H]")
         tokens, hidden = residual.shape
         _need(weight.shape == (hidden,) and weight.is_contiguous(), "weight must be [H]")
+        is_f32, splits, stride = (0, 1, 0)
         if pending is not None:
-            _need(pending.shape == residual.shape and pending.dtype == weight.dtype and pending.is_contiguous(),
-                  "pending must be contiguous [T, H] of the weight's dtype")
+            is_f32, splits, stride = self._partials(pending, tokens, hidden, weight.dtype, "pending")
         out_rows = tokens if rows is None else rows.numel()
         y = torch.empty((out_rows, hidden), dtype=weight.dtype, device=residual.device)
-        _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), _ptr(weight), _ptr(rows),
-                                        float(eps), out_rows, hidden, dtype_code(weight.dtype), self.stream()),
-               "ts_add_rmsnorm")
+        _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight),
+                                        _ptr(rows), float(eps), out_rows, hidden, dtype_code(weight.dtype),
+                                        self.stream()), "ts_add_rmsnorm")
         return y
 
-    def swiglu(self, gate_up: torch.Tensor) -> torch.Tensor:
-        """``silu(gate) * up`` of the fused ``[T, 2 I]`` projection -> ``[T, I]``."""
+    def swiglu(self, gate_up: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+        """``silu(gate) * up`` of the fused ``[T, 2 I]`` projection (or its ``[S, T, 2 I]`` 32-bit
+        partial sums) -> ``[T, I]`` of ``dtype`` (the projection's own if it is not partial)."""
         _gpu(gate_up)
-        _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
-              "gate_up must be contiguous [T, 2 I]")
-        tokens, inter = gate_up.shape[0], gate_up.shape[1] // 2
-        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
-        _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), tokens, inter, dtype_code(gate_up.dtype),
-                                   self.stream()), "ts_swiglu")
+        tokens, width = gate_up.shape[-2], gate_up.shape[-1]
+        _need(width % 2 == 0, "gate_up must be [T, 2 I]")
+        out_dtype = dtype or gate_up.dtype
+        if gate_up.dim() == 3:
+            _need(dtype is not None, "partial sums need the output dtype")
+        is_f32, splits, stride = self._partials(gate_up, tokens, width, out_dtype, "gate_up")
+        inter = width // 2
+        out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
+        _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
+                                   dtype_code(out_dtype), self.stream()), "ts_swiglu")
         return out
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
@@ -217,7 +243,7 @@ class Ops:
 
     def rope_store(
         self,
-        qkv: torch.Tensor,
+        proj: torch.Tensor,
         k_pages: torch.Tensor | None,
         v_pages: torch.Tensor | None,
         cos: torch.Tensor | None,
@@ -229,17 +255,24 @@ class Ops:
         head_dim: int,
         block_size: int,
         max_position: int,
-    ) -> None:
-        """Rotate q and k of ``qkv [T, (Hq + 2 Hkv) D]`` in place (skipped when ``cos`` is
-        ``None``) and store k, v at ``slots`` into pages ``[NB, Hkv, BS, D]`` (skipped when
-        ``slots`` is ``None``).  ``max_position`` is the largest position of the step, known on
-        the host, and must lie inside the tables."""
-        _gpu(qkv, k_pages, v_pages, cos, sin, positions, slots)
+        dtype: torch.dtype | None = None,
+    ) -> tuple[torch.Tensor, int]:
+        """Rotate q and k of the fused projection ``[T, (Hq + 2 Hkv) D]`` (skipped when ``cos`` is
+        ``None``) and store k, v at ``slots`` into key pages ``[NB, Hkv, BS, D]`` and value pages
+        ``[NB, Hkv, D, BS]`` (skipped when ``slots`` is ``None``).  Returns the tensor that holds
+        the encoded queries and its row stride: the projection itself (rotated in place) when it
+        is a tensor of the run dtype, a new ``[T, Hq D]`` tensor of ``dtype`` when it is 32-bit
+        partial sums.  ``max_position`` is the largest position of the step, known on the host,
+        and must lie inside the tables."""
+        _gpu(proj, k_pages, v_pages, cos, sin, positions, slots)
         _i32(positions, "positions")
         _i32(slots, "slots")
         tokens = positions.numel()
         width = (heads + 2 * kv_heads) * head_dim
-        _need(qkv.shape == (tokens, width) and qkv.is_contiguous(), f"qkv must be contiguous [T, {width}]")
+        run_dtype = dtype or proj.dtype
+        if proj.dim() == 3:
+            _need(dtype is not None, "partial sums need the run dtype")
+        is_f32, splits, stride = self._partials(proj, tokens, width, run_dtype, "projection")
         _need(head_dim % 2 == 0, "head_dim must be even")
         if cos is not None:
             half = head_dim // 2
@@ -250,12 +283,18 @@ class Ops:
         if slots is not None:
             _need(slots.numel() == tokens, "one slot per token")
             _need(k_pages is not None and v_pages is not None, "slots given without pages")
-            _check_pages(k_pages, v_pages, qkv.dtype)
+            _check_pages(k_pages, v_pages, run_dtype)
             _need(k_pages.shape[1:] == (kv_heads, block_size, head_dim), "pages do not match the heads' geometry")
-        _check(self.core.ts_rope_store(_ptr(qkv), _ptr(k_pages), _ptr(v_pages), _ptr(cos), _ptr(sin),
-                                       _ptr(positions), _ptr(slots), tokens, heads, kv_heads, head_dim,
-                                       block_size, 0 if cos is None else 1, dtype_code(qkv.dtype), self.stream()),
-               "ts_rope_store")
+        if proj.dim() == 3:
+            q_out = torch.empty((tokens, heads * head_dim), dtype=run_dtype, device=proj.device)
+            q_stride = heads * head_dim
+        else:
+            q_out, q_stride = proj, width
+        _check(self.core.ts_rope_store(_ptr(q_out), q_stride, _ptr(proj), is_f32, splits, stride, _ptr(k_pages),
+                                       _ptr(v_pages), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens,
+                                       heads, kv_heads, head_dim, block_size, 0 if cos is None else 1,
+                                       dtype_code(run_dtype), self.stream()), "ts_rope_store")
+        return q_out, q_stride
 
     # -- attention ----------------------------------------------------------------------------
 
@@ -424,13 +463,51 @@ class Ops:
                "ts_gemm_plain")
         return y
 
+    #: Workgroups a skinny product aims for (four per compute unit of a 256-CU device).
+    skinny_target_blocks = 1024
+    #: Largest batch the skinny product serves; above it the BLAS library is used.
+    skinny_max_rows = 64
+
+    @staticmethod
+    def skinny_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+        """bfloat16, at most 64 rows, K a multiple of 8."""
+        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= 64
+                and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0)
+
+    def gemm_skinny(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                    *, max_splits: int | None = None) -> torch.Tensor:
+        """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
+        K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``."""
+        _gpu(x, weight, bias)
+        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
+              and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
+        _need(self.skinny_supported(x, weight), "the skinny product takes bfloat16, M <= 64 and K % 8 == 0")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
+        chunks = -(-k // 256)
+        row_blocks = -(-n // 64)
+        want = max(1, min(chunks, -(-self.skinny_target_blocks // row_blocks), max_splits or chunks))
+        per_split = -(-chunks // want)
+        splits = -(-chunks // per_split)
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        _check(self.core.ts_gemm_skinny(_ptr(partial), _ptr(x), x.stride(0) if m > 1 else max(k, x.stride(0)),
+                                        _ptr(weight), _ptr(bias), m, n, k, per_split, splits, self.stream()),
+               "ts_gemm_skinny")
+        return partial
+
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
-        """The projection of the serving path: 32-bit runs use :meth:`gemm_plain` (no reduced
-        matrix mode); bfloat16 runs use the BLAS library behind torch, as the reference does
-        for every linear layer (src/turboserve/engine/model/layers.py:142)."""
+        """The projection of the serving path.  32-bit runs use :meth:`gemm_plain` (no reduced
+        matrix mode).  bfloat16 runs with decode-sized batches use :meth:`gemm_skinny` and
+        return ``[S, M, N]`` 32-bit partial sums for the consumer to add up; larger batches use
+        the BLAS library behind torch, as the reference does for every linear layer
+        (src/turboserve/engine/model/layers.py:142)."""
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight, bias)
         _gpu(x, weight, bias)
+        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
+            return self.gemm_skinny(x, weight, bias)
         if bias is None:
             return torch.mm(x, weight.t())
         return torch.addmm(bias, x, weight.t())
@@ -441,6 +518,8 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight)
         _gpu(x, weight)
+        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
+            return self.gemm_skinny(x, weight, max_splits=1)[0]
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
 
     # -- sampling -----------------------------------------------------------------------------

@@ -90,12 +90,15 @@ class GroupedQueryAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
         ops = self.runtime.ops
         qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_tensor)
-        self.position.encode_and_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache)
-        attended = self.attend(qkv, ctx, cache)
+        q, q_stride = self.position.encode_and_store(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache
+        )
+        attended = self.attend(q, q_stride, ctx, cache)
         return ops.linear(attended, self.o_weight, self.o_bias_tensor)
 
-    def attend(self, qkv: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
-        """``[T, Hq D]`` attention output for the step's (encoded) queries in ``qkv``.
+    def attend(self, qkv: torch.Tensor, q_stride: int, ctx, cache: PagedKVView) -> torch.Tensor:
+        """``[T, Hq D]`` attention output for the step's encoded queries: the first ``Hq D``
+        elements of every ``q_stride``-long row of ``qkv``.
 
         bfloat16 runs use the matrix-core kernels where the geometry allows: one launch for the
         multi-token requests at the front of the batch, one for the single-token requests
@@ -107,17 +110,17 @@ class GroupedQueryAttention(Mixer):
             out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
             if ctx.num_prefill_seqs > 0:
                 ops.attention_prefill(
-                    out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
+                    out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     ctx.prefill_blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len,
                 )
             if ctx.num_decode_seqs > 0:
                 ops.attention_decode(
-                    out, qkv, qkv.shape[1], cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
+                    out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     ctx.num_prefill_seqs, ctx.num_decode_seqs, self.num_heads, self.scale, self.window,
                     ctx.max_decode_context_len,
                 )
             return out
         return ops.paged_attention_generic(
-            qkv, qkv.shape[1], cache.k, cache.v, table, ctx.token_seq, ctx.positions,
+            qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
             self.num_heads, self.scale, self.window,
         )

@@ -117,7 +117,7 @@ class ResidualStream:
     part's output ``pending [T, H]`` (run dtype) that has not been added to it yet."""
 
     residual: torch.Tensor
-    pending: torch.Tensor | None = None
+    pending: torch.Tensor | None = None  # [T, H] run dtype, or [S, T, H] 32-bit partial sums
 
 
 # ---------------------------------------------------------------------------------------------
@@ -176,9 +176,11 @@ class PositionEncoding(Part):
         head_dim: int,
         ctx: "StepContext",
         cache: PagedKVView,
-    ) -> None:
-        """``qkv [T, (Hq + 2 Hkv) D]``: encode q and k in place; write k, v at the step's slots
-        of ``cache.group`` unless the cache is not writable."""
+    ) -> tuple[torch.Tensor, int]:
+        """``qkv``: the fused projection ``[T, (Hq + 2 Hkv) D]`` as ``ops.linear`` returned it (a
+        tensor of the run dtype, or 32-bit partial sums ``[S, T, ..]``).  Encodes q and k, writes
+        k, v at the step's slots of ``cache.group`` unless the cache is not writable, and
+        returns the tensor holding the encoded queries with its row stride."""
         raise NotImplementedError
 
 
@@ -189,7 +191,8 @@ class Mixer(Part):
         return None
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: CacheView) -> torch.Tensor:
-        """``x [T, H]`` (normalised) -> ``[T, H]``.  The rows of request ``s`` are
+        """``x [T, H]`` (normalised) -> ``[T, H]`` of the run dtype (or, straight from
+        ``ops.linear``, ``[S, T, H]`` 32-bit partial sums).  The rows of request ``s`` are
         ``ctx.query_start_loc[s]:ctx.query_start_loc[s+1]``, in position order, continuing
         whatever earlier steps left in ``cache``."""
         raise NotImplementedError

@@ -63,12 +63,12 @@ class RotaryEncoding(PositionEncoding):
         self.sin = sin.to(self.runtime.device)
         self.capacity = target
 
-    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView) -> None:
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView):
         self.ensure_capacity(ctx.max_context_len)
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
-        self.runtime.ops.rope_store(
+        return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, self.cos, self.sin, ctx.positions, slots,
-            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1,
+            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
         )
 
 
@@ -81,10 +81,9 @@ class NoPositionEncoding(PositionEncoding):
     def __init__(self, prefix: str, runtime: Runtime) -> None:
         super().__init__(prefix, runtime)
 
-    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView) -> None:
-        if not cache.writable:
-            return
-        self.runtime.ops.rope_store(
-            qkv, cache.k, cache.v, None, None, ctx.positions, ctx.slot_mapping[cache.group],
-            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1,
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView):
+        slots = ctx.slot_mapping[cache.group] if cache.writable else None
+        return self.runtime.ops.rope_store(
+            qkv, cache.k, cache.v, None, None, ctx.positions, slots,
+            num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
         )

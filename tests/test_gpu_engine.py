@@ -125,3 +125,42 @@ def test_smoke_entry_point():
     import __graft_entry__
 
     __graft_entry__.smoke()
+
+
+def test_decode_graphs_replay_like_eager(model):
+    """Steps of single tokens are replayed as HIP graphs.  Every replay must equal the eager
+    step: several replays of one graph with different data, eager work and synchronisation
+    between them, batch sizes that are padded (3 -> 4) and exact, a request leaving the batch."""
+    import json
+    from pathlib import Path
+
+    import trace_helpers as th
+    from turboserve_amd.engine.replay import TraceReplayer
+
+    config = json.loads((Path(model["folder"]) / "config.json").read_text())
+    requests = {f"g{i}": tiny.random_tokens(config["vocab_size"], n, 900 + i) for i, n in enumerate([37, 21, 30])}
+    steps = []
+    for rid, tokens in requests.items():  # prompts whole, except the last 12 tokens
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": tokens[:-12], "want": []}], "end": []})
+    for k in range(12):  # then all three decode together; g1 leaves after 8 tokens
+        entries = [{"id": rid, "tokens": [tokens[len(tokens) - 12 + k]], "want": [0]}
+                   for rid, tokens in requests.items() if not (rid == "g1" and k >= 8)]
+        steps.append({"step": len(steps), "entries": entries, "end": ["g1"] if k == 7 else []})
+    results = {}
+    for dtype in ("float32", "bfloat16"):
+        for use_graphs in (False, True):
+            replayer = TraceReplayer(model["folder"], dtype=dtype, max_tokens=256, page_size=model["page"])
+            if not use_graphs:
+                replayer.runner.graphs = None
+            outs = []
+            for record in steps:
+                logits = replayer.run_step(record)
+                if logits.shape[0]:
+                    outs.append(logits.float().cpu())
+                    torch.cuda.synchronize()
+                    _ = (torch.ones(64, 64, device="cuda") @ torch.ones(64, 64, device="cuda")).sum().item()  # eager work between replays
+            results[(dtype, use_graphs)] = outs
+            if use_graphs:
+                assert replayer.runner.graphs.num_replays == 12
+        for eager, graph in zip(results[(dtype, False)], results[(dtype, True)]):
+            assert torch.equal(eager, graph), f"{dtype}: a graph replay differs from the eager step"

@@ -43,8 +43,11 @@ class CacheStorage:
             )
             for group, count in zip(layout.groups, num_pages)
         ]
+        # One row more than there are slots: the row padded batch entries point at.
+        self.num_state_slots = num_state_slots
+        self.pad_state_slot = num_state_slots
         self.states = [
-            torch.zeros((num_state_slots, *need.shape), dtype=need.dtype, device=device)
+            torch.zeros((num_state_slots + 1, *need.shape), dtype=need.dtype, device=device)
             for _, need in layout.state_entries
         ]
 

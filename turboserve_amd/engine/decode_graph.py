@@ -1,0 +1,201 @@
+"""Decode steps as HIP graphs.
+
+A step that brings one token for each of its requests launches a few hundred small kernels;
+at a batch of one the launches, not the GPU, set the pace.  Such a step is therefore recorded
+once per shape as a HIP graph (``torch.cuda.CUDAGraph``) over static buffers and replayed:
+per step the host fills one pinned int32 buffer (tokens, positions, slots, block tables,
+context lengths), copies it to the device and launches the graph.
+
+Shapes are bucketed so that few graphs serve every batch: the number of requests is rounded up
+to a power of two (the extra rows are padding: position 0, context 1, no cache write, results
+dropped) and each cache group's block-table width to a power of two.  The kernels read the
+true context lengths from the device, so one graph serves every length up to its width.  The
+graphs hold only this engine's own kernels (no library call, no memset node).
+
+The reference has no counterpart: it launches eager torch ops every step
+(src/turboserve/engine/runtime/worker.py:221-233).
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+
+import numpy as np
+import torch
+
+from turboserve_amd.engine.batch import StepContext, StepEntry
+
+
+def next_power_of_two(n: int) -> int:
+    return 1 if n <= 1 else 1 << (n - 1).bit_length()
+
+
+class _Graph:
+    """One recorded shape: its static input buffer, context, output and the graph."""
+
+    def __init__(self, batch: int, widths: tuple[int, ...]) -> None:
+        self.batch = batch
+        self.widths = widths
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.device_ints: torch.Tensor | None = None
+        self.host_ints: list[torch.Tensor] = []
+        self.turn = 0
+        self.ctx: StepContext | None = None
+        self.logits: torch.Tensor | None = None
+        self.offsets: dict[str, tuple[int, int]] = {}
+
+
+class DecodeGraphs:
+    def __init__(self, model, views, *, page_size: int, num_groups: int, pad_state_slot: int,
+                 max_batch: int = 64) -> None:
+        self.model = model
+        self.views = views
+        self.page_size = page_size
+        self.num_groups = num_groups
+        self.pad_state_slot = pad_state_slot
+        self.max_batch = max_batch
+        self.device = model.runtime.device
+        self._graphs: dict[tuple, _Graph] = {}
+        self._pool = None
+        self.num_replays = 0
+
+    # -- shape -----------------------------------------------------------------------------------
+
+    def accepts(self, entries: Sequence[StepEntry]) -> bool:
+        return 0 < len(entries) <= self.max_batch and all(len(e.tokens) == 1 for e in entries)
+
+    def _key(self, entries: Sequence[StepEntry]) -> tuple:
+        batch = next_power_of_two(len(entries))
+        widths = tuple(
+            max(4, next_power_of_two(max(len(e.tables[g]) for e in entries))) for g in range(self.num_groups)
+        )
+        return batch, widths
+
+    # -- buffers ---------------------------------------------------------------------------------
+
+    def _layout(self, batch: int, widths: tuple[int, ...]) -> tuple[dict[str, tuple[int, int]], int]:
+        """Offsets (start, length) of every field in the packed int32 buffer."""
+        offsets: dict[str, tuple[int, int]] = {}
+        cursor = 0
+
+        def take(name: str, length: int) -> None:
+            nonlocal cursor
+            offsets[name] = (cursor, length)
+            cursor += -(-length // 4) * 4  # keep every field 16-byte aligned
+
+        for name in ("token_ids", "positions", "token_seq", "context_lens", "state_slots", "logit_rows"):
+            take(name, batch)
+        take("query_start_loc", batch + 1)
+        for g, width in enumerate(widths):
+            take(f"slots{g}", batch)
+            take(f"table{g}", batch * width)
+        return offsets, cursor
+
+    def _build(self, key: tuple) -> _Graph:
+        batch, widths = key
+        shape = _Graph(batch, widths)
+        shape.offsets, total = self._layout(batch, widths)
+        shape.device_ints = torch.zeros(total, dtype=torch.int32, device=self.device)
+        shape.host_ints = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]
+
+        def view(name: str) -> torch.Tensor:
+            start, length = shape.offsets[name]
+            return shape.device_ints[start:start + length]
+
+        max_context = max(widths) * self.page_size
+        shape.ctx = StepContext(
+            num_tokens=batch,
+            num_seqs=batch,
+            token_ids=view("token_ids"),
+            positions=view("positions"),
+            token_seq=view("token_seq"),
+            query_start_loc=view("query_start_loc"),
+            context_lens=view("context_lens"),
+            state_slots=view("state_slots"),
+            logit_rows=view("logit_rows"),
+            prefill_blocks=torch.zeros((0, 2), dtype=torch.int32, device=self.device),
+            slot_mapping=[view(f"slots{g}") for g in range(self.num_groups)],
+            block_tables=[view(f"table{g}").view(batch, widths[g]) for g in range(self.num_groups)],
+            query_lens=[1] * batch,
+            context_lens_host=[max_context] * batch,
+            max_query_len=1,
+            max_context_len=max_context,
+            num_logit_rows=batch,
+            num_prefill_seqs=0,
+            num_decode_seqs=batch,
+            num_prefill_tokens=0,
+            max_prefill_context_len=0,
+            max_decode_context_len=max_context,
+        )
+        # Harmless contents for the eager warm-up and the recording: every row is padding.
+        shape.device_ints.copy_(self._fill(shape, []))
+
+        def run() -> torch.Tensor:
+            stream = self.model.forward(shape.ctx.token_ids, shape.ctx, self.views)
+            return self.model.logits(stream, shape.ctx.logit_rows)
+
+        # Once eagerly on a side stream (tables grow, libraries load, allocator warms up), then record.
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            run()
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        shape.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(shape.graph, pool=self._pool):
+            shape.logits = run()
+        if self._pool is None:
+            self._pool = shape.graph.pool()
+        return shape
+
+    def _fill(self, shape: _Graph, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Write a step into the next pinned buffer; rows beyond the entries are padding."""
+        shape.turn ^= 1
+        host = shape.host_ints[shape.turn]
+        data = host.numpy()
+        batch, live = shape.batch, len(entries)
+
+        def field(name: str) -> np.ndarray:
+            start, length = shape.offsets[name]
+            return data[start:start + length]
+
+        field("token_ids")[:live] = [e.tokens[0] for e in entries]
+        field("token_ids")[live:] = 0
+        field("positions")[:live] = [e.start for e in entries]
+        field("positions")[live:] = 0
+        field("token_seq")[:] = np.arange(batch, dtype=np.int32)
+        field("context_lens")[:live] = [e.start + 1 for e in entries]
+        field("context_lens")[live:] = 1
+        field("state_slots")[:live] = [e.state_slot for e in entries]
+        field("state_slots")[live:] = self.pad_state_slot
+        field("logit_rows")[:] = np.arange(batch, dtype=np.int32)
+        field("query_start_loc")[:] = np.arange(batch + 1, dtype=np.int32)
+        for g, width in enumerate(shape.widths):
+            slots = field(f"slots{g}")
+            slots[:live] = [e.slots[g][0] for e in entries]
+            slots[live:] = -1  # padding writes nothing
+            table = field(f"table{g}").reshape(batch, width)
+            table[:] = 0  # padding (and the unused tail of a row) points at page 0: never read past the context
+            for i, e in enumerate(entries):
+                row = e.tables[g]
+                table[i, : len(row)] = row
+        return host
+
+    # -- the step --------------------------------------------------------------------------------
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Replay the graph of the entries' shape; returns the graph's own 32-bit logits buffer
+        ``[len(entries), V]`` (overwritten by the next replay of that shape)."""
+        key = self._key(entries)
+        shape = self._graphs.get(key)
+        if shape is None:
+            shape = self._graphs[key] = self._build(key)
+        host = self._fill(shape, entries)
+        shape.device_ints.copy_(host, non_blocking=True)
+        shape.graph.replay()
+        self.num_replays += 1
+        return shape.logits[: len(entries)]
+
+    def release(self) -> None:
+        self._graphs.clear()
+        self._pool = None

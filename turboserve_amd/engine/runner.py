@@ -16,12 +16,14 @@ import torch
 
 from turboserve_amd.cache.layout import CacheLayout
 from turboserve_amd.cache.storage import CacheStorage
-from turboserve_amd.engine.batch import StepContext, StepEntry, build_context
+from turboserve_amd.engine.batch import StepContext, StepEntry, build_context, validate_entries
+from turboserve_amd.engine.decode_graph import DecodeGraphs
 from turboserve_amd.models.decoder import DecoderModel
 
 
 class ModelRunner:
-    def __init__(self, model: DecoderModel, storage: CacheStorage, *, check: bool = True) -> None:
+    def __init__(self, model: DecoderModel, storage: CacheStorage, *, check: bool = True,
+                 use_graphs: bool = True, max_graph_batch: int = 64) -> None:
         self.model = model
         self.storage = storage
         self.layout: CacheLayout = storage.layout
@@ -29,19 +31,32 @@ class ModelRunner:
         self.views = storage.views()
         self.vocab_size = model.plan.vocab_size
         self.num_steps = 0
+        #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``).
+        self.graphs: DecodeGraphs | None = None
+        if use_graphs:
+            self.graphs = DecodeGraphs(
+                model, self.views, page_size=storage.page_size, num_groups=len(self.layout.groups),
+                pad_state_slot=storage.pad_state_slot, max_batch=max_graph_batch,
+            )
 
     def release(self) -> None:
         """Drop the cache tensors (the engine is closing)."""
         self.views = []
         self.storage = None
+        if self.graphs is not None:
+            self.graphs.release()
+            self.graphs = None
+
+    def check_tokens(self, entries: Sequence[StepEntry]) -> None:
+        vocab = self.vocab_size
+        for entry in entries:
+            for token in entry.tokens:
+                if not 0 <= token < vocab:
+                    raise ValueError(f"request {entry.request!r}: token id {token} is outside the vocabulary of {vocab}")
 
     def context_for(self, entries: Sequence[StepEntry]) -> StepContext:
         if self.check:
-            vocab = self.vocab_size
-            for entry in entries:
-                for token in entry.tokens:
-                    if not 0 <= token < vocab:
-                        raise ValueError(f"request {entry.request!r}: token id {token} is outside the vocabulary of {vocab}")
+            self.check_tokens(entries)
         return build_context(
             entries,
             num_groups=len(self.layout.groups),
@@ -59,9 +74,26 @@ class ModelRunner:
         device = self.model.runtime.device
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
+        if self.graphs is not None and self.graphs.accepts(entries):
+            return self._graph_step(entries)
         ctx = self.context_for(entries)
         stream = self.model.forward(ctx.token_ids, ctx, self.views)
         self.num_steps += 1
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
         return self.model.logits(stream, ctx.logit_rows)
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of single tokens through its recorded graph.  The result is the graph's own
+        buffer (or rows gathered from it): read it before the next step."""
+        if self.check:
+            self.check_tokens(entries)
+            validate_entries(entries, len(self.layout.groups), self.storage.page_size)
+        logits = self.graphs.run(entries)
+        self.num_steps += 1
+        wanted = [i for i, entry in enumerate(entries) if len(entry.want) > 0]
+        if len(wanted) == len(entries):
+            return logits
+        if not wanted:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=logits.device)
+        return logits.index_select(0, torch.tensor(wanted, dtype=torch.long, device=logits.device))

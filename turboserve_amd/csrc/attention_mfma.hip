@@ -226,13 +226,21 @@ __device__ __forceinline__ float column_sum(float l) {
 // decode: grid (splits, kv_heads * head_tiles, requests); one wavefront each.
 // partial_acc [requests, heads, splits, D] float; partial_ml [requests, heads, splits, 2] float.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
               const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
               const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
               const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
               int seq_begin, int heads, int kv_heads, int block_shift, float scale_log2, int window,
-              int keys_per_split, int splits) {
+              int keys_per_split, int splits, const int* __restrict__ max_context) {
+  // A recorded launch serves growing contexts: the longest context of the step is then read
+  // from device memory and the keys are divided evenly over the fixed number of splits.
+  if (max_context) {
+    int span = *max_context;
+    if (window > 0 && span > window + WINDOW_KEYS - 1) span = window + WINDOW_KEYS - 1;
+    const int per = (span + WINDOW_KEYS - 1 + splits - 1) / splits;
+    keys_per_split = ((per + WINDOW_KEYS - 1) / WINDOW_KEYS) * WINDOW_KEYS;
+  }
   const int lane = threadIdx.x;
   const int lane16 = lane & 15;
   const int group = lane >> 4;
@@ -410,11 +418,13 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
 // Decode attention for the requests seq_begin .. seq_begin + requests - 1 of the step, each of
 // which brings one token.  `splits` wavefronts share each request's keys, `keys_per_split`
 // (a multiple of 32) each; partial buffers must hold requests * heads * splits entries.
+// max_context (device, may be null): the step's longest context; when given, keys_per_split is
+// derived from it on the device so that `splits * keys_per_split` covers it.
 extern "C" int TS_SYM(ts_attention_decode_d)(
     void* out, void* partial_acc, void* partial_ml, const void* q, long q_stride, const void* k_pages,
     const void* v_pages, const int* block_table, int table_width, const int* query_start_loc,
     const int* context_lens, int seq_begin, int requests, int heads, int kv_heads, int block_size,
-    float scale, int window, int keys_per_split, int splits, hipStream_t stream) {
+    float scale, int window, int keys_per_split, int splits, const int* max_context, hipStream_t stream) {
   if (requests == 0) return TS_OK;
   if (!out || !partial_acc || !partial_ml || !q || !k_pages || !v_pages || !block_table ||
       !query_start_loc || !context_lens)
@@ -432,7 +442,7 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
   hipLaunchKernelGGL(decode_kernel, grid, dim3(64), 0, stream, (float*)partial_acc, (float*)partial_ml,
                      (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages,
                      block_table, table_width, query_start_loc, context_lens, seq_begin, heads, kv_heads,
-                     shift, scale * LOG2E, window, keys_per_split, splits);
+                     shift, scale * LOG2E, window, keys_per_split, splits, max_context);
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
   hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(64), 0, stream, (uint16_t*)out,
                      (const float*)partial_acc, (const float*)partial_ml, query_start_loc, seq_begin, heads,

@@ -109,6 +109,102 @@ extern "C" int ts_rmsnorm(void* y, const void* x, const void* w, float eps, int 
   return ts_launch_status();
 }
 
+// The same, four elements per thread per item and the row kept in registers between the two
+// passes: for hidden sizes that are a multiple of 4 and at most 16 * blockDim.x.  A decode step
+// has few rows, so each row gets a large block and the loads of all splits are in flight at once.
+template <typename T>
+struct Vec4Of;
+template <>
+struct Vec4Of<float> {
+  typedef float4 type;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <>
+struct Vec4Of<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    uint2 x;
+    x.x = (uint32_t)from_float<bf16_t>(v[0]).bits | ((uint32_t)from_float<bf16_t>(v[1]).bits << 16);
+    x.y = (uint32_t)from_float<bf16_t>(v[2]).bits | ((uint32_t)from_float<bf16_t>(v[3]).bits << 16);
+    *reinterpret_cast<uint2*>(p) = x;
+  }
+};
+
+#define NORM_ITEMS 4
+
+template <typename T, typename P>
+__global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ residual,
+                                        const P* __restrict__ pending, int splits, size_t split_stride,
+                                        const T* __restrict__ w, const int* __restrict__ rows, float eps,
+                                        int hidden) {
+  __shared__ float scratch[16];
+  const int src = rows ? rows[blockIdx.x] : blockIdx.x;
+  const size_t in_base = (size_t)src * hidden;
+  const size_t out_base = (size_t)blockIdx.x * hidden;
+  const int quads = hidden / 4;
+  float s[NORM_ITEMS][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NORM_ITEMS; ++it) {
+    const int qd = threadIdx.x + it * blockDim.x;
+    if (qd < quads) {
+      Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
+      if (pending) {
+        for (int sp = 0; sp < splits; ++sp) {
+          float v[4];
+          Vec4Of<P>::load(pending + sp * split_stride + in_base + 4 * qd, v);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[it][e] += v[e];
+        }
+        if (!rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += s[it][e] * s[it][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+  for (int it = 0; it < NORM_ITEMS; ++it) {
+    const int qd = threadIdx.x + it * blockDim.x;
+    if (qd < quads) {
+      float g[4], o[4];
+      Vec4Of<T>::load(w + 4 * qd, g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = g[e] * round_to<T>(s[it][e] * rstd);
+      Vec4Of<T>::store(y + out_base + 4 * qd, o);
+    }
+  }
+}
+
+template <typename T, typename P>
+static void launch_add_rmsnorm(void* y, float* residual, const void* pending, int splits, long split_stride,
+                               const void* w, const int* rows, float eps, int out_rows, int hidden,
+                               hipStream_t stream) {
+  // Few rows (decode): one large block per row; many rows (prefill): just enough threads.
+  int threads = out_rows <= 256 ? 1024 : 256;
+  const int need = (hidden / 4 + NORM_ITEMS - 1) / NORM_ITEMS;
+  if (threads < need) threads = ((need + 63) / 64) * 64;
+  if (hidden % 4 == 0 && threads <= 1024) {
+    hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
+                       (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden);
+  } else {
+    hipLaunchKernelGGL((add_rmsnorm_kernel<T, P>), dim3(out_rows), dim3(hidden <= 1024 ? 256 : 1024), 0, stream,
+                       (T*)y, residual, (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps,
+                       hidden);
+  }
+}
+
 // `out_rows` = rows of y written: the number of entries of `rows` if given, else the tokens.
 // pending_f32 != 0: `pending` holds `splits` 32-bit partial sums, `split_stride` elements apart.
 extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int pending_f32, int splits,
@@ -116,13 +212,12 @@ extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int
                               int hidden, int dtype, hipStream_t stream) {
   if (out_rows == 0) return TS_OK;
   if (!y || !residual || !w || hidden < 1 || splits < 1) return TS_ERR_ARG;
-  dim3 grid(out_rows), block(hidden <= 1024 ? 256 : 1024);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), grid, block, 0, stream, (float*)y, residual, (const float*)pending, splits, (size_t)split_stride, (const float*)w, rows, eps, hidden);
+    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
   else if (dtype == TS_BF16 && pending_f32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)y, residual, (const float*)pending, splits, (size_t)split_stride, (const bf16_t*)w, rows, eps, hidden);
+    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)y, residual, (const bf16_t*)pending, splits, (size_t)split_stride, (const bf16_t*)w, rows, eps, hidden);
+    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -7,8 +7,8 @@
 // product and its consumer.
 //
 // At these batch sizes the product is bound by reading W once from HBM.  Layout of the work:
-//   * a workgroup of 4 wavefronts owns 64 consecutive weight rows (16 per wavefront) and one
-//     k-range; the grid is (row blocks, splits);
+//   * a workgroup of 4 or 8 wavefronts owns 64 or 128 consecutive weight rows (16 per
+//     wavefront) and one k-range; the grid is (row blocks, splits);
 //   * the k-range is walked in chunks of 256; a lane loads 128 contiguous bytes of its weight
 //     row per chunk (the four lane groups of a row cover 512 contiguous bytes), one chunk
 //     ahead of the matrix cores;
@@ -29,8 +29,6 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int CHUNK = 256;          // k per iteration
 constexpr int STEPS = CHUNK / 32;   // matrix-core steps per chunk
 constexpr int ROWS_PER_WAVE = 16;
-constexpr int WAVES = 4;
-constexpr int ROWS_PER_BLOCK = ROWS_PER_WAVE * WAVES;
 constexpr int X_ROW = CHUNK + 8;    // LDS row stride in elements (16 bytes of padding)
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -58,16 +56,17 @@ __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row
 // The activations of one chunk, X[0..m-1][k0 .. k0+255], travel in two hops: global memory to
 // registers (issued a whole iteration before they are needed), registers to LDS.  A thread
 // carries 2 MT pieces of 16 bytes; rows >= m and k >= K are zeros.
-template <int MT>
+template <int MT, int WAVES>
 struct ActivationRegs {
-  u32x4 piece[2 * MT];
+  static constexpr int PIECES = (MT * 16 * (CHUNK / 8) + WAVES * TS_WAVE - 1) / (WAVES * TS_WAVE);
+  u32x4 piece[PIECES];
 };
 
-template <int MT>
-__device__ __forceinline__ void fetch_activations(ActivationRegs<MT>& r, const uint16_t* __restrict__ x,
+template <int MT, int WAVES>
+__device__ __forceinline__ void fetch_activations(ActivationRegs<MT, WAVES>& r, const uint16_t* __restrict__ x,
                                                   long x_stride, int m, int k0, int k_limit) {
 #pragma unroll
-  for (int i = 0; i < 2 * MT; ++i) {
+  for (int i = 0; i < ActivationRegs<MT, WAVES>::PIECES; ++i) {
     const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
     const int row = idx / (CHUNK / 8);
     const int k = k0 + 8 * (idx % (CHUNK / 8));
@@ -76,12 +75,13 @@ __device__ __forceinline__ void fetch_activations(ActivationRegs<MT>& r, const u
   }
 }
 
-template <int MT>
-__device__ __forceinline__ void store_activations(uint16_t* lds, const ActivationRegs<MT>& r) {
+template <int MT, int WAVES>
+__device__ __forceinline__ void store_activations(uint16_t* lds, const ActivationRegs<MT, WAVES>& r) {
 #pragma unroll
-  for (int i = 0; i < 2 * MT; ++i) {
+  for (int i = 0; i < ActivationRegs<MT, WAVES>::PIECES; ++i) {
     const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
-    *reinterpret_cast<u32x4*>(lds + (idx / (CHUNK / 8)) * X_ROW + 8 * (idx % (CHUNK / 8))) = r.piece[i];
+    if (idx < MT * 16 * (CHUNK / 8))
+      *reinterpret_cast<u32x4*>(lds + (idx / (CHUNK / 8)) * X_ROW + 8 * (idx % (CHUNK / 8))) = r.piece[i];
   }
 }
 
@@ -98,7 +98,7 @@ __device__ __forceinline__ void multiply_chunk(f32x4 (&acc)[MT], const WeightChu
   }
 }
 
-template <int MT>
+template <int MT, int WAVES>
 __global__ void __launch_bounds__(WAVES * TS_WAVE)
 gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
                    const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
@@ -109,7 +109,7 @@ gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, 
   const int lane16 = lane & 15;
   const int group = lane >> 4;
   const int split = blockIdx.y;
-  const int n0 = blockIdx.x * ROWS_PER_BLOCK + wave * ROWS_PER_WAVE;
+  const int n0 = (blockIdx.x * WAVES + wave) * ROWS_PER_WAVE;
   const int total_chunks = (k + CHUNK - 1) / CHUNK;
   const int first = split * chunks_per_split;
   const int last = min(first + chunks_per_split, total_chunks);  // exclusive
@@ -127,28 +127,28 @@ gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, 
     // barrier), `xr` holds chunk c + 1's activations (loads issued a round ago), and the
     // weight registers of this round hold chunk c.
     WeightChunk wa, wb;
-    ActivationRegs<MT> xr;
+    ActivationRegs<MT, WAVES> xr;
     load_weights(wa, wrow, first * CHUNK, group, k);
-    fetch_activations<MT>(xr, x, x_stride, m, first * CHUNK, k);
-    store_activations<MT>(xs[0], xr);
-    if (first + 1 < last) fetch_activations<MT>(xr, x, x_stride, m, (first + 1) * CHUNK, k);
+    fetch_activations<MT, WAVES>(xr, x, x_stride, m, first * CHUNK, k);
+    store_activations<MT, WAVES>(xs[0], xr);
+    if (first + 1 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (first + 1) * CHUNK, k);
     __syncthreads();
     int c = first;
     int buf = 0;
     while (true) {
       if (c + 1 < last) {
-        store_activations<MT>(xs[buf ^ 1], xr);  // free since the last barrier
+        store_activations<MT, WAVES>(xs[buf ^ 1], xr);  // free since the last barrier
         load_weights(wb, wrow, (c + 1) * CHUNK, group, k);
-        if (c + 2 < last) fetch_activations<MT>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
+        if (c + 2 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
       }
       multiply_chunk<MT>(acc, wa, xs[buf], lane16, group);
       __syncthreads();
       if (++c >= last) break;
       buf ^= 1;
       if (c + 1 < last) {
-        store_activations<MT>(xs[buf ^ 1], xr);
+        store_activations<MT, WAVES>(xs[buf ^ 1], xr);
         load_weights(wa, wrow, (c + 1) * CHUNK, group, k);
-        if (c + 2 < last) fetch_activations<MT>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
+        if (c + 2 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
       }
       multiply_chunk<MT>(acc, wb, xs[buf], lane16, group);
       __syncthreads();
@@ -185,28 +185,37 @@ gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, 
 
 }  // namespace
 
+template <int WAVES>
+static int launch_skinny(float* partial, const uint16_t* x, long x_stride, const uint16_t* w, const uint16_t* bias,
+                         int m, int n, int k, int chunks_per_split, int splits, hipStream_t stream) {
+  const int rows_per_block = WAVES * ROWS_PER_WAVE;
+  dim3 grid((n + rows_per_block - 1) / rows_per_block, splits), block(WAVES * TS_WAVE);
+  if (grid.y > 65535) return TS_ERR_SHAPE;
+  if (m <= 16)
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
+  else if (m <= 32)
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
+  else if (m <= 48)
+    hipLaunchKernelGGL((gemm_skinny_kernel<3, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
+  else
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
+  return ts_launch_status();
+}
+
 // partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
 // w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
 // chunks_per_split 256-wide chunks of k go to each of `splits` = ceil(ceil(k / 256) / chunks_per_split).
+// waves: wavefronts (16 weight rows each) per workgroup, 4 or 8.
 extern "C" int ts_gemm_skinny(float* partial, const void* x, long x_stride, const void* w, const void* bias,
-                              int m, int n, int k, int chunks_per_split, int splits, hipStream_t stream) {
+                              int m, int n, int k, int chunks_per_split, int splits, int waves, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
   if (m > 64 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
   const int total_chunks = (k + CHUNK - 1) / CHUNK;
   if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
-  dim3 grid((n + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK, splits), block(WAVES * TS_WAVE);
-  if (grid.y > 65535) return TS_ERR_SHAPE;
-  const uint16_t* xp = (const uint16_t*)x;
-  const uint16_t* wp = (const uint16_t*)w;
-  const uint16_t* bp = (const uint16_t*)bias;
-  if (m <= 16)
-    hipLaunchKernelGGL(gemm_skinny_kernel<1>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
-  else if (m <= 32)
-    hipLaunchKernelGGL(gemm_skinny_kernel<2>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
-  else if (m <= 48)
-    hipLaunchKernelGGL(gemm_skinny_kernel<3>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
-  else
-    hipLaunchKernelGGL(gemm_skinny_kernel<4>, grid, block, 0, stream, partial, xp, x_stride, wp, bp, m, n, k, chunks_per_split);
-  return ts_launch_status();
+  if (waves == 4)
+    return launch_skinny<4>(partial, (const uint16_t*)x, x_stride, (const uint16_t*)w, (const uint16_t*)bias, m, n, k, chunks_per_split, splits, stream);
+  if (waves == 8)
+    return launch_skinny<8>(partial, (const uint16_t*)x, x_stride, (const uint16_t*)w, (const uint16_t*)bias, m, n, k, chunks_per_split, splits, stream);
+  return TS_ERR_SHAPE;
 }

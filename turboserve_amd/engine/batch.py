@@ -65,6 +65,9 @@ class StepContext:
     num_prefill_tokens: int = 0
     max_prefill_context_len: int = 0
     max_decode_context_len: int = 0
+    #: In a recorded (graph) step the host lengths above are upper bounds; the true longest
+    #: context of the single-token requests is this one-element device tensor.
+    max_decode_context_dev: torch.Tensor | None = None
 
 
 def validate_entries(entries: Sequence[StepEntry], num_groups: int, page_size: int) -> None:

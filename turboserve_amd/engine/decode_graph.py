@@ -86,6 +86,7 @@ class DecodeGraphs:
         for name in ("token_ids", "positions", "token_seq", "context_lens", "state_slots", "logit_rows"):
             take(name, batch)
         take("query_start_loc", batch + 1)
+        take("max_context", 1)
         for g, width in enumerate(widths):
             take(f"slots{g}", batch)
             take(f"table{g}", batch * width)
@@ -126,6 +127,7 @@ class DecodeGraphs:
             num_prefill_tokens=0,
             max_prefill_context_len=0,
             max_decode_context_len=max_context,
+            max_decode_context_dev=view("max_context"),
         )
         # Harmless contents for the eager warm-up and the recording: every row is padding.
         shape.device_ints.copy_(self._fill(shape, []))
@@ -170,6 +172,7 @@ class DecodeGraphs:
         field("state_slots")[live:] = self.pad_state_slot
         field("logit_rows")[:] = np.arange(batch, dtype=np.int32)
         field("query_start_loc")[:] = np.arange(batch + 1, dtype=np.int32)
+        field("max_context")[0] = max((e.start + 1 for e in entries), default=1)
         for g, width in enumerate(shape.widths):
             slots = field(f"slots{g}")
             slots[:live] = [e.slots[g][0] for e in entries]

@@ -7,6 +7,7 @@ the library cannot be built or loaded, or a tensor is not on a GPU, the op raise
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_float, c_int, c_long, c_void_p
 
 import torch
@@ -51,7 +52,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                        c_float, c_int, c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
-        "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -62,7 +64,7 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
     return {
         f"ts_attention_decode_d{head_dim}": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
                                              c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                             c_int, c_float, c_int, c_int, c_int, c_void_p],
+                                             c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
         f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float,
                                               c_int, c_void_p],
@@ -358,11 +360,15 @@ class Ops:
         scale: float,
         window: int | None,
         max_context: int,
+        max_context_dev: torch.Tensor | None = None,
     ) -> None:
         """Matrix-core attention for the single-token requests ``seq_begin .. seq_begin +
         requests - 1`` of the step; writes their rows of ``out [T, heads * D]``.  ``max_context``
-        (host-known) bounds their context lengths and sizes the split of the keys."""
-        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens)
+        (host-known) bounds their context lengths and fixes the number of splits of the keys;
+        ``max_context_dev`` (one int32 on the device, at most ``max_context``) is the step's
+        true longest context, from which a recorded launch sizes each split."""
+        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens, max_context_dev)
+        _i32(max_context_dev, "max_context_dev")
         _i32(block_table, "block_table")
         _i32(query_start_loc, "query_start_loc")
         _i32(context_lens, "context_lens")
@@ -389,7 +395,7 @@ class Ops:
         _check(fn(_ptr(out), _ptr(partial_acc), _ptr(partial_ml), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages),
                   _ptr(block_table), block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), seq_begin,
                   requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
-                  self.stream()), "ts_attention_decode")
+                  _ptr(max_context_dev), self.stream()), "ts_attention_decode")
 
     def attention_prefill(
         self,
@@ -464,7 +470,11 @@ class Ops:
         return y
 
     #: Workgroups a skinny product aims for (four per compute unit of a 256-CU device).
-    skinny_target_blocks = 1024
+    skinny_target_blocks = int(os.environ.get("TS_SKINNY_TB", "1024"))
+    #: Most ranges of K a skinny product is split into (its consumer adds them up).
+    skinny_max_splits = int(os.environ.get("TS_SKINNY_MAXS", "8"))
+    #: Wavefronts (16 weight rows each) per workgroup of the skinny product: 4 or 8.
+    skinny_waves = int(os.environ.get("TS_SKINNY_WAVES", "4"))
     #: Largest batch the skinny product serves; above it the BLAS library is used.
     skinny_max_rows = 64
 
@@ -487,13 +497,14 @@ class Ops:
         if bias is not None:
             _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
         chunks = -(-k // 256)
-        row_blocks = -(-n // 64)
-        want = max(1, min(chunks, -(-self.skinny_target_blocks // row_blocks), max_splits or chunks))
+        waves = self.skinny_waves
+        row_blocks = -(-n // (16 * waves))
+        want = max(1, min(chunks, -(-self.skinny_target_blocks // row_blocks), max_splits or self.skinny_max_splits))
         per_split = -(-chunks // want)
         splits = -(-chunks // per_split)
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_skinny(_ptr(partial), _ptr(x), x.stride(0) if m > 1 else max(k, x.stride(0)),
-                                        _ptr(weight), _ptr(bias), m, n, k, per_split, splits, self.stream()),
+                                        _ptr(weight), _ptr(bias), m, n, k, per_split, splits, waves, self.stream()),
                "ts_gemm_skinny")
         return partial
 

@@ -118,6 +118,7 @@ class GroupedQueryAttention(Mixer):
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     ctx.num_prefill_seqs, ctx.num_decode_seqs, self.num_heads, self.scale, self.window,
                     min(ctx.max_decode_context_len, table.shape[1] * cache.block_size),
+                    ctx.max_decode_context_dev,
                 )
             return out
         return ops.paged_attention_generic(

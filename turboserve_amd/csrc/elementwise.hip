@@ -243,18 +243,56 @@ __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up
   out[idx] = from_float<T>(act * u);
 }
 
+// Four outputs per thread with 8- or 16-byte loads: for I a multiple of 4.
+template <typename T, typename P>
+__global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
+                                   size_t split_stride, int inter, size_t quads) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= quads) return;
+  const int per_row = inter / 4;
+  const size_t t = idx / per_row;
+  const int i = (int)(idx - t * per_row) * 4;
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < splits; ++sp) {
+    float a[4], b[4];
+    Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + i, a);
+    Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + inter + i, b);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      g[e] += a[e];
+      u[e] += b[e];
+    }
+  }
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  Vec4Of<T>::store(out + t * inter + i, o);
+}
+
+template <typename T, typename P>
+static void launch_swiglu(void* out, const void* gate_up, int splits, long split_stride, int tokens, int inter,
+                          hipStream_t stream) {
+  if (inter % 4 == 0) {
+    const size_t quads = (size_t)tokens * (inter / 4);
+    hipLaunchKernelGGL((swiglu_vec4_kernel<T, P>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+                       (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads);
+  } else {
+    const size_t total = (size_t)tokens * inter;
+    hipLaunchKernelGGL((swiglu_kernel<T, P>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (T*)out,
+                       (const P*)gate_up, splits, (size_t)split_stride, inter, total);
+  }
+}
+
 extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits, long split_stride,
                          int tokens, int inter, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !gate_up || inter < 1 || splits < 1) return TS_ERR_ARG;
-  const size_t total = (size_t)tokens * inter;
-  dim3 block(256), grid((unsigned)((total + 255) / 256));
   if (dtype == TS_F32)
-    hipLaunchKernelGGL((swiglu_kernel<float, float>), grid, block, 0, stream, (float*)out, (const float*)gate_up, splits, (size_t)split_stride, inter, total);
+    launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, stream);
   else if (dtype == TS_BF16 && in_f32)
-    hipLaunchKernelGGL((swiglu_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)out, (const float*)gate_up, splits, (size_t)split_stride, inter, total);
+    launch_swiglu<bf16_t, float>(out, gate_up, splits, split_stride, tokens, inter, stream);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL((swiglu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)gate_up, splits, (size_t)split_stride, inter, total);
+    launch_swiglu<bf16_t, bf16_t>(out, gate_up, splits, split_stride, tokens, inter, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

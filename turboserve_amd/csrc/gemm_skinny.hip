@@ -9,15 +9,15 @@
 // At these batch sizes the product is bound by reading W once from HBM.  Layout of the work:
 //   * a workgroup of 4 or 8 wavefronts owns 64 or 128 consecutive weight rows (16 per
 //     wavefront) and one k-range; the grid is (row blocks, splits);
-//   * the k-range is walked in chunks of 256; a lane loads 128 contiguous bytes of its weight
-//     row per chunk (the four lane groups of a row cover 512 contiguous bytes), one chunk
+//   * the k-range is walked in chunks of 256: eight loads per lane, each of which has the four
+//     lane groups of a weight row cover 64 contiguous bytes (so a load instruction touches 16
+//     rows x 64 bytes, and the eight of a chunk 512 contiguous bytes per row), issued one chunk
 //     ahead of the matrix cores;
 //   * the chunk's activations are staged once per workgroup in LDS (rows padded against bank
 //     conflicts) and read as B operands by all four wavefronts; they are fetched from global
 //     memory into registers two chunks ahead and written to LDS one chunk ahead;
-//   * v_mfma_f32_16x16x32_bf16 with A = 16 weight rows, B = 16 activation rows; k index 8 g + e
-//     of step j stands for k = chunk + 64 g + 8 j + e on both operands, which is what makes the
-//     per-lane loads contiguous.
+//   * v_mfma_f32_16x16x32_bf16 with A = 16 weight rows, B = 16 activation rows, step j of a
+//     chunk covering k = chunk + 32 j .. + 31.
 #include "common.hpp"
 
 namespace {
@@ -34,20 +34,20 @@ constexpr int X_ROW = CHUNK + 8;    // LDS row stride in elements (16 bytes of p
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
 struct WeightChunk {
-  u32x4 piece[STEPS];  // k = chunk + 64 g + 8 j .. + 7 of the lane's row, j = 0..7
+  u32x4 piece[STEPS];  // k = chunk + 32 j + 8 g .. + 7 of the lane's row, j = 0..7
 };
 
 // `row` points at the lane's weight row; k_limit = K: pieces at or beyond it read as zero
 // (K is a multiple of 8, so a piece is wholly inside or wholly outside).
 __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row, int k0, int group, int k_limit) {
-  const int base = k0 + 64 * group;
+  const int base = k0 + 8 * group;
   if (k0 + CHUNK <= k_limit) {
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) w.piece[j] = *reinterpret_cast<const u32x4*>(row + base + 8 * j);
+    for (int j = 0; j < STEPS; ++j) w.piece[j] = *reinterpret_cast<const u32x4*>(row + base + 32 * j);
   } else {
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
-      const int k = base + 8 * j;
+      const int k = base + 32 * j;
       w.piece[j] = (k < k_limit) ? *reinterpret_cast<const u32x4*>(row + k) : u32x4{0u, 0u, 0u, 0u};
     }
   }
@@ -92,7 +92,7 @@ __device__ __forceinline__ void multiply_chunk(f32x4 (&acc)[MT], const WeightChu
   for (int j = 0; j < STEPS; ++j) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const u32x4 b = *reinterpret_cast<const u32x4*>(xs + (16 * t + lane16) * X_ROW + 64 * group + 8 * j);
+      const u32x4 b = *reinterpret_cast<const u32x4*>(xs + (16 * t + lane16) * X_ROW + 8 * group + 32 * j);
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w.piece[j]), as_bf16x8(b), acc[t], 0, 0, 0);
     }
   }

@@ -94,19 +94,61 @@ __device__ __forceinline__ int block_argmax(const float* __restrict__ row, int v
   return best_i == 0x7fffffff ? 0 : best_i;
 }
 
-__global__ void __launch_bounds__(SAMPLE_THREADS)
-argmax_kernel(int* __restrict__ tokens, const float* __restrict__ logits, int vocab) {
+// Greedy rows in two stages, so that a handful of rows still spreads over the device: stage one
+// finds the best (value, lowest index) of each slice of the vocabulary, stage two of each row.
+#define ARGMAX_SLICES 64
+#define ARGMAX_THREADS 256
+
+__global__ void __launch_bounds__(ARGMAX_THREADS)
+argmax_slices_kernel(float* __restrict__ slice_value, int* __restrict__ slice_index,
+                     const float* __restrict__ logits, int vocab) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
-  const float* row = logits + (size_t)blockIdx.x * vocab;
-  const int best = block_argmax(row, vocab, fscratch, iscratch);
-  if (threadIdx.x == 0) tokens[blockIdx.x] = best;
+  const int row = blockIdx.y;
+  const int per = (vocab + ARGMAX_SLICES - 1) / ARGMAX_SLICES;
+  const int begin = blockIdx.x * per;
+  const int count = min(per, vocab - begin);
+  float best_value = -INFINITY;
+  int best = 0x7fffffff;
+  if (count > 0) {
+    const int local = block_argmax(logits + (size_t)row * vocab + begin, count, fscratch, iscratch);
+    best = begin + local;
+    best_value = logits[(size_t)row * vocab + best];
+  }
+  if (threadIdx.x == 0) {
+    slice_value[row * ARGMAX_SLICES + blockIdx.x] = best_value;
+    slice_index[row * ARGMAX_SLICES + blockIdx.x] = best;
+  }
 }
 
-extern "C" int ts_argmax(int* tokens, const float* logits, int rows, int vocab, hipStream_t stream) {
+__global__ void __launch_bounds__(ARGMAX_SLICES)
+argmax_rows_kernel(int* __restrict__ tokens, const float* __restrict__ slice_value,
+                   const int* __restrict__ slice_index) {
+  const int row = blockIdx.x;
+  float v = slice_value[row * ARGMAX_SLICES + threadIdx.x];
+  int i = slice_index[row * ARGMAX_SLICES + threadIdx.x];
+#pragma unroll
+  for (int off = TS_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off, TS_WAVE);
+    const int oi = __shfl_xor(i, off, TS_WAVE);
+    if (oi != 0x7fffffff && (i == 0x7fffffff || ov > v || (ov == v && oi < i))) {
+      v = ov;
+      i = oi;
+    }
+  }
+  if (threadIdx.x == 0) tokens[row] = (i == 0x7fffffff) ? 0 : i;
+}
+
+// scratch: rows * 64 floats followed by rows * 64 ints.
+extern "C" int ts_argmax(int* tokens, const float* logits, void* scratch, int rows, int vocab, hipStream_t stream) {
   if (rows == 0) return TS_OK;
-  if (!tokens || !logits || vocab < 1) return TS_ERR_ARG;
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, tokens, logits, vocab);
+  if (!tokens || !logits || !scratch || vocab < 1 || rows > 65535) return TS_ERR_ARG;
+  float* values = (float*)scratch;
+  int* indices = (int*)(values + (size_t)rows * ARGMAX_SLICES);
+  hipLaunchKernelGGL(argmax_slices_kernel, dim3(ARGMAX_SLICES, rows), dim3(ARGMAX_THREADS), 0, stream, values,
+                     indices, logits, vocab);
+  if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(ARGMAX_SLICES), 0, stream, tokens, values, indices);
   return ts_launch_status();
 }
 

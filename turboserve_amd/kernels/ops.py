@@ -54,7 +54,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                           c_int, c_int, c_void_p],
         "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_void_p],
-        "ts_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
@@ -540,8 +540,9 @@ class Ops:
         _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(),
               "logits must be contiguous float32 [n, V]")
         tokens = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-        _check(self.core.ts_argmax(_ptr(tokens), _ptr(logits), logits.shape[0], logits.shape[1], self.stream()),
-               "ts_argmax")
+        scratch = torch.empty((logits.shape[0], 128), dtype=torch.int32, device=logits.device)
+        _check(self.core.ts_argmax(_ptr(tokens), _ptr(logits), _ptr(scratch), logits.shape[0], logits.shape[1],
+                                   self.stream()), "ts_argmax")
         return tokens
 
     def sample(

@@ -11,7 +11,6 @@ otherwise; ``H`` hidden size; ``Hq``/``Hkv`` query/KV heads; ``D`` head size.
 
 from __future__ import annotations
 
-import math
 from collections.abc import Mapping, Sequence
 
 import torch
@@ -276,16 +275,11 @@ _PHILOX_W1 = 0xBB67AE85
 _MASK32 = 0xFFFFFFFF
 
 
-def philox_uniform(seed: int, index: int) -> float:
-    """Uniform in ``[0, 1)`` from Philox-4x32-10 (Salmon et al. 2011), keyed by ``seed``.
-
-    Counter ``(index, 0, 0, 0)``, key ``(seed & 2^32-1, seed >> 32)``; the result is the top
-    24 bits of the first output word times ``2^-24``.  This is the engine's own rule (the
-    reference draws with ``torch.multinomial``, core/sampler.py:285-296, whose stream a kernel
-    cannot reproduce); it is restated here from the published algorithm.
-    """
-    c = [index & _MASK32, (index >> 32) & _MASK32, 0, 0]
-    k0, k1 = seed & _MASK32, (seed >> 32) & _MASK32
+def philox4x32_10(counter: Sequence[int], key: Sequence[int]) -> list[int]:
+    """The Philox-4x32-10 block function (Salmon et al., "Parallel random numbers: as easy as
+    1, 2, 3", 2011): four 32-bit words out for a four-word counter and a two-word key."""
+    c = [int(v) & _MASK32 for v in counter]
+    k0, k1 = int(key[0]) & _MASK32, int(key[1]) & _MASK32
     for _ in range(10):
         p0 = _PHILOX_M0 * c[0]
         p1 = _PHILOX_M1 * c[2]
@@ -297,7 +291,19 @@ def philox_uniform(seed: int, index: int) -> float:
         ]
         k0 = (k0 + _PHILOX_W0) & _MASK32
         k1 = (k1 + _PHILOX_W1) & _MASK32
-    return (c[0] >> 8) * (1.0 / 16777216.0)
+    return c
+
+
+def philox_uniform(seed: int, index: int) -> float:
+    """Uniform in ``[0, 1)`` for a request's ``index``-th draw.
+
+    Counter ``(index, 0, 0, 0)``, key ``(seed & 2^32-1, seed >> 32)``; the result is the top
+    24 bits of the first output word times ``2^-24``.  This is the engine's own rule (the
+    reference draws with ``torch.multinomial``, core/sampler.py:285-296, whose stream a kernel
+    cannot reproduce).
+    """
+    words = philox4x32_10((index & _MASK32, 0, 0, 0), (seed & _MASK32, (seed >> 32) & _MASK32))
+    return (words[0] >> 8) * (1.0 / 16777216.0)
 
 
 def repetition_penalty(logits: torch.Tensor, history: Sequence[int], penalty: float) -> torch.Tensor:
@@ -386,7 +392,3 @@ def expected_kv_bytes_per_token(cfg: Mapping, itemsize: int) -> int:
     """``2 * L * Hkv * D * itemsize`` (model_config.py:234-242)."""
     values = cfg_values(cfg)
     return 2 * values["layers"] * values["kv_heads"] * values["head_dim"] * itemsize
-
-
-def isclose_angle(a: float, b: float) -> bool:
-    return math.isclose(a, b, rel_tol=1e-6, abs_tol=1e-6)

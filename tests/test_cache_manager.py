@@ -1,0 +1,193 @@
+"""The host side of the cache: page pools, block tables, groups with windows, state slots.
+No page is lost, held twice or freed twice, under random orders of requests."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+import torch
+
+from turboserve_amd.cache.allocator import InvalidPageError, OutOfPagesError, PageAllocator
+from turboserve_amd.cache.layout import CacheLayout
+from turboserve_amd.cache.manager import PAD_PAGE, CacheManager
+from turboserve_amd.cache.sizing import MemoryProfileError, size_cache, window_pages_needed
+from turboserve_amd.cache.state_slots import OutOfStateSlotsError, StateSlotPool
+from turboserve_amd.config.engine_config import SchedulerConfig
+from turboserve_amd.parts.base import FixedState, PagedKV
+
+
+def test_allocator_states_and_fifo_reuse():
+    """tests/unit/test_kv_cache_storage.py:75-127 in the reference."""
+    pool = PageAllocator(4, 16)
+    pages = pool.allocate_many(3)
+    assert pages == [0, 1, 2] and pool.num_free == 1 and pool.num_in_use == 3
+    pool.decref(1)
+    pool.decref(0)
+    pool.check_invariants()
+    assert [pool.allocate(), pool.allocate(), pool.allocate()] == [3, 1, 0]  # least recently freed first
+    with pytest.raises(OutOfPagesError):
+        pool.allocate()
+    with pytest.raises(OutOfPagesError):  # all or nothing
+        PageAllocator(2, 4).allocate_many(3)
+    pool.decref(2)
+    with pytest.raises(InvalidPageError, match="double free"):
+        pool.decref(2)
+    with pytest.raises(InvalidPageError, match="outside the pool"):
+        pool.decref(9)
+    assert pool.incref(3) == 2 and pool.decref(3) == 1 and pool.refcount(3) == 1  # shared pages are counted
+    with pytest.raises(InvalidPageError, match="free"):
+        pool.incref(2)
+    pool.reset()
+    assert pool.num_free == 4
+    pool.check_invariants()
+
+
+def test_slots_are_page_major_and_pages_come_as_tokens_do():
+    """tests/unit/test_block_manager.py:76-101: slot = page * page_size + offset; pages are taken
+    portion by portion, not at admission."""
+    manager = CacheManager([None], 8, 4, 2)
+    held = manager.admit("a")
+    assert held.tables == [[]] and manager.pools[0].num_in_use == 0
+    assert manager.append("a", 6) == [[0, 1, 2, 3, 4, 5]]
+    assert held.tables == [[0, 1]] and held.num_tokens == 6
+    manager.admit("b")
+    assert manager.append("b", 3) == [[8, 9, 10]]
+    assert manager.append("a", 3) == [[6, 7, 12]]  # a's third page is page 3
+    assert manager.get("a").tables == [[0, 1, 3]]
+    manager.check_invariants()
+    manager.free("a")
+    assert manager.pools[0].num_in_use == 1 and not manager.has("a")
+    with pytest.raises(KeyError):
+        manager.free("a")
+    with pytest.raises(ValueError, match="already holds"):
+        manager.admit("b")
+    manager.admit("c")
+    assert manager.append("c", 9) == [[p * 4 + o for p in (4, 5, 6) for o in range(4)][:9]]  # FIFO: freed pages come last
+    manager.check_invariants()
+
+
+def test_running_out_of_pages_is_all_or_nothing():
+    manager = CacheManager([None, None], [3, 2], 4, 4)
+    manager.admit("a")
+    assert manager.can_append("a", 8) and not manager.can_append("a", 9)  # the second group holds 8 tokens
+    assert manager.pages_short("a", 12) == [0, 1]
+    with pytest.raises(OutOfPagesError):
+        manager.append("a", 12)
+    assert manager.pools[0].num_in_use == 0 and manager.pools[1].num_in_use == 0  # nothing was taken
+    manager.append("a", 8)
+    assert not manager.can_append("a", 1)
+    assert manager.fits_pool(8, 8) and not manager.fits_pool(9, 8)
+    assert not manager.can_admit(4, 4)  # no page of group 1 is free
+    manager.check_invariants()
+
+
+def test_window_groups_give_pages_back_while_the_request_runs():
+    """Group 0 keeps every key, group 1 a window of 6: pages wholly below the next query's
+    window go back to the pool and their table entries become PAD_PAGE."""
+    manager = CacheManager([None, 6], [16, 4], 4, 2)
+    manager.admit("a")
+    manager.append("a", 10)  # positions 0..9
+    assert manager.get("a").tables[1] == [0, 1, 2]
+    manager.append("a", 1)  # query at 10 sees keys 5..10: page 0 (keys 0..3) is passed
+    assert manager.get("a").tables[1][0] == PAD_PAGE and manager.pools[1].num_in_use == 2
+    for _ in range(30):
+        manager.append("a", 1)
+        manager.check_invariants()
+    table = manager.get("a").tables[1]
+    assert len(table) == 11 and table.count(PAD_PAGE) == 8 and manager.pools[1].num_in_use == 3
+    assert len(manager.get("a").tables[0]) == 11 and PAD_PAGE not in manager.get("a").tables[0]
+    assert manager.peak_pages(1, 1000, 1) == 3 and manager.peak_pages(0, 1000, 1) == 250
+    assert manager.peak_pages(1, 5, 64) == 2  # a short request needs no more than its own pages
+    assert manager.fits_pool(10_000, 1) is False and CacheManager([6], 4, 4, 1).fits_pool(10_000, 1)
+    manager.free("a")
+    assert manager.pools[1].num_in_use == 0 and manager.pools[0].num_in_use == 0
+    # A portion larger than the window: its own keys must all stay until it has run.
+    manager.admit("b")
+    manager.append("b", 3)
+    manager.append("b", 9)  # queries 3..11; the first sees keys from 0
+    assert PAD_PAGE not in manager.get("b").tables[1]
+
+
+def test_state_slots():
+    pool = StateSlotPool(2)
+    a, b = pool.allocate(), pool.allocate()
+    assert {a, b} == {0, 1} and pool.num_free == 0
+    with pytest.raises(OutOfStateSlotsError):
+        pool.allocate()
+    pool.free(a)
+    with pytest.raises(ValueError):
+        pool.free(a)
+    assert pool.allocate() == a
+    pool.check_invariants()
+    manager = CacheManager([None], 8, 4, 1)
+    manager.admit("a")
+    assert not manager.can_admit(1, 1)  # pages are free, the slot is not
+    manager.free("a")
+    assert manager.can_admit(1, 1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_never_lose_or_share_a_page(seed):
+    rng = random.Random(seed)
+    windows = [None, rng.choice([5, 8, 16])]
+    manager = CacheManager(windows, [rng.randrange(6, 14), rng.randrange(4, 10)], rng.choice([2, 4, 8]), 4)
+    live: list[int] = []
+    counter = 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.25 and len(live) < 4 and manager.can_admit(1, 8):
+            manager.admit(counter)
+            live.append(counter)
+            counter += 1
+        elif action < 0.85 and live:
+            request = rng.choice(live)
+            n = rng.randrange(1, 9)
+            before = manager.get(request).num_tokens
+            if manager.can_append(request, n):
+                slots = manager.append(request, n)
+                for g in range(2):
+                    table = manager.get(request).tables[g]
+                    size = manager.page_size
+                    assert slots[g] == [table[p // size] * size + p % size for p in range(before, before + n)]
+            else:
+                with pytest.raises(OutOfPagesError):
+                    manager.append(request, n)
+                assert manager.get(request).num_tokens == before
+        elif live:
+            manager.free(live.pop(rng.randrange(len(live))))
+        manager.check_invariants()
+        held = [page for entry in manager._requests.values() for page in entry.tables[1] if page != PAD_PAGE]
+        assert len(held) == len(set(held))
+    for request in live:
+        manager.free(request)
+    assert all(pool.num_in_use == 0 for pool in manager.pools) and manager.state_slots.num_free == 4
+
+
+def test_layout_groups_layers_by_their_needs():
+    full, window, state = PagedKV(2, 8), PagedKV(2, 8, 16), FixedState((4, 3))
+    layout = CacheLayout.from_needs([full, window, None, window, state, None, full], [None, None, None, None, None, 1, None])
+    assert [(g.window, g.entries) for g in layout.groups] == [(None, (0, 6)), (16, (1, 3))]
+    assert layout.entry_units == (("pages", 0, 0), ("pages", 1, 0), None, ("pages", 1, 1), ("state", 0), ("reads", 1), ("pages", 0, 1))
+    assert layout.state_entries == ((4, state),) and layout.windows() == [None, 16]
+    # tests/unit/test_kv_cache_storage.py:267-305: 2 layers, pages of 4, 2 heads of 8, 32-bit: 1024 bytes a page.
+    two = CacheLayout.from_needs([full, full], [None, None])
+    assert two.bytes_per_page(4, 4) == [1024] and two.bytes_per_token(4) == 256
+
+
+def test_sizing():
+    layout = CacheLayout.from_needs([PagedKV(2, 8)] * 2, [None, None])
+    scheduler = SchedulerConfig(block_size=4, max_num_batched_tokens=8, max_num_seqs=2)
+    sizing = size_cache(layout, scheduler, itemsize=4, memory=(10_000, 10_000), gpu_memory_utilization=1.0)
+    assert sizing.num_blocks == [9] and sizing.kv_bytes == 9216 and sizing.reason == "memory budget"  # floor(10000 / 1024)
+    capped = size_cache(layout, scheduler, itemsize=4, memory=(10**6, 10**6), max_model_len=10)
+    assert capped.num_blocks == [6] and capped.reason == "max_model_len cap"  # ceil(10 / 4) * 2 requests
+    explicit = size_cache(layout, SchedulerConfig(block_size=4, max_num_batched_tokens=8, num_blocks=5), itemsize=4)
+    assert explicit.num_blocks == [5] and explicit.reason == "explicit num_blocks"
+    with pytest.raises(MemoryProfileError):
+        size_cache(layout, scheduler, itemsize=4, memory=(500, 10_000))
+    mixed = CacheLayout.from_needs([PagedKV(2, 8), PagedKV(2, 8, 16)], [None, None])
+    both = size_cache(mixed, scheduler, itemsize=4, memory=(10**5, 10**5), gpu_memory_utilization=1.0)
+    assert both.num_blocks[1] == window_pages_needed(16, scheduler) == 14
+    assert both.num_blocks[0] == (10**5 - 14 * 512) // 512
+    assert torch.cuda.is_available() or True

@@ -1,0 +1,294 @@
+"""The parts of a model, alone and recombined: each built-in part against the plain
+implementation; a toy mixer with state of its own and a toy architecture, defined here and
+registered without touching the framework; a run order that names a layer twice and lets a
+layer read another layer's cache; long decoding and the first tokens of a sequence."""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+import tiny
+import trace_helpers as th
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def make_runtime(dtype):
+    from turboserve_amd.engine.loading import make_runtime
+
+    return make_runtime(dtype, DEV)
+
+
+def assert_matches(got: torch.Tensor, want: torch.Tensor, dtype) -> None:
+    """32-bit: 1e-4 absolute.  bfloat16 against the plain implementation in 32-bit: relative to
+    the largest value, the criterion of the replay tests."""
+    worst = float((got - want).abs().max())
+    bound = 1e-4 if dtype == torch.float32 else 2e-2 * float(want.abs().max())
+    assert worst <= bound, f"max |diff| {worst:.3e} > {bound:.3e}"
+
+
+def one_request_context(tokens: int, page: int, start: int = 0, groups: int = 1):
+    """A step context for one request bringing ``tokens`` tokens at ``start``, pages 0, 1, ..."""
+    from turboserve_amd.engine.batch import StepEntry, build_context
+
+    pages = list(range(-(-(start + tokens) // page)))
+    slots = [pages[p // page] * page + p % page for p in range(start, start + tokens)]
+    entry = StepEntry(request="r", tokens=[0] * tokens, start=start, tables=[pages] * groups, slots=[slots] * groups,
+                      want=list(range(tokens)))
+    return build_context([entry], num_groups=groups, page_size=page, device=DEV)
+
+
+# -- built-in parts alone ----------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from turboserve_amd.parts.base import PartSpec, ResidualStream
+    from turboserve_amd.parts.registry import build_part
+
+    runtime = make_runtime(dtype)
+    norm = build_part("norm", PartSpec("rmsnorm", {"size": 72, "eps": 3e-6}), "n", runtime)
+    assert list(norm.tensor_specs()) == ["n.weight"] and norm.tensor_specs()["n.weight"].init == "ones"
+    g = torch.Generator().manual_seed(0)
+    w = (1 + 0.1 * torch.randn(72, generator=g)).to(dtype)
+    norm.load({"n.weight": w.to(DEV)})
+    x = torch.randn(5, 72, generator=g).to(dtype)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(norm.forward(x.to(DEV)).float().cpu(), plain.rms_norm(x.float(), w.float(), 3e-6), **tol)
+    stream = ResidualStream(torch.randn(5, 72, generator=g).to(DEV), x.to(DEV))
+    before = stream.residual.clone()
+    y = norm.forward_residual(stream)
+    assert stream.pending is None
+    torch.testing.assert_close(stream.residual.cpu(), before.cpu() + x.float(), rtol=0, atol=1e-6)
+    torch.testing.assert_close(y.float().cpu(), plain.rms_norm(before.cpu() + x.float(), w.float(), 3e-6), **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_and_feed_forward_and_block_parts(dtype, window):
+    """One attention mixer, one SwiGLU and one pre-norm block built from specs with sizes of
+    their own (not a model's), stepped in two portions, against the plain functions."""
+    from turboserve_amd.parts.base import PagedKVView, PartSpec, ResidualStream
+    from turboserve_amd.parts.registry import build_part
+
+    runtime = make_runtime(dtype)
+    hidden, heads, kv_heads, dim, inter, page, eps = 48, 6, 2, 16, 40, 8, 1e-5
+    position = PartSpec("rope", {"head_dim": dim, "theta": 5000.0, "scaling_factor": 1.0, "max_positions": 64})
+    mixer_spec = PartSpec("gqa_attention", {
+        "hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": dim, "scale": dim ** -0.5,
+        "qkv_bias": True, "out_bias": False, "window": window, "position": position})
+    ff_spec = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter})
+    norm_spec = PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    block = build_part("block", PartSpec("prenorm", {"mixer": mixer_spec, "feed_forward": ff_spec,
+                                                     "mixer_norm": norm_spec, "ff_norm": norm_spec}), "model.layers.0", runtime)
+    from turboserve_amd.parts.base import PagedKV
+
+    assert block.mixer.cache_need() == PagedKV(kv_heads, dim, window)
+    g = torch.Generator().manual_seed(1)
+    tensors = {}
+    for name, spec in block.tensor_specs().items():
+        t = torch.ones(spec.shape) + 0.1 * torch.randn(spec.shape, generator=g) if spec.init == "ones" else 0.2 * torch.randn(spec.shape, generator=g)
+        tensors[name] = t.to(dtype)
+    block.load({k: v.to(DEV) for k, v in tensors.items()})
+    cfg = {"hidden_size": hidden, "num_hidden_layers": 1, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+           "head_dim": dim, "intermediate_size": inter, "vocab_size": 8, "rms_norm_eps": eps, "rope_theta": 5000.0,
+           "use_sliding_window": window is not None, "sliding_window": window, "max_window_layers": 0}
+    values = plain.cfg_values(cfg)
+    ftensors = {k: v.float() for k, v in tensors.items()}
+    tokens = 13
+    h = torch.randn(tokens, hidden, generator=g).to(dtype)
+    want = plain.decoder_layer(h.float(), ftensors, 0, values, torch.arange(tokens))
+    kpages = torch.zeros(4, kv_heads, page, dim, dtype=dtype, device=DEV)
+    vpages = torch.zeros(4, kv_heads, dim, page, dtype=dtype, device=DEV)
+    cache = PagedKVView(kpages, vpages, group=0, block_size=page, window=window)
+    got = []
+    for start, count in ((0, 9), (9, 4)):
+        ctx = one_request_context(count, page, start)
+        stream = block.forward(ResidualStream(h[start:start + count].float().to(DEV)), ctx, cache)
+        total = stream.residual + runtime.ops.dense(stream.pending, dtype).float()
+        got.append(total.cpu())
+    assert_matches(torch.cat(got), want, dtype)
+    # the mixer alone, and the feed-forward alone
+    x = plain.rms_norm(h.float(), ftensors["model.layers.0.input_layernorm.weight"], eps)
+    attn_want = plain.attention_block(x, ftensors, "model.layers.0.self_attn", values, torch.arange(tokens), window)
+    ctx = one_request_context(tokens, page)
+    kpages.zero_(); vpages.zero_()
+    attn = runtime.ops.dense(block.mixer.forward(x.to(dtype).to(DEV), ctx, cache), dtype).float().cpu()
+    assert_matches(attn, attn_want, dtype)
+    ff_want = plain.swiglu_mlp(x, *(ftensors[f"model.layers.0.mlp.{p}_proj.weight"] for p in ("gate", "up", "down")))
+    ff = runtime.ops.dense(block.feed_forward.forward(x.to(dtype).to(DEV), ctx), dtype).float().cpu()
+    assert_matches(ff, ff_want, dtype)
+
+
+# -- a toy mixer with state of its own, and a toy architecture ---------------------------------------
+
+
+def register_toy_architecture():
+    """Everything a new mixer and a new architecture need, using only the public registries."""
+    from turboserve_amd.config import registry as arch_registry
+    from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
+    from turboserve_amd.parts import registry as part_registry
+    from turboserve_amd.parts.base import FixedState, Mixer, PartSpec, TensorSpec
+
+    if "running_mean" not in part_registry.MIXERS:
+
+        @part_registry.register_mixer("running_mean")
+        class RunningMean(Mixer):
+            """out_t = W * mean(x_0 .. x_t): per request a running sum [H] and a count."""
+
+            def __init__(self, prefix, runtime, *, hidden_size):
+                super().__init__(prefix, runtime)
+                self.hidden = hidden_size
+                self.weight = None
+
+            def cache_need(self):
+                return FixedState((self.hidden + 1,), torch.float32)
+
+            def tensor_specs(self):
+                return {self.name("mix.weight"): TensorSpec((self.hidden, self.hidden))}
+
+            def load(self, tensors):
+                self.weight = tensors[self.name("mix.weight")]
+
+            def forward(self, x, ctx, cache):
+                out = torch.empty_like(x)
+                row = 0
+                for s, count in enumerate(ctx.query_lens):
+                    slot = ctx.state_slots[s:s + 1].long()
+                    state = cache.state.index_select(0, slot)[0]
+                    sums = state[: self.hidden] + torch.cumsum(x[row:row + count].float(), dim=0)
+                    counts = state[self.hidden] + torch.arange(1, count + 1, device=x.device, dtype=torch.float32)
+                    mean = (sums / counts[:, None]).to(x.dtype)
+                    out[row:row + count] = mean @ self.weight.t()
+                    cache.state.index_copy_(0, slot, torch.cat((sums[-1], counts[-1:]))[None])
+                    row += count
+                return out
+
+    if "ToyForCausalLM" not in arch_registry.ARCHITECTURES:
+
+        def parse(data, name_or_path=""):
+            return dict(data)
+
+        def plan(cfg):
+            hidden = cfg["hidden_size"]
+            norm = PartSpec("rmsnorm", {"size": hidden, "eps": cfg["eps"]})
+            ff = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": cfg["intermediate_size"]})
+            attention = PartSpec("gqa_attention", {
+                "hidden_size": hidden, "num_heads": cfg["heads"], "num_kv_heads": cfg["kv_heads"], "head_dim": cfg["head_dim"],
+                "scale": cfg["head_dim"] ** -0.5, "qkv_bias": True, "out_bias": False, "window": None,
+                "position": PartSpec("rope", {"head_dim": cfg["head_dim"], "theta": 1e4, "scaling_factor": 1.0, "max_positions": 256})})
+            toy = PartSpec("running_mean", {"hidden_size": hidden})
+            layers = []
+            for index, kind in enumerate(cfg["mixers"]):  # the mixer is chosen layer by layer
+                block = PartSpec("prenorm", {"mixer": attention if kind == "attention" else toy, "feed_forward": ff,
+                                             "mixer_norm": norm, "ff_norm": norm})
+                layers.append(LayerSpec(f"model.layers.{index}", block))
+            schedule = tuple(LayerCall(layer, cache_of) for layer, cache_of in cfg["schedule"])
+            return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=hidden, layers=tuple(layers), schedule=schedule,
+                             final_norm=norm, tie_head=True)
+
+        arch_registry.register_architecture("ToyForCausalLM", parse, plan)
+
+
+def toy_plain_logits(cfg, tensors, tokens):
+    """The toy model by the plain functions: whole sequence, no cache."""
+    values = {"heads": cfg["heads"], "kv_heads": cfg["kv_heads"], "head_dim": cfg["head_dim"], "theta": 1e4,
+              "rope_factor": 1.0, "eps": cfg["eps"]}
+    h = tensors["model.embed_tokens.weight"][torch.tensor(tokens)]
+    pos = torch.arange(len(tokens))
+    kv_of_call = {}
+    for call, (layer, cache_of) in enumerate(cfg["schedule"]):
+        p = f"model.layers.{layer}"
+        x = plain.rms_norm(h, tensors[f"{p}.input_layernorm.weight"], cfg["eps"])
+        if cfg["mixers"][layer] == "attention":
+            heads, kvh, dim = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+            angles = plain.rope_angles(pos, dim, 1e4)
+            q = (x @ tensors[f"{p}.self_attn.q_proj.weight"].T + tensors[f"{p}.self_attn.q_proj.bias"]).view(-1, heads, dim)
+            q = plain.apply_rope(q, angles)
+            if cache_of is None:
+                k = (x @ tensors[f"{p}.self_attn.k_proj.weight"].T + tensors[f"{p}.self_attn.k_proj.bias"]).view(-1, kvh, dim)
+                v = (x @ tensors[f"{p}.self_attn.v_proj.weight"].T + tensors[f"{p}.self_attn.v_proj.bias"]).view(-1, kvh, dim)
+                kv_of_call[call] = (plain.apply_rope(k, angles), v)
+            k, v = kv_of_call[call if cache_of is None else cache_of]
+            mixed = plain.attention(q, k, v, plain.attention_mask(pos, len(tokens), None), dim ** -0.5)
+            mixed = mixed.reshape(len(tokens), -1) @ tensors[f"{p}.self_attn.o_proj.weight"].T
+        else:
+            mean = torch.cumsum(x, dim=0) / torch.arange(1, len(tokens) + 1)[:, None]
+            mixed = mean @ tensors[f"{p}.self_attn.mix.weight"].T
+        h = h + mixed
+        x = plain.rms_norm(h, tensors[f"{p}.post_attention_layernorm.weight"], cfg["eps"])
+        h = h + plain.swiglu_mlp(x, *(tensors[f"{p}.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+    h = plain.rms_norm(h, tensors["model.norm.weight"], cfg["eps"])
+    return h @ tensors["model.embed_tokens.weight"].T
+
+
+TOY_CONFIG = {
+    "architectures": ["ToyForCausalLM"], "hidden_size": 40, "intermediate_size": 56, "vocab_size": 97, "heads": 5,
+    "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "mixers": ["attention", "state", "attention"],
+    # layer 0, the stateful layer, layer 0 AGAIN (weights reused, a cache of its own), then
+    # layer 2 reading the cache of the first call instead of keeping one.
+    "schedule": [[0, None], [1, None], [0, None], [2, 0]],
+}
+
+
+@pytest.fixture(scope="module")
+def toy_folder(tmp_path_factory):
+    from turboserve_amd.weights.random_init import write_random_model
+
+    register_toy_architecture()
+    return write_random_model(TOY_CONFIG, tmp_path_factory.mktemp("toy"), seed=5, dtype=torch.float32)
+
+
+def test_toy_model_is_data(toy_folder):
+    from turboserve_amd.cache.layout import CacheLayout
+    from turboserve_amd.weights.random_init import describe_model
+
+    _, model = describe_model(TOY_CONFIG)
+    layout = CacheLayout.from_model(model)
+    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads"]
+    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2) and layout.state_entries[0][0] == 1
+    names = list(model.tensor_specs())
+    assert "model.layers.1.self_attn.mix.weight" in names and "model.layers.2.self_attn.q_proj.weight" in names
+
+
+@pytest.mark.parametrize("cut", ["whole", "prefix_then_single", "portions", "mixed"])
+def test_toy_architecture_steps_like_its_plain_form(toy_folder, cut):
+    """Registered, built, loaded and stepped through the ordinary replay path under every
+    cutting: the state slot carries the running mean across steps, padded graph rows and
+    requests that end and free their slot for the next one."""
+    from test_gpu_replay import CUTS, run_trace
+
+    register_toy_architecture()
+    raw, tensors = tiny.read_model_dir(toy_folder)
+    requests = {f"t{i}": tiny.random_tokens(97, n, 300 + i) for i, n in enumerate([9, 41, 23, 60, 34])}
+    steps = CUTS[cut](requests)
+    got = th.collect(steps, run_trace(toy_folder, "float32", 8, steps), requests)
+    for rid, toks in requests.items():
+        want = toy_plain_logits(raw, tensors, toks)
+        assert float((got[rid] - want).abs().max()) <= 1e-4, f"{cut} {rid}"
+
+
+# -- long decoding, first tokens ----------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(tmp_path, dtype):
+    """A request that starts from a single token and is decoded token by token for 300 steps
+    (through a window of 40 keys and pages of 32 that are given back on the way)."""
+    from test_gpu_replay import check, run_trace
+
+    config, seed, page = tiny.TINY["C"]
+    folder = tiny.make_model_dir(tmp_path, config, seed, torch.float32 if dtype == "float32" else torch.bfloat16)
+    tokens = tiny.random_tokens(config["vocab_size"], 301, 77)
+    steps = [{"step": i, "entries": [{"id": "long", "tokens": [t], "want": [0]}], "end": ["long"] if i == 300 else []}
+             for i, t in enumerate(tokens)]
+    outputs = run_trace(folder, dtype, page, steps, max_tokens=320)
+    got = th.collect(steps, outputs, {"long": tokens})
+    check(got, {"long": tiny.plain_logits(folder, tokens)}, dtype, "long decoding")

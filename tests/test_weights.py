@@ -1,0 +1,150 @@
+"""Weights by tensor name: discovery, name mapping, conversion and the one error that lists
+everything that does not fit (the reference's cases: tests/unit/test_model_config.py:229-420)."""
+
+from __future__ import annotations
+
+import json
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+import tiny
+from turboserve_amd.parts.base import TensorSpec
+from turboserve_amd.weights.loader import (
+    WeightLoadError,
+    iter_checkpoint_tensors,
+    load_model_weights,
+    load_tensors,
+    map_weight_name,
+    resolve_model_dir,
+    safetensors_files,
+)
+from turboserve_amd.weights.random_init import describe_model, draw_tensors, write_random_model
+
+
+def cpu_model(config):
+    _, model = describe_model(config)
+    return model
+
+
+def test_name_map():
+    assert map_weight_name("model.layers.0.self_attn.q_proj.weight") == "model.layers.0.self_attn.q_proj.weight"
+    assert map_weight_name("transformer.layers.1.mlp.up_proj.weight") == "model.layers.1.mlp.up_proj.weight"
+    assert map_weight_name("language_model.model.norm.weight") == "model.norm.weight"
+    assert map_weight_name("language_model.lm_head.weight") == "lm_head.weight"
+    assert map_weight_name("model.decoder.embed_tokens.weight") == "model.embed_tokens.weight"
+    assert map_weight_name("model.layers.0.self_attn.rotary_emb.inv_freq") is None
+    assert map_weight_name("h.0.attn.masked_bias") is None
+
+
+def test_expected_tensor_names_are_the_checkpoint_contract():
+    config, _, _ = tiny.TINY["B"]
+    names = list(cpu_model(config).tensor_specs())
+    assert names[0] == "model.embed_tokens.weight" and names[-1] == "lm_head.weight" and names[-2] == "model.norm.weight"
+    layer0 = [n for n in names if n.startswith("model.layers.0.")]
+    assert set(layer0) == {f"model.layers.0.{s}" for s in (
+        "input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.q_proj.bias", "self_attn.k_proj.weight",
+        "self_attn.k_proj.bias", "self_attn.v_proj.weight", "self_attn.v_proj.bias", "self_attn.o_proj.weight",
+        "post_attention_layernorm.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight")}
+    specs = cpu_model(config).tensor_specs()
+    assert specs["model.layers.2.self_attn.k_proj.weight"].shape == (32, 96)
+    assert specs["model.layers.2.mlp.down_proj.weight"].shape == (96, 200)
+    tied = cpu_model(tiny.TINY["A"][0])
+    assert "lm_head.weight" not in tied.tensor_specs() and tied.ignorable_names() == {"lm_head.weight"}
+    assert tied.num_parameters() == 90688  # incl. the tied embedding once
+    assert cpu_model(config).num_parameters() == 309120
+
+
+def test_shard_discovery(tmp_path):
+    with pytest.raises(WeightLoadError, match="no safetensors"):
+        safetensors_files(tmp_path)
+    (tmp_path / "pytorch_model.bin").write_bytes(b"x")
+    with pytest.raises(WeightLoadError, match="pickle"):
+        safetensors_files(tmp_path)
+    save_file({"a": torch.zeros(1)}, str(tmp_path / "model-00002-of-00002.safetensors"))
+    save_file({"b": torch.zeros(1)}, str(tmp_path / "model-00001-of-00002.safetensors"))
+    assert [p.name for p in safetensors_files(tmp_path)] == ["model-00001-of-00002.safetensors", "model-00002-of-00002.safetensors"]
+    index = {"weight_map": {"b": "model-00001-of-00002.safetensors", "a": "model-00002-of-00002.safetensors",
+                            "c": "model-00003-of-00003.safetensors"}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(WeightLoadError, match="absent"):
+        safetensors_files(tmp_path)
+    del index["weight_map"]["c"]
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    assert len(safetensors_files(tmp_path)) == 2
+    assert dict(iter_checkpoint_tensors(safetensors_files(tmp_path))).keys() == {"a", "b"}
+    with pytest.raises(WeightLoadError, match="is a file"):
+        resolve_model_dir(tmp_path / "pytorch_model.bin")
+    with pytest.raises(WeightLoadError, match="does not exist"):
+        resolve_model_dir(tmp_path / "missing")
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    config, seed, _ = tiny.TINY["A"]
+    folder = write_random_model(config, tmp_path, seed=seed)
+    tensors = load_file(str(folder / "model.safetensors"))
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.extra.weight"] = torch.zeros(3)
+    tensors["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(65)
+    tensors["model.embed_tokens.weight"] = torch.zeros(256, 64, dtype=torch.int64)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)  # derived: skipped silently
+    save_file(tensors, str(folder / "model.safetensors"))
+    model = cpu_model(config)
+    with pytest.raises(WeightLoadError) as err:
+        load_model_weights(model, folder)
+    text = str(err.value)
+    assert "missing (2)" in text and "model.layers.1.mlp.up_proj.weight" in text and "model.norm.weight" in text
+    assert "unexpected (1)" in text and "model.layers.0.extra.weight" in text
+    assert "wrong shape (1)" in text and "model has (64,), checkpoint has (65,)" in text
+    assert "wrong type (1)" in text and "model.embed_tokens.weight" in text
+    assert "inv_freq" not in text
+
+
+def test_conversion_rules():
+    specs = {"w": TensorSpec((2, 2)), "keep": TensorSpec((2,), kind="float_keep32"), "half": TensorSpec((2,), kind="float_keep32"),
+             "table": TensorSpec((3,), kind="int")}
+    source = [("w", torch.ones(2, 2, dtype=torch.float32)), ("keep", torch.ones(2, dtype=torch.float32)),
+              ("half", torch.ones(2, dtype=torch.float16)), ("table", torch.tensor([1, 2, 3], dtype=torch.int64))]
+    out, report = load_tensors(specs, iter(source), dtype=torch.bfloat16, device="cpu")
+    assert report.ok and out["w"].dtype == torch.bfloat16  # weights are kept in the run's dtype
+    assert out["keep"].dtype == torch.float32  # stored in 32-bit: stays so
+    assert out["half"].dtype == torch.bfloat16
+    assert out["table"].dtype == torch.int32 and out["table"].tolist() == [1, 2, 3]
+    out32, _ = load_tensors(specs, iter(source), dtype=torch.float32, device="cpu")
+    assert out32["w"].dtype == torch.float32 and out32["half"].dtype == torch.float32
+
+
+def test_tied_checkpoint_may_carry_the_head(tmp_path):
+    config, seed, _ = tiny.TINY["A"]
+    folder = write_random_model(config, tmp_path, seed=seed)
+    tensors = load_file(str(folder / "model.safetensors"))
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    save_file(tensors, str(folder / "model.safetensors"))
+    model = cpu_model(config)
+    report = load_model_weights(model, folder)
+    assert report.ok and report.ignored == ["lm_head.weight"]
+    assert model.head is model.embedding
+
+
+def test_random_model_is_a_function_of_config_and_seed(tmp_path):
+    config, _, _ = tiny.TINY["B"]
+    a = load_file(str(write_random_model(config, tmp_path / "a", seed=3) / "model.safetensors"))
+    b = load_file(str(write_random_model(config, tmp_path / "b", seed=3) / "model.safetensors"))
+    c = load_file(str(write_random_model(config, tmp_path / "c", seed=4) / "model.safetensors"))
+    assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
+    assert not torch.equal(a["model.layers.0.self_attn.q_proj.bias"], c["model.layers.0.self_attn.q_proj.bias"])
+    assert torch.equal(a["model.norm.weight"], torch.ones(96))
+    assert float(a["model.layers.1.self_attn.k_proj.bias"].abs().max()) > 0  # biases are drawn, not zero
+    assert abs(float(a["model.embed_tokens.weight"].std()) - 0.02) < 0.002
+    assert json.loads((tmp_path / "a" / "config.json").read_text())["torch_dtype"] == "float32"
+    half = load_file(str(write_random_model(config, tmp_path / "h", seed=3, dtype=torch.bfloat16) / "model.safetensors"))
+    assert all(t.dtype == torch.bfloat16 for t in half.values())
+    assert torch.equal(half["lm_head.weight"], a["lm_head.weight"].bfloat16())  # same draws, rounded
+    model = cpu_model(config)
+    assert [name for name, _ in draw_tensors(model.tensor_specs(), 3)] == list(model.tensor_specs())
+    load_model_weights(model, tmp_path / "a")
+    assert model.blocks[0].mixer.qkv_weight.shape == (96 + 2 * 32, 96)  # q, k, v fused at load
+    assert torch.equal(model.blocks[0].mixer.qkv_weight[96:128], a["model.layers.0.self_attn.k_proj.weight"])
+    assert model.blocks[2].feed_forward.gate_up_weight.shape == (400, 96)

@@ -10,7 +10,9 @@ The default run has the 7B shape of BASELINE.json's configs[2], random weights
 (cache filled with random keys and values; what is timed is real decode steps on top of it).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times one
 2,048-token prompt; ``roofline`` prices the decode step against HBM bandwidth; ``points``
-holds decode at batch 1 and 64.  Peaks are the published MI355X figures: HBM 8 TB/s, dense
+holds decode at batch 1 and 64.  The prefill's projections are BLAS-library products; which
+of the library's kernels runs each is timed once before the measurement
+(``--no-gemm-tuning`` leaves it to the library's heuristic).  Peaks are the published MI355X figures: HBM 8 TB/s, dense
 bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
 """
 
@@ -18,7 +20,9 @@ from __future__ import annotations
 
 import argparse
 import json
+import os
 import sys
+import tempfile
 import time
 
 HBM_PEAK_GBS = 8000.0
@@ -57,6 +61,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--no-gemm-tuning", action="store_true",
+                   help="leave the choice of the BLAS library's prefill kernels to its heuristic")
     p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     return p.parse_args()
 
@@ -145,9 +151,11 @@ def prefill_flops(config, layers: int, tokens: int) -> float:
     return 2.0 * tokens * linear + attention + 2.0 * config.vocab_size * h
 
 
-def run_prefill(model, config, tokens: int, repeats: int = 3) -> float:
+def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True) -> float:
     """Seconds (best of ``repeats``) for one step over a ``tokens``-long prompt, to its last
-    position's logits on the host."""
+    position's logits on the host.  With ``tune`` the BLAS library's kernels for the step's
+    products are timed first in a dry step and the fastest kept, as an engine started with
+    ``tune_gemm_tokens`` does."""
     import torch
 
     from turboserve_amd.cache.manager import CacheManager
@@ -159,6 +167,11 @@ def run_prefill(model, config, tokens: int, repeats: int = 3) -> float:
     storage = build_storage(model, num_pages, PAGE, 1)
     manager = CacheManager(storage.layout.windows(), num_pages, PAGE, 1)
     runner = ModelRunner(model, storage, check=False)
+    if tune and model.runtime.dtype == torch.bfloat16:
+        from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
+
+        with LibraryGemmTuning(os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")):
+            runner.dry_run(tokens)
     generator = torch.Generator().manual_seed(4321)
     prompt = torch.randint(0, config.vocab_size, (tokens,), generator=generator).tolist()
     best = float("inf")
@@ -210,7 +223,7 @@ def main() -> int:
         return batch * steps / seconds, seconds / steps
 
     if args.only_prefill:
-        seconds = run_prefill(model, config, PREFILL_TOKENS)
+        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=not args.no_gemm_tuning)
         print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}))
         return 0
 
@@ -249,6 +262,7 @@ def main() -> int:
             "tie_word_embeddings": config.tie_word_embeddings,
             "page_size": PAGE,
             "prefill_tokens": PREFILL_TOKENS,
+            "prefill_gemm_choice": "library heuristic" if args.no_gemm_tuning else "library candidates timed at start-up",
             "sampling": "greedy",
         },
         "roofline": {
@@ -260,7 +274,7 @@ def main() -> int:
         },
     }
     if not args.no_prefill:
-        seconds = run_prefill(model, config, PREFILL_TOKENS)
+        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=not args.no_gemm_tuning)
         flops = prefill_flops(config, layers, PREFILL_TOKENS)
         result["prefill"] = {
             "value": round(PREFILL_TOKENS / seconds, 1),

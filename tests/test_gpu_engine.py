@@ -164,3 +164,35 @@ def test_decode_graphs_replay_like_eager(model):
                 assert replayer.runner.graphs.num_replays == 12
         for eager, graph in zip(results[(dtype, False)], results[(dtype, True)]):
             assert torch.equal(eager, graph), f"{dtype}: a graph replay differs from the eager step"
+
+
+def test_timed_library_products_and_the_dry_step(model, tmp_path):
+    """An engine asked to time the BLAS library's kernels at start-up: the dry step it runs for
+    that leaves every cache page as it was, the choices are written to the given file, and a
+    prompt longer than the skinny product's 64 rows (so that the library computes its
+    projections) still gives the plain implementation's log-probabilities."""
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    results = tmp_path / "choices.csv"
+    prompt = tiny.random_tokens(model["vocab"], 100, 77)
+    engine = LLMEngine(EngineConfig(
+        model=str(model["folder"]), dtype="bfloat16", tune_gemm_tokens=(100,), gemm_tuning_file=str(results),
+        scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=128, block_size=model["page"], num_blocks=32),
+    ))
+    try:
+        assert results.exists() and "Gemm" in results.read_text()
+        assert not torch.cuda.tunable.tuning_is_enabled()  # nothing is timed once the engine serves
+        before = [t.clone() for t in engine.storage.pages]
+        engine.runner.dry_run(70)
+        assert all(torch.equal(a, b) for a, b in zip(before, engine.storage.pages))
+        out = engine.generate([prompt], SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True, logprobs=True))[0]
+    finally:
+        engine.close()
+        torch.cuda.tunable.enable(False)
+    sequence = prompt + out.new_token_ids
+    logits = plain.forward_logits(model["raw"], plain.as_float32(model["tensors"]), sequence)
+    for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
+        want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
+        assert abs(got - want) <= 0.05, (i, got, want)

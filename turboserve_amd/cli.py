@@ -30,6 +30,8 @@ def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> Non
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--max-num-seqs", type=int, default=max_num_seqs)
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    p.add_argument("--tune-gemm", action="store_true",
+                   help="time the BLAS library's kernels for a full step of prompt tokens at start-up and keep the fastest")
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -84,6 +86,7 @@ def _generate(args: argparse.Namespace) -> int:
         return 2
     config = EngineConfig(
         model=args.model, device=args.device, dtype=args.dtype, seed=args.seed,
+        tune_gemm_tokens=(args.max_num_batched_tokens,) if args.tune_gemm else (),
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
             block_size=args.block_size, num_blocks=args.num_blocks,

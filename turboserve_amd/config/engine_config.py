@@ -47,6 +47,12 @@ class EngineConfig:
     max_model_len: int | None = None
     seed: int | None = None
     scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
+    #: Step sizes (tokens) at which the BLAS library's kernels for this model's projections are
+    #: timed at start-up and the fastest kept (bfloat16 only; a few seconds per size).  Empty:
+    #: the library's own heuristic picks.  No counterpart in the reference.
+    tune_gemm_tokens: tuple[int, ...] = ()
+    #: Where the timed choices are kept between runs; None is a per-user cache file.
+    gemm_tuning_file: str | None = None
 
     def __post_init__(self) -> None:
         if self.dtype not in ("auto", "bfloat16", "float32"):
@@ -57,6 +63,9 @@ class EngineConfig:
             raise ValueError(f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization!r}")
         if self.max_model_len is not None and self.max_model_len < 1:
             raise ValueError(f"max_model_len must be >= 1, got {self.max_model_len!r}")
+        self.tune_gemm_tokens = tuple(self.tune_gemm_tokens)
+        if any(isinstance(t, bool) or not isinstance(t, int) or t < 1 for t in self.tune_gemm_tokens):
+            raise ValueError(f"tune_gemm_tokens must be ints >= 1, got {self.tune_gemm_tokens!r}")
 
     @property
     def block_size(self) -> int:

@@ -183,6 +183,96 @@ gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, 
   }
 }
 
+
+// The same product for M <= 16 with the activations resident in LDS: a workgroup stages its
+// split's activations X[0..mpad-1][k-range] once (in stretches of `stage_chunks` chunks when
+// the range is longer than LDS should hold) and its wavefronts then stream their weight rows
+// without meeting at a barrier again, two chunks of loads in flight each.  mpad is 8 or 16;
+// lanes whose activation row is beyond mpad read a real row again and drop the result.
+template <int WAVES>
+__global__ void __launch_bounds__(WAVES * TS_WAVE)
+gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
+                            const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int mpad,
+                            int n, int k, int chunks_per_split, int stage_chunks) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t xs_resident[];
+  const int lane = threadIdx.x & (TS_WAVE - 1);
+  const int wave = threadIdx.x / TS_WAVE;
+  const int lane16 = lane & 15;
+  const int group = lane >> 4;
+  const int split = blockIdx.y;
+  const int n0 = (blockIdx.x * WAVES + wave) * ROWS_PER_WAVE;
+  const int total_chunks = (k + CHUNK - 1) / CHUNK;
+  const int first = split * chunks_per_split;
+  const int last = min(first + chunks_per_split, total_chunks);  // exclusive
+
+  const int row_index = min(n0 + lane16, n - 1);
+  const uint16_t* wrow = w + (size_t)row_index * k;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+
+  if (first < last) {
+    const int stage = min(stage_chunks, last - first);  // chunks per stretch; even unless it is the whole range
+    const int x_row = stage * CHUNK + 8;                 // LDS row stride in elements
+    const int pieces_per_row = stage * (CHUNK / 8);
+    const uint16_t* xl = xs_resident + (lane16 % mpad) * x_row + 8 * group;
+    WeightChunk wa, wb;
+    load_weights(wa, wrow, first * CHUNK, group, k);
+    if (first + 1 < last) load_weights(wb, wrow, (first + 1) * CHUNK, group, k);
+    for (int begin = first; begin < last; begin += stage) {
+      const int end = min(begin + stage, last);
+      if (begin != first) __syncthreads();  // everyone has read the previous stretch
+      const int k_begin = begin * CHUNK;
+      const int live_pieces = (end - begin) * (CHUNK / 8);
+      for (int idx = threadIdx.x; idx < mpad * pieces_per_row; idx += WAVES * TS_WAVE) {
+        const int row = idx / pieces_per_row;
+        const int piece = idx - row * pieces_per_row;
+        if (piece >= live_pieces) continue;
+        const int kk = k_begin + 8 * piece;
+        const u32x4 v = (row < m && kk < k) ? *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + kk)
+                                            : u32x4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4*>(xs_resident + row * x_row + 8 * piece) = v;
+      }
+      __syncthreads();
+      // A stretch other than the last has an even number of chunks, so it starts on `wa`.
+      for (int c = begin; c < end; c += 2) {
+        const uint16_t* xc = xl + (c - begin) * CHUNK;
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) {
+          const u32x4 b = *reinterpret_cast<const u32x4*>(xc + 32 * j);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa.piece[j]), as_bf16x8(b), acc, 0, 0, 0);
+        }
+        if (c + 2 < last) load_weights(wa, wrow, (c + 2) * CHUNK, group, k);
+        if (c + 1 >= end) break;
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) {
+          const u32x4 b = *reinterpret_cast<const u32x4*>(xc + CHUNK + 32 * j);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb.piece[j]), as_bf16x8(b), acc, 0, 0, 0);
+        }
+        if (c + 3 < last) load_weights(wb, wrow, (c + 3) * CHUNK, group, k);
+      }
+    }
+  }
+
+  // acc[i] = sum for weight row n0 + 4 g + i and activation row lane16.
+  const int nrow = n0 + 4 * group;
+  if (nrow < n && lane16 < m) {
+    f32x4 b = {0.f, 0.f, 0.f, 0.f};
+    if (bias && split == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nrow + i < n) b[i] = to_float(bf16_t{bias[nrow + i]});
+    }
+    float* dst = partial + ((size_t)split * m + lane16) * n + nrow;
+    const f32x4 v = acc + b;
+    if (nrow + 3 < n && (n & 3) == 0) {
+      *reinterpret_cast<f32x4*>(dst) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nrow + i < n) dst[i] = v[i];
+    }
+  }
+}
+
 }  // namespace
 
 template <int WAVES>
@@ -218,4 +308,35 @@ extern "C" int ts_gemm_skinny(float* partial, const void* x, long x_stride, cons
   if (waves == 8)
     return launch_skinny<8>(partial, (const uint16_t*)x, x_stride, (const uint16_t*)w, (const uint16_t*)bias, m, n, k, chunks_per_split, splits, stream);
   return TS_ERR_SHAPE;
+}
+
+// The variant for m <= 16 that keeps a split's activations in LDS (see the kernel).  stage_chunks:
+// chunks staged at a time, an even number unless it covers a whole split; the LDS it needs,
+// mpad * (min(stage_chunks, chunks_per_split) * 256 + 8) * 2 bytes with mpad = 8 or 16, must be <= 64 KiB.
+extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
+                                       int m, int n, int k, int chunks_per_split, int splits, int waves,
+                                       int stage_chunks, hipStream_t stream) {
+  if (m == 0 || n == 0) return TS_OK;
+  if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
+  if (m > 16 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
+  const int total_chunks = (k + CHUNK - 1) / CHUNK;
+  if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
+  if (stage_chunks < 1 || (stage_chunks < chunks_per_split && (stage_chunks & 1) != 0)) return TS_ERR_SHAPE;
+  const int mpad = m <= 8 ? 8 : 16;
+  const int stage = stage_chunks < chunks_per_split ? stage_chunks : chunks_per_split;
+  const size_t lds = (size_t)mpad * (stage * CHUNK + 8) * sizeof(uint16_t);
+  if (lds > 64 * 1024 || splits > 65535) return TS_ERR_SHAPE;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* bp = (const uint16_t*)bias;
+  if (waves == 4) {
+    dim3 grid((n + 63) / 64, splits), block(4 * TS_WAVE);
+    hipLaunchKernelGGL((gemm_skinny_resident_kernel<4>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks);
+  } else if (waves == 8) {
+    dim3 grid((n + 127) / 128, splits), block(8 * TS_WAVE);
+    hipLaunchKernelGGL((gemm_skinny_resident_kernel<8>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks);
+  } else {
+    return TS_ERR_SHAPE;
+  }
+  return ts_launch_status();
 }

@@ -86,6 +86,8 @@ class LLMEngine:
         self.scheduler = scheduler
         self.runner = runner if runner is not None else ModelRunner(model, storage)
         self.sampler = sampler if sampler is not None else Sampler(model.runtime.ops)
+        if config.tune_gemm_tokens and runner is None:
+            self._tune_library_products()
         self._decoders: dict[str, StreamingDecoder] = {}
         self._seed = config.seed if config.seed is not None else time.time_ns() & 0xFFFFFFFF
         self._num_generated_tokens = 0
@@ -93,6 +95,22 @@ class LLMEngine:
         self._closed = False
 
     # -- helpers --------------------------------------------------------------------------------
+
+    def _tune_library_products(self) -> None:
+        """Time the BLAS library's kernels for this model's projections at the configured step
+        sizes (dry steps that leave the cache alone) and keep the fastest."""
+        if self.model.runtime.dtype != torch.bfloat16:
+            return  # the 32-bit path uses this engine's own product kernel
+        from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
+
+        budget = self.config.scheduler.max_num_batched_tokens
+        started = time.perf_counter()
+        with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
+            for tokens in sorted({min(t, budget) for t in self.config.tune_gemm_tokens}):
+                self.runner.dry_run(tokens)
+        logger.info("library products timed for steps of %s tokens in %.1f s (%d choices kept in %s)",
+                    list(self.config.tune_gemm_tokens), time.perf_counter() - started, tuning.num_results(),
+                    tuning.results_file)
 
     def _resolve_eos_token_ids(self) -> frozenset[int]:
         """The checkpoint's end-of-sequence ids (engine.py:223-237)."""

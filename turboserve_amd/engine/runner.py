@@ -83,6 +83,23 @@ class ModelRunner:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
         return self.model.logits(stream, ctx.logit_rows)
 
+    @torch.inference_mode()
+    def dry_run(self, num_tokens: int) -> None:
+        """One step of a made-up prompt of ``num_tokens`` tokens that writes nothing into the
+        cache (every slot is the skip mark) and whose result is dropped: it makes every product
+        of the model run once at that size, for warming up or for timing the library's kernels."""
+        page = self.storage.page_size
+        groups = len(self.layout.groups)
+        entry = StepEntry(
+            request="dry-run", tokens=[0] * num_tokens, start=0,
+            tables=[[0] * (-(-num_tokens // page))] * groups, slots=[[-1] * num_tokens] * groups,
+            state_slot=self.storage.pad_state_slot, want=[num_tokens - 1],
+        )
+        ctx = build_context([entry], num_groups=groups, page_size=page, device=self.model.runtime.device, check=False)
+        stream = self.model.forward(ctx.token_ids, ctx, self.views)
+        self.model.logits(stream, ctx.logit_rows)
+        torch.cuda.synchronize(self.model.runtime.device)
+
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """A step of single tokens through its recorded graph.  The result is the graph's own
         buffer (or rows gathered from it): read it before the next step."""

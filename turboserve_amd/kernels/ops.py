@@ -54,6 +54,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                           c_int, c_int, c_void_p],
         "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_void_p],
+        "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -477,6 +479,14 @@ class Ops:
     skinny_waves = int(os.environ.get("TS_SKINNY_WAVES", "4"))
     #: Largest batch the skinny product serves; above it the BLAS library is used.
     skinny_max_rows = 64
+    #: Up to this many rows the skinny product keeps a split's activations resident in LDS.
+    skinny_resident_rows = int(os.environ.get("TS_SKINNY_RROWS", "16"))
+    #: Wavefronts (16 weight rows x one range of K each) the resident variant aims for: 16 per compute unit.
+    skinny_resident_waves = int(os.environ.get("TS_SKINNY_RW", "4096"))
+    #: Wavefronts per workgroup of the resident variant (4 or 8); 0 chooses by the grid's size.
+    skinny_resident_wg = int(os.environ.get("TS_SKINNY_RWG", "0"))
+    #: Chunks of 256 staged in LDS at a time for up to 8 rows and for up to 16 rows (even numbers).
+    skinny_stage_chunks = tuple(int(v) for v in os.environ.get("TS_SKINNY_STAGE", "10,4").split(","))
 
     @staticmethod
     def skinny_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -497,13 +507,27 @@ class Ops:
         if bias is not None:
             _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
         chunks = -(-k // 256)
+        x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
+        if m <= self.skinny_resident_rows:
+            # Activations resident in LDS, no barrier per chunk: splits sized for a number of wavefronts.
+            limit = min(chunks, max_splits or self.skinny_max_splits)
+            want = max(1, min(limit, -(-self.skinny_resident_waves // -(-n // 16))))
+            per_split = -(-chunks // want)
+            splits = -(-chunks // per_split)
+            waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 1024) else 4)
+            stage = self.skinny_stage_chunks[0 if m <= 8 else 1]
+            partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+            _check(self.core.ts_gemm_skinny_resident(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias),
+                                                     m, n, k, per_split, splits, waves, stage, self.stream()),
+                   "ts_gemm_skinny_resident")
+            return partial
         waves = self.skinny_waves
         row_blocks = -(-n // (16 * waves))
         want = max(1, min(chunks, -(-self.skinny_target_blocks // row_blocks), max_splits or self.skinny_max_splits))
         per_split = -(-chunks // want)
         splits = -(-chunks // per_split)
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-        _check(self.core.ts_gemm_skinny(_ptr(partial), _ptr(x), x.stride(0) if m > 1 else max(k, x.stride(0)),
+        _check(self.core.ts_gemm_skinny(_ptr(partial), _ptr(x), x_stride,
                                         _ptr(weight), _ptr(bias), m, n, k, per_split, splits, waves, self.stream()),
                "ts_gemm_skinny")
         return partial

@@ -315,6 +315,8 @@ ATTENTION_GEOMETRIES = [
     (8, 1, 64, 16),
     (40, 2, 80, 16),    # G = 20: more than one tile of heads per KV head
     (2, 1, 256, 64),
+    (6, 2, 256, 16),    # G = 3 at the largest head size: staged windows above 64 KiB of LDS
+    (10, 2, 48, 8),     # G = 5, a head size that is no multiple of 32
 ]
 
 

@@ -60,8 +60,44 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef u32x4 Frag8;  // 8 bfloat16
 typedef u32x2 Frag4;  // 4 bfloat16
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ uint32_t bf16_bits(float v) { return from_float<bf16_t>(v).bits; }
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) { return bf16_bits(lo) | (bf16_bits(hi) << 16); }
+// Two floats rounded to nearest-even bfloat16 in one word (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
+// 2^x by the hardware instruction alone: results below the smallest normal number flush to
+// zero, which is what a softmax weight that small is worth.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Reductions of a column's value over the four lane groups (lanes l, l ^ 16, l ^ 32, l ^ 48)
+// with the row-swap instructions of gfx950: no trip through LDS.
+__device__ __forceinline__ void swap_rows(float v, bool halves, float& a, float& b) {
+  const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+  const u32x2 r = halves ? __builtin_amdgcn_permlane32_swap(bits, bits, false, false)
+                         : __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  // Elements go through scalars first: __builtin_bit_cast applied to `r[1]` directly reads
+  // element 0 with this compiler.
+  const uint32_t first = r[0], second = r[1];
+  a = __builtin_bit_cast(float, first);
+  b = __builtin_bit_cast(float, second);
+}
+__device__ __forceinline__ float groups_max(float v) {
+  float a, b;
+  swap_rows(v, false, a, b);
+  v = fmaxf(a, b);
+  swap_rows(v, true, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float groups_sum(float v) {
+  float a, b;
+  swap_rows(v, false, a, b);
+  v = a + b;
+  swap_rows(v, true, a, b);
+  return a + b;
+}
 __device__ __forceinline__ bf16x8 as_bf16x8(Frag8 f) { return __builtin_bit_cast(bf16x8, f); }
 __device__ __forceinline__ Frag8 load8(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 
@@ -85,48 +121,82 @@ struct PageGeometry {
   const uint16_t* k_pages;
   const uint16_t* v_pages;
   const int* table;  // this request's block table
+  int table_width;
   int kv_heads;
   int kvh;
   int block_shift;  // log2(block size)
   int block_mask;
 };
 
+// The pages that hold the keys w .. w + 31 of a 32-aligned window: 32 / block size of them (one
+// when a block holds 32 keys or more).  `w` is the same in every lane, so these are scalar
+// loads: they do not queue behind the vector loads of the windows in flight, which a per-lane
+// table lookup would have to wait for before it could form an address.  Entries past the
+// table's width are never selected (the keys they would hold are past the context).
+struct WindowPages {
+  int page[4];
+};
+
+__device__ __forceinline__ WindowPages window_pages(const PageGeometry& g, int w) {
+  WindowPages wp;
+  const int first = __builtin_amdgcn_readfirstlane(w) >> g.block_shift;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) wp.page[i] = g.table[min(first + i, g.table_width - 1)];
+  return wp;
+}
+
+// Page of `key`, a key of the window starting at w (a block of 32 keys or more: always the first).
+__device__ __forceinline__ long long page_of(const PageGeometry& g, const WindowPages& wp, int w, int key) {
+  const int i = (key - w) >> g.block_shift;
+  return i == 0 ? wp.page[0] : (i == 1 ? wp.page[1] : (i == 2 ? wp.page[2] : wp.page[3]));
+}
+
+// A key outside lo..last is replaced by the nearest live key of its window (every window that
+// is processed holds one): loads stay unconditional and inside live pages, so they can be
+// issued windows ahead; what they bring is masked in the softmax.
+__device__ __forceinline__ int live_key(int key, int w, int lo, int last) {
+  return min(max(key, max(w, lo)), min(w + WINDOW_KEYS - 1, last));
+}
+
 // Key row pointer: key pages are [NB, Hkv, BS, D].
-__device__ __forceinline__ const uint16_t* key_row(const PageGeometry& g, int key) {
-  const long long blk = g.table[key >> g.block_shift];
+__device__ __forceinline__ const uint16_t* key_row(const PageGeometry& g, const WindowPages& wp, int w, int key) {
+  const long long blk = page_of(g, wp, w, key);
   return g.k_pages + ((blk * g.kv_heads + g.kvh) << g.block_shift) * D + (long long)(key & g.block_mask) * D;
 }
 
 // Pointer to the values of 8 consecutive keys (key % 8 == 0) at head dimension 0: value pages
 // are [NB, Hkv, D, BS]; dimension d is `d << block_shift` elements further.
-__device__ __forceinline__ const uint16_t* value_chunk(const PageGeometry& g, int key) {
-  const long long blk = g.table[key >> g.block_shift];
+__device__ __forceinline__ const uint16_t* value_chunk(const PageGeometry& g, const WindowPages& wp, int w, int key) {
+  const long long blk = page_of(g, wp, w, key);
   return g.v_pages + ((blk * g.kv_heads + g.kvh) << g.block_shift) * D + (key & g.block_mask);
 }
 
 // Everything one 32-key window contributes, as matrix-core operands: the lane's two key rows
 // (A operands of the score tiles) and its 8-key value chunk for every head-dimension tile.
-struct WindowFrags {
+struct KeyFrags {
   Frag8 k[2][KJ > 0 ? KJ : 1];
   Frag8 ktail[2];
+};
+struct ValueFrags {
   Frag8 v[NT];
 };
+struct WindowFrags : KeyFrags, ValueFrags {};
 
-// Issue the loads of window `w`.  A key or chunk outside lo..last is redirected to `safe_key`
-// (a key of the request that is certainly in a live page): the loads stay unconditional, so
-// they can be issued a whole window ahead; what they bring is masked in the softmax.
+// Issue the loads of window `w` (keys outside lo..last: see live_key).
 __device__ __forceinline__ void load_window(WindowFrags& f, const PageGeometry& g, int w, int lo, int last,
-                                            int safe_key, int lane16, int group) {
+                                            int lane16, int group) {
+  const WindowPages wp = window_pages(g, w);
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key = w + 8 * (lane16 >> 2) + 4 * t + (lane16 & 3);
-    const uint16_t* row = key_row(g, (key >= lo && key <= last) ? key : safe_key);
+    const uint16_t* row = key_row(g, wp, w, live_key(key, w, lo, last));
 #pragma unroll
     for (int j = 0; j < KJ; ++j) f.k[t][j] = load8(row + 32 * j + 8 * group);
     if (KTAIL) f.ktail[t] = group < 2 ? load8(row + 32 * KJ + 8 * group) : Frag8{0u, 0u, 0u, 0u};
   }
   const int chunk = w + 8 * group;
-  const uint16_t* vp = value_chunk(g, (chunk + 7 >= lo && chunk <= last) ? chunk : (safe_key & ~7));
+  const bool live = chunk + 7 >= lo && chunk <= last;
+  const uint16_t* vp = value_chunk(g, wp, w, live ? chunk : (live_key(chunk, w, lo, last) & ~7));
 #pragma unroll
   for (int n = 0; n < NT; ++n)
     f.v[n] = load8(vp + ((long long)(16 * n + lane16) << g.block_shift));
@@ -154,7 +224,7 @@ __device__ __forceinline__ void clear_stale_values(WindowFrags& f, int w, int lo
 }
 
 // S^T tile t of the window for the 16 columns whose queries are in `q`.
-__device__ __forceinline__ f32x4 score_tile(const WindowFrags& f, int t, const QueryFrags& q) {
+__device__ __forceinline__ f32x4 score_tile(const KeyFrags& f, int t, const QueryFrags& q) {
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int j = 0; j < KJ; ++j)
@@ -177,50 +247,78 @@ __device__ __forceinline__ void init_state(ColumnState& st) {
   for (int n = 0; n < NT; ++n) st.acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-// One window for one set of 16 columns: scores, masked online softmax, O^T += V^T P^T.
-// The lane's column sees the keys first_valid..last_valid (inclusive).
-__device__ __forceinline__ void attend_window(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w,
-                                              int group, int first_valid, int last_valid, float scale_log2) {
-  const f32x4 s0 = score_tile(f, 0, q);
-  const f32x4 s1 = score_tile(f, 1, q);
-  float s[8];
+// The softmax step of one window for one set of 16 columns, from the two score tiles: updates
+// the running maximum and sum, returns the probabilities as the B operand of the second
+// product and the factor the accumulators must be scaled by first.  With MASKED the lane's
+// column sees only the keys first_valid..last_valid (inclusive); without, the caller vouches
+// that every key of the window is visible to every column of the wavefront.
+template <bool MASKED>
+__device__ __forceinline__ Frag8 softmax_window(ColumnState& st, const f32x4 s0, const f32x4 s1, int w, int group,
+                                                int first_valid, int last_valid, float scale_log2, float& alpha) {
+  float s[8];  // unscaled scores; e = 4 t + i is row 4 g + i of tile t
   float mx = -INFINITY;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int key = w + 8 * group + e;  // e = 4 t + i: row 4 g + i of tile t
-    const float raw = (e < 4 ? s0[e & 3] : s1[e & 3]) * scale_log2;
-    s[e] = (key >= first_valid && key <= last_valid) ? raw : -INFINITY;
+    const float raw = e < 4 ? s0[e & 3] : s1[e & 3];
+    if (MASKED) {
+      const int key = w + 8 * group + e;
+      s[e] = (key >= first_valid && key <= last_valid) ? raw : -INFINITY;
+    } else {
+      s[e] = raw;
+    }
     mx = fmaxf(mx, s[e]);
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, TS_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, TS_WAVE));
+  mx = groups_max(mx) * scale_log2;  // the scale is positive: the maximum commutes with it
   const float m_new = fmaxf(st.m, mx);
   // Nothing visible to this column so far: keep the state, contribute zeros.
-  const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-  const float alpha = exp2f(st.m - m_use);  // 0 when st.m is -inf
+  const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
+  alpha = fast_exp2(st.m - m_use);  // 0 when st.m is -inf
   float pe[8];
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    pe[e] = exp2f(s[e] - m_use);  // 0 for masked keys
+    pe[e] = fast_exp2(fmaf(s[e], scale_log2, -m_use));  // 0 for masked keys
     sum += pe[e];
   }
-  const Frag8 p = {pack2(pe[0], pe[1]), pack2(pe[2], pe[3]), pack2(pe[4], pe[5]), pack2(pe[6], pe[7])};
   st.l = st.l * alpha + sum;
   st.m = m_new;
+  return Frag8{pack2(pe[0], pe[1]), pack2(pe[2], pe[3]), pack2(pe[4], pe[5]), pack2(pe[6], pe[7])};
+}
+
+// O^T = alpha O^T + V^T P^T.  Once a column's maximum has settled, alpha is exactly 1: the
+// rescaling is skipped when that holds for the whole wavefront.
+__device__ __forceinline__ void accumulate(ColumnState& st, const ValueFrags& f, const Frag8 p, float alpha) {
+  if (__any(alpha != 1.f)) {
 #pragma unroll
-  for (int n = 0; n < NT; ++n) {
-    st.acc[n] *= alpha;
-    st.acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(f.v[n]), as_bf16x8(p), st.acc[n], 0, 0, 0);
+    for (int n = 0; n < NT; ++n) st.acc[n] *= alpha;
   }
+#pragma unroll
+  for (int n = 0; n < NT; ++n)
+    st.acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(f.v[n]), as_bf16x8(p), st.acc[n], 0, 0, 0);
+}
+
+// One window for one set of 16 columns: scores, online softmax, O^T += V^T P^T.
+template <bool MASKED>
+__device__ __forceinline__ void attend_window(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w,
+                                              int group, int first_valid, int last_valid, float scale_log2) {
+  const f32x4 s0 = score_tile(f, 0, q);
+  const f32x4 s1 = score_tile(f, 1, q);
+  float alpha;
+  const Frag8 p = softmax_window<MASKED>(st, s0, s1, w, group, first_valid, last_valid, scale_log2, alpha);
+  accumulate(st, f, p, alpha);
+}
+
+// Dispatch on a wavefront-uniform flag: `interior` windows need no masks.
+__device__ __forceinline__ void attend(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w, int group,
+                                       int first_valid, int last_valid, float scale_log2, bool interior) {
+  if (interior)
+    attend_window<false>(st, f, q, w, group, first_valid, last_valid, scale_log2);
+  else
+    attend_window<true>(st, f, q, w, group, first_valid, last_valid, scale_log2);
 }
 
 // Sum of the lane's column over the four lane groups.
-__device__ __forceinline__ float column_sum(float l) {
-  l += __shfl_xor(l, 16, TS_WAVE);
-  l += __shfl_xor(l, 32, TS_WAVE);
-  return l;
-}
+__device__ __forceinline__ float column_sum(float l) { return groups_sum(l); }
 
 // ---------------------------------------------------------------------------------------------
 // decode: grid (splits, kv_heads * head_tiles, requests); one wavefront each.
@@ -259,7 +357,7 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
   const int begin = (lo & ~(WINDOW_KEYS - 1)) + split * keys_per_split;
   const int end = min(begin + keys_per_split, ctx);
 
-  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, kv_heads, kvh, block_shift,
+  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, table_width, kv_heads, kvh, block_shift,
                    (1 << block_shift) - 1};
   ColumnState st;
   init_state(st);
@@ -268,17 +366,17 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
     QueryFrags qf;
     load_query(qf, head_valid ? q + (size_t)token * q_stride + (size_t)head * D : nullptr, group);
     WindowFrags fa, fb;
-    load_window(fa, geo, begin, lo, p, p, lane16, group);
+    load_window(fa, geo, begin, lo, p, lane16, group);
     int w = begin;
     while (true) {
-      if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo, p, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fa, w, lo, p, group);
-      attend_window(st, fa, qf, w, group, lo, p, scale_log2);
+      attend_window<true>(st, fa, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;
       if (w >= end) break;
-      if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo, p, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fb, w, lo, p, group);
-      attend_window(st, fb, qf, w, group, lo, p, scale_log2);
+      attend_window<true>(st, fb, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;
       if (w >= end) break;
     }
@@ -366,8 +464,11 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
   const int lo_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const int begin = lo_first & ~(WINDOW_KEYS - 1);
   const int end = p_last + 1;
+  // A window every column of the block sees in full: no masks needed.
+  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+  auto interior = [&](int w) { return cols == 16 && w >= lo_last && w + WINDOW_KEYS - 1 <= pos0; };
 
-  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, kv_heads, kvh, block_shift,
+  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, table_width, kv_heads, kvh, block_shift,
                    (1 << block_shift) - 1};
   QueryFrags qf[CT];
   ColumnState st[CT];
@@ -380,19 +481,19 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
   }
 
   WindowFrags fa, fb;
-  load_window(fa, geo, begin, lo_first, p_last, p_last, lane16, group);
+  load_window(fa, geo, begin, lo_first, p_last, lane16, group);
   int w = begin;
   while (true) {
-    if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo_first, p_last, p_last, lane16, group);
+    if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo_first, p_last, lane16, group);
     if (w < lo_first || w + WINDOW_KEYS > end) clear_stale_values(fa, w, lo_first, p_last, group);
 #pragma unroll
-    for (int c = 0; c < CT; ++c) attend_window(st[c], fa, qf[c], w, group, lo_col, p_col, scale_log2);
+    for (int c = 0; c < CT; ++c) attend(st[c], fa, qf[c], w, group, lo_col, p_col, scale_log2, interior(w));
     w += WINDOW_KEYS;
     if (w >= end) break;
-    if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo_first, p_last, p_last, lane16, group);
+    if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo_first, p_last, lane16, group);
     if (w < lo_first || w + WINDOW_KEYS > end) clear_stale_values(fb, w, lo_first, p_last, group);
 #pragma unroll
-    for (int c = 0; c < CT; ++c) attend_window(st[c], fb, qf[c], w, group, lo_col, p_col, scale_log2);
+    for (int c = 0; c < CT; ++c) attend(st[c], fb, qf[c], w, group, lo_col, p_col, scale_log2, interior(w));
     w += WINDOW_KEYS;
     if (w >= end) break;
   }
@@ -411,6 +512,333 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
       }
     }
   }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// prefill with shared windows: grid (query blocks, kv_heads * head_chunks), HW wavefronts per
+// workgroup.  Wavefront i handles query head (chunk * HW + i) of the KV head for the block's 16
+// tokens; all of them see the same keys, so each 32-key window is fetched from the pages once
+// per workgroup, staged in LDS (double-buffered, rows padded so that the 16 lanes of one LDS
+// pass hit distinct banks) and read from there as matrix-core operands by every wavefront.
+// Window w + 1 travels from global memory to registers while window w is computed.
+// ---------------------------------------------------------------------------------------------
+constexpr int K_ROW = D + 8;              // LDS stride of a key row (elements)
+constexpr int V_ROW = WINDOW_KEYS + 8;    // LDS stride of a head dimension's 32 values
+constexpr int K_TILE = WINDOW_KEYS * K_ROW;
+constexpr int V_TILE = D * V_ROW;
+constexpr int K_PIECES = WINDOW_KEYS * (D / 8);  // 16-byte pieces of a window's keys
+constexpr int V_PIECES = D * (WINDOW_KEYS / 8);  // and of its values
+
+template <int HW>
+struct StagedWindow {
+  static constexpr int THREADS = HW * TS_WAVE;
+  static constexpr int K_EACH = (K_PIECES + THREADS - 1) / THREADS;
+  static constexpr int V_EACH = (V_PIECES + THREADS - 1) / THREADS;
+  static constexpr int PIECES = K_EACH + V_EACH;
+  u32x4 k[K_EACH];
+  u32x4 v[V_EACH];
+};
+
+// What a thread's pieces have in common in every window, worked out once: which of the
+// window's pages a piece lies in, its byte address but for the page's own offset, and where it
+// goes in LDS.  Per window that leaves a select of the page id and one multiply-add per piece.
+template <int HW>
+struct PiecePlan {
+  using W = StagedWindow<HW>;
+  int k_sel[W::K_EACH];
+  unsigned long long k_base[W::K_EACH];
+  int k_lds[W::K_EACH];  // element offset in the staged key tile, -1: a spare thread
+  int v_sel[W::V_EACH];
+  unsigned long long v_base[W::V_EACH];
+  int v_lds[W::V_EACH];
+  unsigned page_bytes;  // bytes from one page of the pool to the next
+};
+
+template <int HW>
+__device__ __forceinline__ void plan_pieces(PiecePlan<HW>& plan, const PageGeometry& g) {
+  using W = StagedWindow<HW>;
+  plan.page_bytes = (unsigned)((g.kv_heads << g.block_shift) * D * 2);
+  const unsigned long long head_bytes = (unsigned long long)((g.kvh << g.block_shift) * D) * 2;
+#pragma unroll
+  for (int i = 0; i < W::K_EACH; ++i) {
+    const int raw = threadIdx.x + i * W::THREADS;
+    const int idx = min(raw, K_PIECES - 1);  // spare threads repeat the last piece
+    const int ko = idx / (D / 8);
+    const int col = 8 * (idx % (D / 8));
+    plan.k_sel[i] = ko >> g.block_shift;
+    plan.k_base[i] = (unsigned long long)g.k_pages + head_bytes + (unsigned long long)((ko & g.block_mask) * D + col) * 2;
+    // Key offset ko of the window goes to the row the score tiles read it from: tile
+    // t = (ko / 4) % 2, row m = 4 (ko / 8) + ko % 4, stored at 16 t + m, so that the 16 lanes
+    // of an LDS pass read 16 consecutive rows (distinct banks with the padded stride).
+    const int slot = 16 * ((ko >> 2) & 1) + ((ko >> 3) << 2) + (ko & 3);
+    plan.k_lds[i] = raw < K_PIECES ? slot * K_ROW + col : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < W::V_EACH; ++i) {
+    const int raw = threadIdx.x + i * W::THREADS;
+    const int idx = min(raw, V_PIECES - 1);
+    const int d = idx / (WINDOW_KEYS / 8);
+    const int kc = 8 * (idx % (WINDOW_KEYS / 8));
+    plan.v_sel[i] = kc >> g.block_shift;
+    plan.v_base[i] = (unsigned long long)g.v_pages + head_bytes +
+                     (unsigned long long)((d << g.block_shift) + (kc & g.block_mask)) * 2;
+    plan.v_lds[i] = raw < V_PIECES ? d * V_ROW + kc : -1;
+  }
+}
+
+// Issue the loads of this thread's pieces of window `w`.  Nothing here looks at what the loads
+// bring, so they stay in flight until the window is staged.  A window wholly inside lo..last
+// takes the planned addresses; one at the edge replaces keys outside lo..last (see live_key).
+template <int HW>
+__device__ __forceinline__ void fetch_window(StagedWindow<HW>& r, const PiecePlan<HW>& plan, const PageGeometry& g,
+                                             int w, int lo, int last) {
+  using W = StagedWindow<HW>;
+  const WindowPages wp = window_pages(g, w);
+  if (w >= lo && w + WINDOW_KEYS - 1 <= last) {
+    // A block of more than 32 keys holds the window at offset w % block size.
+    const unsigned long long k_in_page = (unsigned long long)((w & g.block_mask) * D) * 2;
+    const unsigned long long v_in_page = (unsigned long long)(w & g.block_mask) * 2;
+#pragma unroll
+    for (int i = 0; i < W::K_EACH; ++i) {
+      const int sel = plan.k_sel[i];
+      const unsigned page = sel == 0 ? wp.page[0] : (sel == 1 ? wp.page[1] : (sel == 2 ? wp.page[2] : wp.page[3]));
+      r.k[i] = load8(reinterpret_cast<const uint16_t*>(plan.k_base[i] + ((unsigned long long)page * plan.page_bytes + k_in_page)));
+    }
+#pragma unroll
+    for (int i = 0; i < W::V_EACH; ++i) {
+      const int sel = plan.v_sel[i];
+      const unsigned page = sel == 0 ? wp.page[0] : (sel == 1 ? wp.page[1] : (sel == 2 ? wp.page[2] : wp.page[3]));
+      r.v[i] = load8(reinterpret_cast<const uint16_t*>(plan.v_base[i] + ((unsigned long long)page * plan.page_bytes + v_in_page)));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < W::K_EACH; ++i) {
+      const int idx = min((int)threadIdx.x + i * W::THREADS, K_PIECES - 1);
+      const int key = w + idx / (D / 8);
+      r.k[i] = load8(key_row(g, wp, w, live_key(key, w, lo, last)) + 8 * (idx % (D / 8)));
+    }
+#pragma unroll
+    for (int i = 0; i < W::V_EACH; ++i) {
+      const int idx = min((int)threadIdx.x + i * W::THREADS, V_PIECES - 1);
+      const int d = idx / (WINDOW_KEYS / 8);
+      const int chunk = w + 8 * (idx % (WINDOW_KEYS / 8));
+      const bool live = chunk + 7 >= lo && chunk <= last;
+      r.v[i] = load8(value_chunk(g, wp, w, live ? chunk : (live_key(chunk, w, lo, last) & ~7)) +
+                     ((long long)d << g.block_shift));
+    }
+  }
+}
+
+// Write the fetched window `w` to LDS.  Values of keys outside lo..last are whatever an earlier
+// owner of the page left: they are cleared here, so that a stale non-finite value cannot meet a
+// zero probability (only a window that is not wholly inside lo..last needs it).
+template <int HW>
+__device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const StagedWindow<HW>& r,
+                                             const PiecePlan<HW>& plan, int w, int lo, int last) {
+  using W = StagedWindow<HW>;
+#pragma unroll
+  for (int i = 0; i < W::K_EACH; ++i)
+    if (plan.k_lds[i] >= 0) *reinterpret_cast<u32x4*>(ks + plan.k_lds[i]) = r.k[i];
+  const bool edge = w < lo || w + WINDOW_KEYS - 1 > last;
+#pragma unroll
+  for (int i = 0; i < W::V_EACH; ++i) {
+    if (plan.v_lds[i] < 0) continue;
+    u32x4 value = r.v[i];
+    if (edge) {
+      const int idx = threadIdx.x + i * W::THREADS;
+      const int chunk = w + 8 * (idx % (WINDOW_KEYS / 8));
+      const bool live = chunk + 7 >= lo && chunk <= last;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t low = (live && chunk + 2 * e <= last) ? 0x0000ffffu : 0u;
+        const uint32_t high = (live && chunk + 2 * e + 1 <= last) ? 0xffff0000u : 0u;
+        value[e] &= low | high;
+      }
+    }
+    *reinterpret_cast<u32x4*>(vs + plan.v_lds[i]) = value;
+  }
+}
+
+// The lane's operands of the staged window, in the layout load_window gives.
+__device__ __forceinline__ void read_keys(KeyFrags& f, const uint16_t* ks, int lane16, int group) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const uint16_t* row = ks + (16 * t + lane16) * K_ROW;
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) f.k[t][j] = load8(row + 32 * j + 8 * group);
+    if (KTAIL) f.ktail[t] = group < 2 ? load8(row + 32 * KJ + 8 * group) : Frag8{0u, 0u, 0u, 0u};
+  }
+}
+__device__ __forceinline__ void read_values(ValueFrags& f, const uint16_t* vs, int lane16, int group) {
+#pragma unroll
+  for (int n = 0; n < NT; ++n) f.v[n] = load8(vs + (16 * n + lane16) * V_ROW + 8 * group);
+}
+
+template <int HW, int CT>
+__global__ void __launch_bounds__(HW * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
+                      const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
+                      const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
+                      const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
+                      int pair_blocks, int heads, int kv_heads, int block_shift, float scale_log2, int window) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
+  uint16_t* ks = staged;
+  uint16_t* vs = staged + 2 * K_TILE;
+  const int lane = threadIdx.x & (TS_WAVE - 1);
+  const int wave = threadIdx.x / TS_WAVE;
+  const int lane16 = lane & 15;
+  const int group = lane >> 4;
+  const int gsize = heads / kv_heads;
+  const int head_chunks = (gsize + HW * CT - 1) / (HW * CT);
+  // Workgroup id -> (block, KV head and chunk of its query heads), the latter fastest.  Blocks
+  // come heaviest first.  With pair_blocks (the host sets it when all workgroups are resident
+  // at once, two per compute unit) the second half of the grid walks the lighter half of the
+  // blocks backwards, so that the two workgroups a compute unit is handed in turn, i and
+  // i + n / 2, are a heavy and a light one.
+  const int lanes_y = kv_heads * head_chunks;
+  const int y = blockIdx.x % lanes_y;
+  int block = blockIdx.x / lanes_y;
+  if (pair_blocks && block >= (num_blocks + 1) / 2) block = num_blocks - 1 - (block - (num_blocks + 1) / 2);
+  const int kvh = y / head_chunks;
+  const int first_head = ((y % head_chunks) * HW + wave) * CT;  // within the KV head's group
+  const int seq = blocks[2 * block];
+  const int row0 = blocks[2 * block + 1];
+  const int row_end = query_start_loc[seq + 1];
+  const int ctx = context_lens[seq];
+  const int pos0 = ctx - (row_end - query_start_loc[seq]) + (row0 - query_start_loc[seq]);  // position of row0
+  const int cols = min(16, row_end - row0);
+  const bool col_valid = lane16 < cols;
+  const int p_col = col_valid ? pos0 + lane16 : -1;
+  const int lo_col = (window > 0 && p_col - window + 1 > 0) ? p_col - window + 1 : 0;
+  const int p_last = pos0 + cols - 1;
+  const int lo_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int begin = lo_first & ~(WINDOW_KEYS - 1);
+  const int end = p_last + 1;
+  // A window every column of the block sees in full: no masks needed.
+  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+  auto interior = [&](int w) { return cols == 16 && w >= lo_last && w + WINDOW_KEYS - 1 <= pos0; };
+
+  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, table_width, kv_heads, kvh, block_shift,
+                   (1 << block_shift) - 1};
+  QueryFrags qf[CT];
+  ColumnState st[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int hg = first_head + c;
+    load_query(qf[c], (col_valid && hg < gsize) ? q + (size_t)(row0 + lane16) * q_stride + (size_t)(kvh * gsize + hg) * D
+                                                : nullptr, group);
+    init_state(st[c]);
+  }
+  const bool wave_live = first_head < gsize;
+
+  // Windows travel global memory -> registers -> LDS.  A ring of P register sets keeps the
+  // loads of P windows in flight, so a load has P - 1 rounds of computing to arrive in; LDS
+  // holds two windows (the one being read, the next being written).
+  constexpr int P = StagedWindow<HW>::PIECES * CT <= 4 ? 3 : 2;
+  StagedWindow<HW> ring[P];
+  PiecePlan<HW> plan;
+  plan_pieces<HW>(plan, geo);
+  // Every round issues its fetch, past the last window too (that window again, dropped): with a
+  // fetch that may or may not have been issued the compiler cannot count the loads in flight
+  // and waits for all of them before each staging.
+  const int last_window = (end - 1) & ~(WINDOW_KEYS - 1);
+#pragma unroll
+  for (int u = 0; u < P; ++u)
+    fetch_window<HW>(ring[u], plan, geo, min(begin + u * WINDOW_KEYS, last_window), lo_first, p_last);
+  stage_window<HW>(ks, vs, ring[0], plan, begin, lo_first, p_last);
+  __syncthreads();
+  int buf = 0;
+  int w = begin;
+  while (w < end) {
+#pragma unroll
+    for (int u = 0; u < P; ++u) {
+      // ring[u] held window w, which is staged: refill it with the window P rounds ahead.
+      fetch_window<HW>(ring[u], plan, geo, min(w + P * WINDOW_KEYS, last_window), lo_first, p_last);
+      if (wave_live) {
+        // Keys first, values only once the probabilities stand: the two sets of operands are
+        // never in registers together.
+        Frag8 prob[CT];
+        float alpha[CT];
+        {
+          KeyFrags kf;
+          read_keys(kf, ks + buf * K_TILE, lane16, group);
+          const bool inside = interior(w);
+#pragma unroll
+          for (int c = 0; c < CT; ++c) {
+            const f32x4 s0 = score_tile(kf, 0, qf[c]);
+            const f32x4 s1 = score_tile(kf, 1, qf[c]);
+            prob[c] = inside ? softmax_window<false>(st[c], s0, s1, w, group, lo_col, p_col, scale_log2, alpha[c])
+                             : softmax_window<true>(st[c], s0, s1, w, group, lo_col, p_col, scale_log2, alpha[c]);
+          }
+        }
+        ValueFrags vf;
+        read_values(vf, vs + buf * V_TILE, lane16, group);
+#pragma unroll
+        for (int c = 0; c < CT; ++c) accumulate(st[c], vf, prob[c], alpha[c]);
+      }
+      if (w + WINDOW_KEYS < end)  // the other LDS window was last read a round ago
+        stage_window<HW>(ks + (buf ^ 1) * K_TILE, vs + (buf ^ 1) * V_TILE, ring[(u + 1) % P], plan,
+                         w + WINDOW_KEYS, lo_first, p_last);
+      __syncthreads();
+      buf ^= 1;
+      w += WINDOW_KEYS;
+      if (w >= end) break;
+    }
+  }
+
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int hg = first_head + c;
+    const float l_total = column_sum(st[c].l);
+    if (col_valid && hg < gsize) {
+      const float inv = 1.f / l_total;
+      uint16_t* orow = out + ((size_t)(row0 + lane16) * heads + kvh * gsize + hg) * D;
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+        const f32x4 a = st[c].acc[n] * inv;
+        *reinterpret_cast<u32x2*>(orow + 16 * n + 4 * group) = Frag4{pack2(a[0], a[1]), pack2(a[2], a[3])};
+      }
+    }
+  }
+}
+
+template <int HW, int CT>
+static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16_t* q, long q_stride,
+                                 const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
+                                 int table_width, const int* query_start_loc, const int* context_lens,
+                                 const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
+                                 float scale_log2, int window) {
+  constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
+  static_assert(lds <= 160 * 1024, "the staged windows must fit in LDS");
+  if (lds > 48 * 1024) {
+    static bool raised = false;  // per process; the attribute belongs to the kernel
+    if (!raised) {
+      if (hipFuncSetAttribute((const void*)prefill_shared_kernel<HW, CT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess)
+        return TS_ERR_LAUNCH;
+      raised = true;
+    }
+  }
+  const int gsize = heads / kv_heads;
+  const int chunks = (gsize + HW * CT - 1) / (HW * CT);
+  const long long total = (long long)num_blocks * kv_heads * chunks;
+  if (total > 0x7fffffffLL) return TS_ERR_SHAPE;
+  // Two workgroups fit a compute unit; when the whole grid is resident at once the hardware
+  // cannot even out the blocks' unequal lengths by handing out work as units free up, so
+  // heavy and light blocks are paired instead (see the kernel).
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int device = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return TS_ERR_LAUNCH;
+    compute_units = prop.multiProcessorCount;
+  }
+  const int pair_blocks = total <= 2LL * compute_units ? 1 : 0;
+  hipLaunchKernelGGL((prefill_shared_kernel<HW, CT>), dim3((unsigned)total), dim3(HW * TS_WAVE), lds, stream, out, q,
+                     q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks,
+                     num_blocks, pair_blocks, heads, kv_heads, shift, scale_log2, window);
+  return ts_launch_status();
 }
 
 }  // namespace
@@ -465,6 +893,17 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   int shift = 0;
   while ((1 << shift) < block_size) ++shift;
   const int gsize = heads / kv_heads;
+  // Three or more query heads per KV head: workgroups of four wavefronts, one or two heads each,
+  // share every window of keys and values through LDS.
+  if (gsize >= 3) {
+    if (gsize >= 5)
+      return launch_prefill_shared<4, 2>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
+                                         (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
+                                         context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+    return launch_prefill_shared<4, 1>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
+                                       (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
+                                       context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+  }
   constexpr int CT = TS_PREFILL_HEADS;
   const int head_chunks = (gsize + CT - 1) / CT;
   if (kv_heads * head_chunks > 65535) return TS_ERR_SHAPE;

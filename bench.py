@@ -45,6 +45,11 @@ SHAPE_7B = {
     "use_sliding_window": False,
     "max_position_embeddings": 32768,
 }
+#: BASELINE.json configs[3] and configs[4]: the other layer shapes a run can be asked for.
+SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
+                 intermediate_size=13824, rms_norm_eps=1e-5)
+SHAPE_32B = dict(SHAPE_14B, num_hidden_layers=64, intermediate_size=27648)
+SHAPES = {"7b": ("Qwen2.5-7B", SHAPE_7B), "14b": ("Qwen2.5-14B", SHAPE_14B), "32b": ("Qwen2.5-32B", SHAPE_32B)}
 CONTEXT = 8192
 PREFILL_TOKENS = 2048
 PAGE = 16
@@ -64,6 +69,11 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-gemm-tuning", action="store_true",
                    help="leave the choice of the BLAS library's prefill kernels to its heuristic")
     p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
+    p.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (the default run is 7b)")
+    p.add_argument("--fill-hbm", action="store_true",
+                   help="size the cache pool to the free device memory and interleave the requests' pages in it")
+    p.add_argument("--mixed-prefill", type=int, default=0, metavar="N",
+                   help="time steps that hold the batch's decode tokens and one N-token portion of a prompt")
     return p.parse_args()
 
 
@@ -71,7 +81,8 @@ class DecodeBench:
     """Requests with a given context already in the cache, decoded one token per step through
     the engine's own cache manager, step function and sampler."""
 
-    def __init__(self, model, config, batch: int, context: int, steps_total: int) -> None:
+    def __init__(self, model, config, batch: int, context: int, steps_total: int, *, fill_hbm: bool = False,
+                 extra_tokens: int = 0) -> None:
         import torch
 
         from turboserve_amd.cache.manager import CacheManager
@@ -82,25 +93,52 @@ class DecodeBench:
         self.torch = torch
         self.batch = batch
         self.context = context
+        self.vocab_size = config.vocab_size
         pages_per_request = -(-(context + steps_total + 1) // PAGE)
-        num_pages = batch * pages_per_request
-        self.storage = build_storage(model, num_pages, PAGE, batch)
+        num_pages = batch * pages_per_request + -(-extra_tokens // PAGE)
+        if fill_hbm:
+            # As many pages as 90% of what is free holds (at least what the requests need).
+            free, _ = torch.cuda.mem_get_info()
+            page_bytes = config.kv_bytes_per_token(model.runtime.dtype) * PAGE
+            num_pages = max(num_pages, int(free * 0.9) // page_bytes)
+        self.num_pages = num_pages
+        self.storage = build_storage(model, num_pages, PAGE, batch + 1)
         for pages in self.storage.pages:
-            pages.normal_(0.0, 0.5)
-        self.manager = CacheManager(self.storage.layout.windows(), num_pages, PAGE, batch)
+            for member in pages:  # piecewise: a 200 GB pool is not filled in one launch's temporaries
+                member.normal_(0.0, 0.5)
+        self.manager = CacheManager(self.storage.layout.windows(), num_pages, PAGE, batch + 1)
         self.runner = ModelRunner(model, self.storage, check=False)
         self.sampler = Sampler(model.runtime.ops)
         generator = torch.Generator().manual_seed(1234)
         self.tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
+        self.portion = torch.randint(0, config.vocab_size, (max(extra_tokens, 1),), generator=generator).tolist()
         for request in range(batch):
             self.manager.admit(request)
-            self.manager.append(request, context - 1)  # the context's last token is decoded below
+        if fill_hbm:
+            # Page by page in turn, as requests that grow together get them: interleaved tables.
+            remaining = [context - 1] * batch
+            while any(remaining):
+                for request in range(batch):
+                    take = min(PAGE, remaining[request])
+                    if take:
+                        self.manager.append(request, take)
+                        remaining[request] -= take
+        else:
+            for request in range(batch):
+                self.manager.append(request, context - 1)  # the context's last token is decoded below
 
-    def step(self) -> None:
+    def step(self, portion_tokens: int = 0) -> None:
+        """One decode step of the batch; with ``portion_tokens`` the step also holds the first
+        portion, that long, of a new request's prompt (its pages are given back afterwards)."""
         from turboserve_amd.engine.batch import StepEntry
         from turboserve_amd.sampling.params import SamplingParams
 
         entries = []
+        if portion_tokens:
+            held = self.manager.admit("portion")
+            slots = self.manager.append("portion", portion_tokens)
+            entries.append(StepEntry(request="portion", tokens=self.portion[:portion_tokens], start=0,
+                                     tables=held.tables, slots=slots, state_slot=held.state_slot, want=[]))
         for request in range(self.batch):
             held = self.manager.get(request)
             start = held.num_tokens
@@ -111,16 +149,18 @@ class DecodeBench:
         greedy = SamplingParams(temperature=0.0)
         out = self.sampler.sample(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
         self.tokens = out.token_ids
+        if portion_tokens:
+            self.manager.free("portion")
 
-    def run(self, steps: int, warmup: int) -> float:
-        """Seconds for ``steps`` decode steps after ``warmup`` untimed ones."""
+    def run(self, steps: int, warmup: int, portion_tokens: int = 0) -> float:
+        """Seconds for ``steps`` steps after ``warmup`` untimed ones."""
         torch = self.torch
         for _ in range(warmup):
-            self.step()
+            self.step(portion_tokens)
         torch.cuda.synchronize()
         started = time.perf_counter()
         for _ in range(steps):
-            self.step()
+            self.step(portion_tokens)
         torch.cuda.synchronize()
         return time.perf_counter() - started
 
@@ -204,7 +244,8 @@ def main() -> int:
     from turboserve_amd.hwinfo import collect
     from turboserve_amd.weights.random_init import random_tensors_on_device
 
-    shape = dict(SHAPE_7B)
+    shape_name, shape = SHAPES[args.shape]
+    shape = dict(shape)
     full_layers = shape["num_hidden_layers"]
     if args.layers is not None:
         shape["num_hidden_layers"] = args.layers
@@ -216,9 +257,19 @@ def main() -> int:
     itemsize = 2 if dtype == torch.bfloat16 else 4
     dtype_key = "bf16" if dtype == torch.bfloat16 else "fp32"
 
+    pool_tokens = 0
+
     def decode_rate(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        bench = DecodeBench(model, config, batch, args.context, steps + warmup)
-        seconds = bench.run(steps, warmup)
+        nonlocal pool_tokens
+        bench = DecodeBench(model, config, batch, args.context, steps + warmup, fill_hbm=args.fill_hbm,
+                            extra_tokens=args.mixed_prefill)
+        pool_tokens = bench.num_pages * PAGE
+        if args.mixed_prefill and not args.no_gemm_tuning and dtype == torch.bfloat16:
+            from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
+
+            with LibraryGemmTuning(os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")):
+                bench.runner.dry_run(args.mixed_prefill + batch)
+        seconds = bench.run(steps, warmup, args.mixed_prefill)
         bench.close()
         return batch * steps / seconds, seconds / steps
 
@@ -228,11 +279,26 @@ def main() -> int:
         return 0
 
     value, step_seconds = decode_rate(args.batch, args.steps, args.warmup)
+    if args.mixed_prefill:
+        # A mixed step is priced by its products' flops, not by bytes: say what ran and stop there.
+        flops = (prefill_flops(config, layers, args.mixed_prefill)
+                 + 2.0 * args.batch * decode_bytes(config, layers, 0, 0, 1)  # every weight once per decode token
+                 + 4.0 * args.batch * layers * config.q_proj_size * args.context)  # and its attention
+        print(json.dumps({
+            "metric": f"mixed step: {args.batch} decode tokens + one {args.mixed_prefill}-token prompt portion "
+                      f"({shape_name} shape, one MI355X)",
+            "value": round((args.batch + args.mixed_prefill) / step_seconds, 1), "unit": "tokens/s",
+            "decode_tokens_per_s": round(value, 2), "ms_per_step": round(step_seconds * 1e3, 3),
+            "steps": args.steps, "warmup": args.warmup, "dtype": dtype_key, "decode_context": args.context,
+            "layers": layers, "kv_pool_tokens": pool_tokens,
+            "flops_frac": round(flops / step_seconds / PEAK_FLOPS[dtype_key], 4),
+        }))
+        return 0
     mean_context = args.context + args.warmup + args.steps / 2
     read = decode_bytes(config, layers, args.batch, mean_context, itemsize)
     achieved = read / step_seconds / 1e9
     result = {
-        "metric": "decode tok/s (Qwen2.5-7B shape, paged cache, one MI355X)",
+        "metric": f"decode tok/s ({shape_name} shape, paged cache, one MI355X)",
         "value": round(value, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -245,7 +311,7 @@ def main() -> int:
         "dtype": dtype_key,
         "data": "synthetic: random weights N(0,0.02), uniform-random token ids, cache pre-filled with random keys/values",
         "config": {
-            "model": "Qwen2.5-7B shape (Qwen2ForCausalLM)",
+            "model": f"{shape_name} shape (Qwen2ForCausalLM)",
             "global_batch": args.batch,
             "seq_len": args.context,
             "parallelism": "single GPU",
@@ -261,6 +327,7 @@ def main() -> int:
             "rms_norm_eps": config.rms_norm_eps,
             "tie_word_embeddings": config.tie_word_embeddings,
             "page_size": PAGE,
+            "kv_pool_tokens": pool_tokens,
             "prefill_tokens": PREFILL_TOKENS,
             "prefill_gemm_choice": "library heuristic" if args.no_gemm_tuning else "library candidates timed at start-up",
             "sampling": "greedy",

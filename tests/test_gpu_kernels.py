@@ -155,6 +155,24 @@ def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):
     torch.testing.assert_close(full.sum(0)[17:18], one.sum(0), rtol=1e-5, atol=1e-3)
 
 
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("hidden,inter", [(96, 200), (320, 2056), (3584, 18944)])
+def test_swiglu_inside_the_down_product(ops, m, hidden, inter):
+    """The down projection that applies SwiGLU to the gate|up partial sums while staging them
+    gives, bit for bit, what the stand-alone SwiGLU kernel followed by the product gives."""
+    g = torch.Generator().manual_seed(m + inter)
+    gate_up = torch.randn(3, m, 2 * inter, generator=g).to(DEV)
+    w = (torch.randn(hidden, inter, generator=g) * 0.05).bfloat16().to(DEV)
+    assert ops.swiglu_linear_possible(gate_up, w)
+    fused = ops.swiglu_linear(gate_up, w)
+    plain_way = ops.gemm_skinny(ops.swiglu(gate_up, torch.bfloat16), w)
+    assert torch.equal(fused, plain_way)
+    total = gate_up.sum(0).double().cpu()
+    act = torch.nn.functional.silu(total[:, :inter]) * total[:, inter:]
+    want = act.bfloat16().double() @ w.double().cpu().T
+    assert float((fused.sum(0).double().cpu() - want).abs().max()) <= 2e-2 * float(want.abs().max() + 1)
+
+
 def test_consumers_add_up_partial_sums(ops):
     """Norm, SwiGLU and rotary/cache write take the skinny product's 32-bit partial sums and
     give what they give for the summed tensor."""

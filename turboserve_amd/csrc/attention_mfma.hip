@@ -397,37 +397,60 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
 }
 
 // Combine the splits of one (request, head): out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
-// grid (requests, heads), one wavefront: lanes first share the splits (weights), then the head
-// dimensions.
-__global__ void __launch_bounds__(64)
+// grid (requests, heads), 256 threads.  Each thread first owns one split (its weight), then the
+// threads form 1024 / D groups that share the splits between them, a thread adding up four
+// head dimensions (one 16-byte load per split), and the groups' sums meet in LDS.
+constexpr int REDUCE_THREADS = 256;
+static_assert(DECODE_MAX_SPLITS <= REDUCE_THREADS, "one thread per split in the first phase");
+
+__global__ void __launch_bounds__(REDUCE_THREADS)
 decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_acc,
                      const float* __restrict__ partial_ml, const int* __restrict__ query_start_loc,
                      int seq_begin, int heads, int splits) {
+  constexpr int LANES_PER_GROUP = D / 4;
+  constexpr int GROUPS = REDUCE_THREADS / LANES_PER_GROUP;
   __shared__ float weights[DECODE_MAX_SPLITS];
+  __shared__ float sums[GROUPS][D];
+  __shared__ float wave_part[2][REDUCE_THREADS / TS_WAVE];
   const int seq = seq_begin + blockIdx.x;
   const int head = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
+  const int wave = tid / TS_WAVE;
   const size_t base = ((size_t)blockIdx.x * heads + head) * splits;
-  float m_max = -INFINITY;
-  for (int s = lane; s < splits; s += TS_WAVE) m_max = fmaxf(m_max, partial_ml[(base + s) * 2]);
-  m_max = wave_max(m_max);
-  float den = 0.f;
-  for (int s = lane; s < splits; s += TS_WAVE) {
-    const float m = partial_ml[(base + s) * 2];
-    const float wgt = (m == -INFINITY) ? 0.f : exp2f(m - m_max);  // a split past the request's keys
-    weights[s] = wgt;
-    den += partial_ml[(base + s) * 2 + 1] * wgt;
-  }
-  den = wave_sum(den);
+
+  const bool owns = tid < splits;
+  const float m = owns ? partial_ml[(base + tid) * 2] : -INFINITY;
+  const float l = owns ? partial_ml[(base + tid) * 2 + 1] : 0.f;
+  const float wmax = wave_max(m);
+  if ((tid & (TS_WAVE - 1)) == 0) wave_part[0][wave] = wmax;
   __syncthreads();
-  const int token = query_start_loc[seq];
-  uint16_t* orow = out + ((size_t)token * heads + head) * D;
-  const float inv = 1.f / den;
-  for (int d = lane; d < D; d += TS_WAVE) {
+  float m_max = wave_part[0][0];
+#pragma unroll
+  for (int i = 1; i < REDUCE_THREADS / TS_WAVE; ++i) m_max = fmaxf(m_max, wave_part[0][i]);
+  const float wgt = (m == -INFINITY) ? 0.f : exp2f(m - m_max);  // a split past the request's keys
+  if (owns) weights[tid] = wgt;
+  const float wsum = wave_sum(l * wgt);
+  if ((tid & (TS_WAVE - 1)) == 0) wave_part[1][wave] = wsum;
+  __syncthreads();
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < REDUCE_THREADS / TS_WAVE; ++i) den += wave_part[1][i];
+
+  const int g = tid / LANES_PER_GROUP;
+  const int d4 = 4 * (tid % LANES_PER_GROUP);
+  if (g < GROUPS) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = g; sp < splits; sp += GROUPS)
+      acc += *reinterpret_cast<const f32x4*>(partial_acc + (base + sp) * D + d4) * weights[sp];
+    *reinterpret_cast<f32x4*>(&sums[g][d4]) = acc;
+  }
+  __syncthreads();
+  if (tid < D) {
     float num = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < splits; ++s) num = fmaf(partial_acc[(base + s) * D + d], weights[s], num);
-    orow[d] = (uint16_t)bf16_bits(num * inv);
+#pragma unroll
+    for (int i = 0; i < GROUPS; ++i) num += sums[i][tid];
+    const int token = query_start_loc[seq];
+    out[((size_t)token * heads + head) * D + tid] = (uint16_t)bf16_bits(num / den);
   }
 }
 
@@ -872,7 +895,7 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
                      block_table, table_width, query_start_loc, context_lens, seq_begin, heads, kv_heads,
                      shift, scale * LOG2E, window, keys_per_split, splits, max_context);
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
-  hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(64), 0, stream, (uint16_t*)out,
+  hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(REDUCE_THREADS), 0, stream, (uint16_t*)out,
                      (const float*)partial_acc, (const float*)partial_ml, query_start_loc, seq_begin, heads,
                      splits);
   return ts_launch_status();

@@ -189,11 +189,20 @@ gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, 
 // the range is longer than LDS should hold) and its wavefronts then stream their weight rows
 // without meeting at a barrier again, two chunks of loads in flight each.  mpad is 8 or 16;
 // lanes whose activation row is beyond mpad read a real row again and drop the result.
-template <int WAVES>
+//
+// GATED: the activations do not exist yet.  `x` then points at the 32-bit partial sums
+// [gated_splits, m, 2 k] of a fused gate|up projection (row stride x_stride, splits
+// gated_stride elements apart) and the staging computes silu(gate) * up from them, rounded to
+// bfloat16 once, exactly as the stand-alone SwiGLU kernel does: one kernel and one pass over
+// that intermediate fewer per layer.
+template <int WAVES, bool GATED>
 __global__ void __launch_bounds__(WAVES * TS_WAVE)
-gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
-                            const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int mpad,
-                            int n, int k, int chunks_per_split, int stage_chunks) {
+gemm_skinny_resident_kernel(float* __restrict__ partial, const void* __restrict__ x_any, long x_stride,
+                            int gated_splits, long gated_stride, const uint16_t* __restrict__ w,
+                            const uint16_t* __restrict__ bias, int m, int mpad, int n, int k, int chunks_per_split,
+                            int stage_chunks) {
+  const uint16_t* x = static_cast<const uint16_t*>(x_any);
+  const float* xg = static_cast<const float*>(x_any);
   extern __shared__ __attribute__((aligned(16))) uint16_t xs_resident[];
   const int lane = threadIdx.x & (TS_WAVE - 1);
   const int wave = threadIdx.x / TS_WAVE;
@@ -227,8 +236,33 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restr
         const int piece = idx - row * pieces_per_row;
         if (piece >= live_pieces) continue;
         const int kk = k_begin + 8 * piece;
-        const u32x4 v = (row < m && kk < k) ? *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + kk)
-                                            : u32x4{0u, 0u, 0u, 0u};
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row < m && kk < k) {
+          if (GATED) {
+            float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < gated_splits; ++sp) {
+              const float* src = xg + (size_t)sp * gated_stride + (size_t)row * x_stride + kk;
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(src + 4 * h);
+                const f32x4 b = *reinterpret_cast<const f32x4*>(src + k + 4 * h);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  g[4 * h + e] += a[e];
+                  u[4 * h + e] += b[e];
+                }
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float lo = g[2 * e] / (1.f + expf(-g[2 * e])) * u[2 * e];
+              const float hi = g[2 * e + 1] / (1.f + expf(-g[2 * e + 1])) * u[2 * e + 1];
+              v[e] = (uint32_t)from_float<bf16_t>(lo).bits | ((uint32_t)from_float<bf16_t>(hi).bits << 16);
+            }
+          } else {
+            v = *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + kk);
+          }
+        }
         *reinterpret_cast<u32x4*>(xs_resident + row * x_row + 8 * piece) = v;
       }
       __syncthreads();
@@ -313,12 +347,18 @@ extern "C" int ts_gemm_skinny(float* partial, const void* x, long x_stride, cons
 // The variant for m <= 16 that keeps a split's activations in LDS (see the kernel).  stage_chunks:
 // chunks staged at a time, an even number unless it covers a whole split; the LDS it needs,
 // mpad * (min(stage_chunks, chunks_per_split) * 256 + 8) * 2 bytes with mpad = 8 or 16, must be <= 64 KiB.
-extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
-                                       int m, int n, int k, int chunks_per_split, int splits, int waves,
-                                       int stage_chunks, hipStream_t stream) {
+// gated_splits == 0: x is bfloat16 [m, k].  gated_splits >= 1: x is float [gated_splits, m, 2 k]
+// (splits gated_stride elements apart), the partial sums of a gate|up projection, and the
+// product's left operand is silu(gate) * up (k % 8 == 0, x_stride >= 2 k, no bias).
+static int skinny_resident(float* partial, const void* x, long x_stride, int gated_splits, long gated_stride,
+                           const void* w, const void* bias, int m, int n, int k, int chunks_per_split, int splits,
+                           int waves, int stage_chunks, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
-  if (m > 16 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
+  const bool gated = gated_splits > 0;
+  if (m > 16 || (k & 7) != 0 || x_stride < (gated ? 2L * k : (long)k) || (x_stride & (gated ? 3 : 7)) != 0)
+    return TS_ERR_SHAPE;
+  if (gated && (bias || (gated_stride & 3) != 0)) return TS_ERR_ARG;
   const int total_chunks = (k + CHUNK - 1) / CHUNK;
   if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
   if (stage_chunks < 1 || (stage_chunks < chunks_per_split && (stage_chunks & 1) != 0)) return TS_ERR_SHAPE;
@@ -326,17 +366,33 @@ extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_str
   const int stage = stage_chunks < chunks_per_split ? stage_chunks : chunks_per_split;
   const size_t lds = (size_t)mpad * (stage * CHUNK + 8) * sizeof(uint16_t);
   if (lds > 64 * 1024 || splits > 65535) return TS_ERR_SHAPE;
-  const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (waves == 4) {
-    dim3 grid((n + 63) / 64, splits), block(4 * TS_WAVE);
-    hipLaunchKernelGGL((gemm_skinny_resident_kernel<4>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks);
-  } else if (waves == 8) {
-    dim3 grid((n + 127) / 128, splits), block(8 * TS_WAVE);
-    hipLaunchKernelGGL((gemm_skinny_resident_kernel<8>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks);
-  } else {
-    return TS_ERR_SHAPE;
-  }
+  if (waves != 4 && waves != 8) return TS_ERR_SHAPE;
+  dim3 grid((n + 16 * waves - 1) / (16 * waves), splits), block(waves * TS_WAVE);
+#define TS_LAUNCH_RESIDENT(W, G)                                                                                   \
+  hipLaunchKernelGGL((gemm_skinny_resident_kernel<W, G>), grid, block, lds, stream, partial, x, x_stride,         \
+                     gated_splits, gated_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks)
+  if (waves == 4 && !gated) TS_LAUNCH_RESIDENT(4, false);
+  else if (waves == 8 && !gated) TS_LAUNCH_RESIDENT(8, false);
+  else if (waves == 4) TS_LAUNCH_RESIDENT(4, true);
+  else TS_LAUNCH_RESIDENT(8, true);
+#undef TS_LAUNCH_RESIDENT
   return ts_launch_status();
+}
+
+extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
+                                       int m, int n, int k, int chunks_per_split, int splits, int waves,
+                                       int stage_chunks, hipStream_t stream) {
+  return skinny_resident(partial, x, x_stride, 0, 0, w, bias, m, n, k, chunks_per_split, splits, waves, stage_chunks,
+                         stream);
+}
+
+extern "C" int ts_gemm_skinny_resident_gated(float* partial, const float* gate_up, long row_stride, int gated_splits,
+                                             long gated_stride, const void* w, int m, int n, int k,
+                                             int chunks_per_split, int splits, int waves, int stage_chunks,
+                                             hipStream_t stream) {
+  if (gated_splits < 1) return TS_ERR_ARG;
+  return skinny_resident(partial, gate_up, row_stride, gated_splits, gated_stride, w, nullptr, m, n, k,
+                         chunks_per_split, splits, waves, stage_chunks, stream);
 }

@@ -56,6 +56,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                            c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_void_p],
+        "ts_gemm_skinny_resident_gated": [c_void_p, c_void_p, c_long, c_int, c_long, c_void_p, c_int, c_int, c_int,
+                                          c_int, c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -494,6 +496,48 @@ class Ops:
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= 64
                 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0)
 
+    def _resident_plan(self, m: int, n: int, chunks: int, max_splits: int | None) -> tuple[int, int, int, int]:
+        """(chunks per split, splits, wavefronts per workgroup, chunks staged at a time) of the
+        skinny product with resident activations: splits sized for a number of wavefronts."""
+        limit = min(chunks, max_splits or self.skinny_max_splits)
+        want = max(1, min(limit, -(-self.skinny_resident_waves // -(-n // 16))))
+        per_split = -(-chunks // want)
+        splits = -(-chunks // per_split)
+        waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 1024) else 4)
+        return per_split, splits, waves, self.skinny_stage_chunks[0 if m <= 8 else 1]
+
+    #: Up to this many rows a feed-forward hands the gate|up partial sums straight to the down
+    #: product, which applies SwiGLU while staging its activations (one kernel fewer per layer).
+    #: Every workgroup of that product redoes the activation for its range of K, which at 8 rows
+    #: already costs more than the kernel it saves (measured at the 7B shape).
+    swiglu_fuse_rows = int(os.environ.get("TS_FUSE_SWIGLU_ROWS", "4"))
+
+    def swiglu_linear_possible(self, gate_up: torch.Tensor, weight: torch.Tensor) -> bool:
+        """Whether :meth:`swiglu_linear` takes these operands at all."""
+        return (gate_up.dim() == 3 and gate_up.dtype == torch.float32 and weight.dtype == torch.bfloat16
+                and gate_up.shape[1] <= self.skinny_resident_rows and gate_up.shape[2] == 2 * weight.shape[1]
+                and weight.shape[1] % 8 == 0 and gate_up.is_contiguous())
+
+    def swiglu_linear_supported(self, gate_up: torch.Tensor, weight: torch.Tensor) -> bool:
+        """Whether a feed-forward should use :meth:`swiglu_linear` for these operands."""
+        return self.swiglu_linear_possible(gate_up, weight) and gate_up.shape[1] <= self.swiglu_fuse_rows
+
+    def swiglu_linear(self, gate_up: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """``[S', M, N]`` 32-bit partial sums of ``(silu(gate) * up) @ weight^T`` from the 32-bit
+        partial sums ``gate_up [S, M, 2 I]`` of a fused gate|up projection: what :meth:`swiglu`
+        followed by :meth:`gemm_skinny` gives, bit for bit, in one kernel."""
+        _gpu(gate_up, weight)
+        _need(self.swiglu_linear_possible(gate_up, weight) and weight.is_contiguous(),
+              "swiglu_linear takes contiguous 32-bit partial sums [S, M <= 16, 2 I] and a bfloat16 weight [N, I]")
+        gated_splits, m, width = gate_up.shape
+        n, k = weight.shape
+        per_split, splits, waves, stage = self._resident_plan(m, n, -(-k // 256), None)
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=gate_up.device)
+        _check(self.core.ts_gemm_skinny_resident_gated(_ptr(partial), _ptr(gate_up), width, gated_splits, m * width,
+                                                       _ptr(weight), m, n, k, per_split, splits, waves, stage,
+                                                       self.stream()), "ts_gemm_skinny_resident_gated")
+        return partial
+
     def gemm_skinny(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                     *, max_splits: int | None = None) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
@@ -509,13 +553,7 @@ class Ops:
         chunks = -(-k // 256)
         x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
         if m <= self.skinny_resident_rows:
-            # Activations resident in LDS, no barrier per chunk: splits sized for a number of wavefronts.
-            limit = min(chunks, max_splits or self.skinny_max_splits)
-            want = max(1, min(limit, -(-self.skinny_resident_waves // -(-n // 16))))
-            per_split = -(-chunks // want)
-            splits = -(-chunks // per_split)
-            waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 1024) else 4)
-            stage = self.skinny_stage_chunks[0 if m <= 8 else 1]
+            per_split, splits, waves, stage = self._resident_plan(m, n, chunks, max_splits)
             partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
             _check(self.core.ts_gemm_skinny_resident(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias),
                                                      m, n, k, per_split, splits, waves, stage, self.stream()),

@@ -146,9 +146,16 @@ __device__ __forceinline__ WindowPages window_pages(const PageGeometry& g, int w
 }
 
 // Page of `key`, a key of the window starting at w (a block of 32 keys or more: always the first).
+// The ids are copied to vector registers first (the empty asm pins them there): selecting
+// among scalar registers per lane, the compiler builds a tree of divergent branches instead of
+// three v_cndmask.
 __device__ __forceinline__ long long page_of(const PageGeometry& g, const WindowPages& wp, int w, int key) {
+  int p0 = wp.page[0], p1 = wp.page[1], p2 = wp.page[2], p3 = wp.page[3];
+  asm("" : "+v"(p0), "+v"(p1), "+v"(p2), "+v"(p3));
   const int i = (key - w) >> g.block_shift;
-  return i == 0 ? wp.page[0] : (i == 1 ? wp.page[1] : (i == 2 ? wp.page[2] : wp.page[3]));
+  const int low = (i & 1) ? p1 : p0;
+  const int high = (i & 1) ? p3 : p2;
+  return (i & 2) ? high : low;
 }
 
 // A key outside lo..last is replaced by the nearest live key of its window (every window that
@@ -539,116 +546,73 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
 
 
 // ---------------------------------------------------------------------------------------------
-// prefill with shared windows: grid (query blocks, kv_heads * head_chunks), HW wavefronts per
-// workgroup.  Wavefront i handles query head (chunk * HW + i) of the KV head for the block's 16
-// tokens; all of them see the same keys, so each 32-key window is fetched from the pages once
-// per workgroup, staged in LDS (double-buffered, rows padded so that the 16 lanes of one LDS
-// pass hit distinct banks) and read from there as matrix-core operands by every wavefront.
-// Window w + 1 travels from global memory to registers while window w is computed.
+// prefill with shared windows: one workgroup of four wavefronts per (query block, KV head, chunk
+// of its query heads).  Each wavefront handles CT query heads for the block's 16 tokens; all of
+// them see the same keys, so each 32-key window is fetched from the pages once per workgroup,
+// staged in LDS (double-buffered; rows padded and key rows permuted so that the 16 lanes of one
+// LDS pass hit distinct banks) and read from there as matrix-core operands by every wavefront.
+// Windows travel global memory -> registers (a ring, two or three windows in flight) -> LDS.
 // ---------------------------------------------------------------------------------------------
 constexpr int K_ROW = D + 8;              // LDS stride of a key row (elements)
 constexpr int V_ROW = WINDOW_KEYS + 8;    // LDS stride of a head dimension's 32 values
 constexpr int K_TILE = WINDOW_KEYS * K_ROW;
 constexpr int V_TILE = D * V_ROW;
-constexpr int K_PIECES = WINDOW_KEYS * (D / 8);  // 16-byte pieces of a window's keys
-constexpr int V_PIECES = D * (WINDOW_KEYS / 8);  // and of its values
 
-template <int HW>
+// How a workgroup of four wavefronts divides a window between them: wavefront i fetches the
+// keys 8 i .. 8 i + 7 (whole rows) and the values of the same eight keys (one 16-byte chunk per
+// head dimension).  Eight aligned keys lie in one page, so a wavefront needs one page id per
+// window, a scalar load, and its addresses are a scalar base plus a per-lane constant.
+constexpr int STAGE_WAVES = 4;
+constexpr int KEYS_PER_WAVE = WINDOW_KEYS / STAGE_WAVES;
+static_assert(KEYS_PER_WAVE == 8, "a wavefront's keys must be one aligned group of eight");
+constexpr int K_WAVE_PIECES = KEYS_PER_WAVE * (D / 8);                   // 16-byte pieces of eight key rows
+constexpr int K_EACH = (K_WAVE_PIECES + TS_WAVE - 1) / TS_WAVE;          // per lane
+constexpr int V_EACH = (D + TS_WAVE - 1) / TS_WAVE;                      // head dimensions per lane
+
 struct StagedWindow {
-  static constexpr int THREADS = HW * TS_WAVE;
-  static constexpr int K_EACH = (K_PIECES + THREADS - 1) / THREADS;
-  static constexpr int V_EACH = (V_PIECES + THREADS - 1) / THREADS;
-  static constexpr int PIECES = K_EACH + V_EACH;
   u32x4 k[K_EACH];
   u32x4 v[V_EACH];
 };
 
-// What a thread's pieces have in common in every window, worked out once: which of the
-// window's pages a piece lies in, its byte address but for the page's own offset, and where it
-// goes in LDS.  Per window that leaves a select of the page id and one multiply-add per piece.
-template <int HW>
-struct PiecePlan {
-  using W = StagedWindow<HW>;
-  int k_sel[W::K_EACH];
-  unsigned long long k_base[W::K_EACH];
-  int k_lds[W::K_EACH];  // element offset in the staged key tile, -1: a spare thread
-  int v_sel[W::V_EACH];
-  unsigned long long v_base[W::V_EACH];
-  int v_lds[W::V_EACH];
-  unsigned page_bytes;  // bytes from one page of the pool to the next
-};
-
-template <int HW>
-__device__ __forceinline__ void plan_pieces(PiecePlan<HW>& plan, const PageGeometry& g) {
-  using W = StagedWindow<HW>;
-  plan.page_bytes = (unsigned)((g.kv_heads << g.block_shift) * D * 2);
-  const unsigned long long head_bytes = (unsigned long long)((g.kvh << g.block_shift) * D) * 2;
-#pragma unroll
-  for (int i = 0; i < W::K_EACH; ++i) {
-    const int raw = threadIdx.x + i * W::THREADS;
-    const int idx = min(raw, K_PIECES - 1);  // spare threads repeat the last piece
-    const int ko = idx / (D / 8);
-    const int col = 8 * (idx % (D / 8));
-    plan.k_sel[i] = ko >> g.block_shift;
-    plan.k_base[i] = (unsigned long long)g.k_pages + head_bytes + (unsigned long long)((ko & g.block_mask) * D + col) * 2;
-    // Key offset ko of the window goes to the row the score tiles read it from: tile
-    // t = (ko / 4) % 2, row m = 4 (ko / 8) + ko % 4, stored at 16 t + m, so that the 16 lanes
-    // of an LDS pass read 16 consecutive rows (distinct banks with the padded stride).
-    const int slot = 16 * ((ko >> 2) & 1) + ((ko >> 3) << 2) + (ko & 3);
-    plan.k_lds[i] = raw < K_PIECES ? slot * K_ROW + col : -1;
-  }
-#pragma unroll
-  for (int i = 0; i < W::V_EACH; ++i) {
-    const int raw = threadIdx.x + i * W::THREADS;
-    const int idx = min(raw, V_PIECES - 1);
-    const int d = idx / (WINDOW_KEYS / 8);
-    const int kc = 8 * (idx % (WINDOW_KEYS / 8));
-    plan.v_sel[i] = kc >> g.block_shift;
-    plan.v_base[i] = (unsigned long long)g.v_pages + head_bytes +
-                     (unsigned long long)((d << g.block_shift) + (kc & g.block_mask)) * 2;
-    plan.v_lds[i] = raw < V_PIECES ? d * V_ROW + kc : -1;
-  }
-}
-
 // Issue the loads of this thread's pieces of window `w`.  Nothing here looks at what the loads
 // bring, so they stay in flight until the window is staged.  A window wholly inside lo..last
-// takes the planned addresses; one at the edge replaces keys outside lo..last (see live_key).
-template <int HW>
-__device__ __forceinline__ void fetch_window(StagedWindow<HW>& r, const PiecePlan<HW>& plan, const PageGeometry& g,
-                                             int w, int lo, int last) {
-  using W = StagedWindow<HW>;
-  const WindowPages wp = window_pages(g, w);
+// takes the scalar path; one at the edge replaces keys outside lo..last (see live_key), whose
+// pages it looks up per lane.
+__device__ __forceinline__ void fetch_window(StagedWindow& r, const PageGeometry& g, int w, int lo, int last, int wave,
+                                             int lane) {
+  const int first_key = w + KEYS_PER_WAVE * wave;  // the same in every lane of the wavefront
   if (w >= lo && w + WINDOW_KEYS - 1 <= last) {
-    // A block of more than 32 keys holds the window at offset w % block size.
-    const unsigned long long k_in_page = (unsigned long long)((w & g.block_mask) * D) * 2;
-    const unsigned long long v_in_page = (unsigned long long)(w & g.block_mask) * 2;
+    const long long page = g.table[__builtin_amdgcn_readfirstlane(first_key) >> g.block_shift];
+    const long long head = ((page * g.kv_heads + g.kvh) << g.block_shift) * D;
+    const uint16_t* kbase = g.k_pages + head + (long long)(first_key & g.block_mask) * D;
+    const uint16_t* vbase = g.v_pages + head + (first_key & g.block_mask);
 #pragma unroll
-    for (int i = 0; i < W::K_EACH; ++i) {
-      const int sel = plan.k_sel[i];
-      const unsigned page = sel == 0 ? wp.page[0] : (sel == 1 ? wp.page[1] : (sel == 2 ? wp.page[2] : wp.page[3]));
-      r.k[i] = load8(reinterpret_cast<const uint16_t*>(plan.k_base[i] + ((unsigned long long)page * plan.page_bytes + k_in_page)));
+    for (int i = 0; i < K_EACH; ++i) {
+      const int piece = min(lane + i * TS_WAVE, K_WAVE_PIECES - 1);  // spare lanes repeat the last piece
+      r.k[i] = load8(kbase + 8 * piece);                             // eight rows of D are contiguous
     }
 #pragma unroll
-    for (int i = 0; i < W::V_EACH; ++i) {
-      const int sel = plan.v_sel[i];
-      const unsigned page = sel == 0 ? wp.page[0] : (sel == 1 ? wp.page[1] : (sel == 2 ? wp.page[2] : wp.page[3]));
-      r.v[i] = load8(reinterpret_cast<const uint16_t*>(plan.v_base[i] + ((unsigned long long)page * plan.page_bytes + v_in_page)));
+    for (int i = 0; i < V_EACH; ++i) {
+      const int d = min(lane + i * TS_WAVE, D - 1);
+      r.v[i] = load8(vbase + ((long long)d << g.block_shift));
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < W::K_EACH; ++i) {
-      const int idx = min((int)threadIdx.x + i * W::THREADS, K_PIECES - 1);
-      const int key = w + idx / (D / 8);
-      r.k[i] = load8(key_row(g, wp, w, live_key(key, w, lo, last)) + 8 * (idx % (D / 8)));
+    for (int i = 0; i < K_EACH; ++i) {
+      const int piece = min(lane + i * TS_WAVE, K_WAVE_PIECES - 1);
+      const int key = live_key(first_key + piece / (D / 8), w, lo, last);
+      const long long page = g.table[key >> g.block_shift];
+      r.k[i] = load8(g.k_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D +
+                     (long long)(key & g.block_mask) * D + 8 * (piece % (D / 8)));
     }
+    const bool live = first_key + 7 >= lo && first_key <= last;
+    const int chunk = live ? first_key : (live_key(first_key, w, lo, last) & ~7);
+    const long long page = g.table[chunk >> g.block_shift];
+    const uint16_t* vbase = g.v_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D + (chunk & g.block_mask);
 #pragma unroll
-    for (int i = 0; i < W::V_EACH; ++i) {
-      const int idx = min((int)threadIdx.x + i * W::THREADS, V_PIECES - 1);
-      const int d = idx / (WINDOW_KEYS / 8);
-      const int chunk = w + 8 * (idx % (WINDOW_KEYS / 8));
-      const bool live = chunk + 7 >= lo && chunk <= last;
-      r.v[i] = load8(value_chunk(g, wp, w, live ? chunk : (live_key(chunk, w, lo, last) & ~7)) +
-                     ((long long)d << g.block_shift));
+    for (int i = 0; i < V_EACH; ++i) {
+      const int d = min(lane + i * TS_WAVE, D - 1);
+      r.v[i] = load8(vbase + ((long long)d << g.block_shift));
     }
   }
 }
@@ -656,21 +620,28 @@ __device__ __forceinline__ void fetch_window(StagedWindow<HW>& r, const PiecePla
 // Write the fetched window `w` to LDS.  Values of keys outside lo..last are whatever an earlier
 // owner of the page left: they are cleared here, so that a stale non-finite value cannot meet a
 // zero probability (only a window that is not wholly inside lo..last needs it).
-template <int HW>
-__device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const StagedWindow<HW>& r,
-                                             const PiecePlan<HW>& plan, int w, int lo, int last) {
-  using W = StagedWindow<HW>;
+__device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const StagedWindow& r, int w, int lo, int last,
+                                             int wave, int lane) {
 #pragma unroll
-  for (int i = 0; i < W::K_EACH; ++i)
-    if (plan.k_lds[i] >= 0) *reinterpret_cast<u32x4*>(ks + plan.k_lds[i]) = r.k[i];
+  for (int i = 0; i < K_EACH; ++i) {
+    const int piece = lane + i * TS_WAVE;
+    if (piece < K_WAVE_PIECES) {
+      // Key offset ko of the window goes to the row the score tiles read it from: tile
+      // t = (ko / 4) % 2, row m = 4 (ko / 8) + ko % 4, stored at 16 t + m, so that the 16 lanes
+      // of an LDS pass read 16 consecutive rows (distinct banks with the padded stride).
+      const int ko = KEYS_PER_WAVE * wave + piece / (D / 8);
+      const int slot = 16 * ((ko >> 2) & 1) + ((ko >> 3) << 2) + (ko & 3);
+      *reinterpret_cast<u32x4*>(ks + slot * K_ROW + 8 * (piece % (D / 8))) = r.k[i];
+    }
+  }
+  const int chunk = w + KEYS_PER_WAVE * wave;
   const bool edge = w < lo || w + WINDOW_KEYS - 1 > last;
 #pragma unroll
-  for (int i = 0; i < W::V_EACH; ++i) {
-    if (plan.v_lds[i] < 0) continue;
+  for (int i = 0; i < V_EACH; ++i) {
+    const int d = lane + i * TS_WAVE;
+    if (d >= D) continue;
     u32x4 value = r.v[i];
     if (edge) {
-      const int idx = threadIdx.x + i * W::THREADS;
-      const int chunk = w + 8 * (idx % (WINDOW_KEYS / 8));
       const bool live = chunk + 7 >= lo && chunk <= last;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -679,7 +650,7 @@ __device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const S
         value[e] &= low | high;
       }
     }
-    *reinterpret_cast<u32x4*>(vs + plan.v_lds[i]) = value;
+    *reinterpret_cast<u32x4*>(vs + d * V_ROW + KEYS_PER_WAVE * wave) = value;
   }
 }
 
@@ -698,8 +669,8 @@ __device__ __forceinline__ void read_values(ValueFrags& f, const uint16_t* vs, i
   for (int n = 0; n < NT; ++n) f.v[n] = load8(vs + (16 * n + lane16) * V_ROW + 8 * group);
 }
 
-template <int HW, int CT>
-__global__ void __launch_bounds__(HW * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int CT>
+__global__ void __launch_bounds__(STAGE_WAVES * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
 prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
                       const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                       const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
@@ -713,6 +684,7 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
   const int lane16 = lane & 15;
   const int group = lane >> 4;
   const int gsize = heads / kv_heads;
+  constexpr int HW = STAGE_WAVES;
   const int head_chunks = (gsize + HW * CT - 1) / (HW * CT);
   // Workgroup id -> (block, KV head and chunk of its query heads), the latter fastest.  Blocks
   // come heaviest first.  With pair_blocks (the host sets it when all workgroups are resident
@@ -758,18 +730,16 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
   // Windows travel global memory -> registers -> LDS.  A ring of P register sets keeps the
   // loads of P windows in flight, so a load has P - 1 rounds of computing to arrive in; LDS
   // holds two windows (the one being read, the next being written).
-  constexpr int P = StagedWindow<HW>::PIECES * CT <= 4 ? 3 : 2;
-  StagedWindow<HW> ring[P];
-  PiecePlan<HW> plan;
-  plan_pieces<HW>(plan, geo);
+  constexpr int P = (K_EACH + V_EACH) * CT <= 4 ? 3 : 2;
+  StagedWindow ring[P];
   // Every round issues its fetch, past the last window too (that window again, dropped): with a
   // fetch that may or may not have been issued the compiler cannot count the loads in flight
   // and waits for all of them before each staging.
   const int last_window = (end - 1) & ~(WINDOW_KEYS - 1);
 #pragma unroll
   for (int u = 0; u < P; ++u)
-    fetch_window<HW>(ring[u], plan, geo, min(begin + u * WINDOW_KEYS, last_window), lo_first, p_last);
-  stage_window<HW>(ks, vs, ring[0], plan, begin, lo_first, p_last);
+    fetch_window(ring[u], geo, min(begin + u * WINDOW_KEYS, last_window), lo_first, p_last, wave, lane);
+  stage_window(ks, vs, ring[0], begin, lo_first, p_last, wave, lane);
   __syncthreads();
   int buf = 0;
   int w = begin;
@@ -777,7 +747,7 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
 #pragma unroll
     for (int u = 0; u < P; ++u) {
       // ring[u] held window w, which is staged: refill it with the window P rounds ahead.
-      fetch_window<HW>(ring[u], plan, geo, min(w + P * WINDOW_KEYS, last_window), lo_first, p_last);
+      fetch_window(ring[u], geo, min(w + P * WINDOW_KEYS, last_window), lo_first, p_last, wave, lane);
       if (wave_live) {
         // Keys first, values only once the probabilities stand: the two sets of operands are
         // never in registers together.
@@ -801,8 +771,8 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
         for (int c = 0; c < CT; ++c) accumulate(st[c], vf, prob[c], alpha[c]);
       }
       if (w + WINDOW_KEYS < end)  // the other LDS window was last read a round ago
-        stage_window<HW>(ks + (buf ^ 1) * K_TILE, vs + (buf ^ 1) * V_TILE, ring[(u + 1) % P], plan,
-                         w + WINDOW_KEYS, lo_first, p_last);
+        stage_window(ks + (buf ^ 1) * K_TILE, vs + (buf ^ 1) * V_TILE, ring[(u + 1) % P], w + WINDOW_KEYS, lo_first,
+                     p_last, wave, lane);
       __syncthreads();
       buf ^= 1;
       w += WINDOW_KEYS;
@@ -826,7 +796,7 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
   }
 }
 
-template <int HW, int CT>
+template <int CT>
 static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16_t* q, long q_stride,
                                  const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
                                  int table_width, const int* query_start_loc, const int* context_lens,
@@ -837,12 +807,13 @@ static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16
   if (lds > 48 * 1024) {
     static bool raised = false;  // per process; the attribute belongs to the kernel
     if (!raised) {
-      if (hipFuncSetAttribute((const void*)prefill_shared_kernel<HW, CT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+      if (hipFuncSetAttribute((const void*)prefill_shared_kernel<CT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)lds) != hipSuccess)
         return TS_ERR_LAUNCH;
       raised = true;
     }
   }
+  constexpr int HW = STAGE_WAVES;
   const int gsize = heads / kv_heads;
   const int chunks = (gsize + HW * CT - 1) / (HW * CT);
   const long long total = (long long)num_blocks * kv_heads * chunks;
@@ -858,7 +829,7 @@ static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16
     compute_units = prop.multiProcessorCount;
   }
   const int pair_blocks = total <= 2LL * compute_units ? 1 : 0;
-  hipLaunchKernelGGL((prefill_shared_kernel<HW, CT>), dim3((unsigned)total), dim3(HW * TS_WAVE), lds, stream, out, q,
+  hipLaunchKernelGGL((prefill_shared_kernel<CT>), dim3((unsigned)total), dim3(HW * TS_WAVE), lds, stream, out, q,
                      q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks,
                      num_blocks, pair_blocks, heads, kv_heads, shift, scale_log2, window);
   return ts_launch_status();
@@ -920,10 +891,10 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   // share every window of keys and values through LDS.
   if (gsize >= 3) {
     if (gsize >= 5)
-      return launch_prefill_shared<4, 2>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
+      return launch_prefill_shared<2>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                          (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
                                          context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
-    return launch_prefill_shared<4, 1>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
+    return launch_prefill_shared<1>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                        (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
                                        context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
   }

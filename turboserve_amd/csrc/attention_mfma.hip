@@ -3,8 +3,8 @@
 //
 // Both kernels compute, for 16 "columns" at a time, S^T = K Q^T (rows: keys, columns: queries)
 // with v_mfma_f32_16x16x32_bf16, an online softmax over 32-key windows in the accumulator
-// layout, and O^T = V^T P^T with the same instruction.  Two choices make that work without any
-// staging through LDS:
+// layout, and O^T = V^T P^T with the same instruction.  Two choices let a wavefront feed the
+// matrix cores straight from what it loaded, with no transposition in between:
 //   * value pages are stored transposed ([NB, Hkv, D, BS]), so the A operand of the second
 //     product (8 consecutive keys of one head dimension per lane) is one 16-byte load;
 //   * the rows of the two 16-key score tiles of a window are assigned to keys so that a lane's
@@ -20,9 +20,11 @@
 // (src/turboserve/engine/model/triton_attention.py:110-174) and, with a window, keeps only
 // the keys p - window + 1 .. p.
 //
-// Prefill kernel: the 16 columns are 16 consecutive tokens of one request's portion, for one
-// query head; up to PF_HEADS heads of the same KV head share each loaded window.  Column j at
-// position p_j sees keys lo_j..p_j (src/turboserve/engine/model/attention.py:139-148).
+// Prefill kernels: the 16 columns are 16 consecutive tokens of one request's portion, for one
+// query head.  Column j at position p_j sees keys lo_j..p_j
+// (src/turboserve/engine/model/attention.py:139-148).  With three or more query heads per KV
+// head a workgroup of four wavefronts shares every window through LDS (prefill_shared_kernel);
+// with fewer, one wavefront serves two heads from registers alone (prefill_kernel).
 #include "common.hpp"
 
 #ifndef TS_HEAD_DIM

@@ -196,3 +196,35 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
     for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
         want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
         assert abs(got - want) <= 0.05, (i, got, want)
+
+
+def test_command_line_generates_the_plain_tokens(tmp_path):
+    """`turboserve engine random-model` writes a model folder and `turboserve engine generate
+    --prompt-ids` (no tokenizer there) prints, per prompt, the greedy tokens of the plain
+    implementation; `kv-size` prints its sizing as JSON."""
+    import json
+    import re
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(tiny.CONFIG_A))
+    folder = tmp_path / "model"
+    run = lambda *args: subprocess.run([sys.executable, str(root / "bin" / "turboserve"), *args], capture_output=True,
+                                       text=True, timeout=240)
+    made = run("engine", "random-model", "--config", str(config_file), "--out", str(folder), "--seed", "3",
+               "--dtype", "float32")
+    assert made.returncode == 0, made.stderr
+    raw, tensors = tiny.read_model_dir(folder)
+    prompts = [[5, 17, 3, 200], [9, 9, 9, 9, 9, 9, 1]]
+    out = run("engine", "generate", "--model", str(folder), "--dtype", "float32", "--max-tokens", "6", "--ignore-eos",
+              "--num-blocks", "16", "--stats", *[a for p in prompts for a in ("--prompt-ids", ",".join(map(str, p)))])
+    assert out.returncode == 0, out.stderr
+    shown = [json.loads(m) for m in re.findall(r"^output \d+: (\[.*\])$", out.stdout, flags=re.M)]
+    assert shown == [plain.greedy_generate(raw, tensors, p, 6) for p in prompts]
+    assert "2 completions in" in out.stdout and "finish_reason=length" in out.stdout
+    sizing = run("engine", "kv-size", "--model", str(folder), "--dtype", "float32", "--max-model-len", "64")
+    assert sizing.returncode == 0, sizing.stderr
+    assert min(json.loads(sizing.stdout[sizing.stdout.index("{"):])["num_blocks"]) >= 1  # one pool per cache group

@@ -1,6 +1,7 @@
 """The parts of a model, alone and recombined: each built-in part against the plain
-implementation; a toy mixer with state of its own and a toy architecture, defined here and
-registered without touching the framework; a run order that names a layer twice and lets a
+implementation; a toy mixer with state of its own, a toy feed-forward with routing, a toy
+position encoding and a toy architecture made of them, all defined here and registered
+without touching the framework; a run order that names a layer twice and lets a
 layer read another layer's cache; long decoding and the first tokens of a sequence."""
 
 from __future__ import annotations
@@ -135,7 +136,7 @@ def register_toy_architecture():
     from turboserve_amd.config import registry as arch_registry
     from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
     from turboserve_amd.parts import registry as part_registry
-    from turboserve_amd.parts.base import FixedState, Mixer, PartSpec, TensorSpec
+    from turboserve_amd.parts.base import FeedForward, FixedState, Mixer, PartSpec, PositionEncoding, TensorSpec
 
     if "running_mean" not in part_registry.MIXERS:
 
@@ -171,6 +172,69 @@ def register_toy_architecture():
                     row += count
                 return out
 
+    if "top1_experts" not in part_registry.FEED_FORWARDS:
+
+        @part_registry.register_feed_forward("top1_experts")
+        class Top1Experts(FeedForward):
+            """A feed-forward with routing: 32-bit router logits pick one SwiGLU expert per token."""
+
+            def __init__(self, prefix, runtime, *, hidden_size, intermediate_size, num_experts):
+                super().__init__(prefix, runtime)
+                self.hidden, self.inter, self.experts = hidden_size, intermediate_size, num_experts
+                self.router = None
+                self.weights = []
+
+            def tensor_specs(self):
+                specs = {self.name("router.weight"): TensorSpec((self.experts, self.hidden), kind="float_keep32")}
+                for e in range(self.experts):
+                    specs[self.name(f"experts.{e}.gate_proj.weight")] = TensorSpec((self.inter, self.hidden))
+                    specs[self.name(f"experts.{e}.up_proj.weight")] = TensorSpec((self.inter, self.hidden))
+                    specs[self.name(f"experts.{e}.down_proj.weight")] = TensorSpec((self.hidden, self.inter))
+                return specs
+
+            def load(self, tensors):
+                self.router = tensors[self.name("router.weight")].float()
+                self.weights = [tuple(tensors[self.name(f"experts.{e}.{n}_proj.weight")] for n in ("gate", "up", "down"))
+                                for e in range(self.experts)]
+
+            def forward(self, x, ctx):
+                # Every expert on every row, the chosen one kept: nothing is read back to the
+                # host, so the step stays recordable into a HIP graph (a toy may be wasteful).
+                choice = (x.float() @ self.router.t()).argmax(dim=-1)
+                out = torch.zeros_like(x)
+                for e, (gate, up, down) in enumerate(self.weights):
+                    act = torch.nn.functional.silu(x @ gate.t()) * (x @ up.t())
+                    out = torch.where((choice == e)[:, None], act @ down.t(), out)
+                return out
+
+    if "learned_positions" not in part_registry.POSITION_ENCODINGS:
+
+        @part_registry.register_position_encoding("learned_positions")
+        class LearnedPositions(PositionEncoding):
+            """Another position encoding: a learned vector per position, added to every head's
+            query and key before the keys are stored (no rotation)."""
+
+            def __init__(self, prefix, runtime, *, head_dim, max_positions):
+                super().__init__(prefix, runtime)
+                self.head_dim, self.max_positions = head_dim, max_positions
+                self.table = None
+
+            def tensor_specs(self):
+                return {self.name("position_table"): TensorSpec((self.max_positions, self.head_dim))}
+
+            def load(self, tensors):
+                self.table = tensors[self.name("position_table")]
+
+            def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache):
+                ops = self.runtime.ops
+                qkv = ops.dense(qkv, self.runtime.dtype).clone()
+                offsets = self.table.index_select(0, ctx.positions.long())
+                rotated = qkv[:, : (num_heads + num_kv_heads) * head_dim].view(qkv.shape[0], -1, head_dim)
+                rotated += offsets[:, None, :]
+                slots = ctx.slot_mapping[cache.group] if cache.writable else None
+                return ops.rope_store(qkv, cache.k, cache.v, None, None, ctx.positions, slots, num_heads, num_kv_heads,
+                                      head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype)
+
     if "ToyForCausalLM" not in arch_registry.ARCHITECTURES:
 
         def parse(data, name_or_path=""):
@@ -184,10 +248,16 @@ def register_toy_architecture():
                 "hidden_size": hidden, "num_heads": cfg["heads"], "num_kv_heads": cfg["kv_heads"], "head_dim": cfg["head_dim"],
                 "scale": cfg["head_dim"] ** -0.5, "qkv_bias": True, "out_bias": False, "window": None,
                 "position": PartSpec("rope", {"head_dim": cfg["head_dim"], "theta": 1e4, "scaling_factor": 1.0, "max_positions": 256})})
+            learned = PartSpec("gqa_attention", dict(attention.params, position=PartSpec(
+                "learned_positions", {"head_dim": cfg["head_dim"], "max_positions": 128})))
             toy = PartSpec("running_mean", {"hidden_size": hidden})
+            routed = PartSpec("top1_experts", {"hidden_size": hidden, "intermediate_size": cfg["intermediate_size"],
+                                               "num_experts": cfg["experts"]})
+            mixers = {"attention": attention, "attention_learned": learned, "state": toy}
             layers = []
-            for index, kind in enumerate(cfg["mixers"]):  # the mixer is chosen layer by layer
-                block = PartSpec("prenorm", {"mixer": attention if kind == "attention" else toy, "feed_forward": ff,
+            for index, kind in enumerate(cfg["mixers"]):  # mixer and feed-forward are chosen layer by layer
+                block = PartSpec("prenorm", {"mixer": mixers[kind],
+                                             "feed_forward": routed if cfg["feed_forwards"][index] == "routed" else ff,
                                              "mixer_norm": norm, "ff_norm": norm})
                 layers.append(LayerSpec(f"model.layers.{index}", block))
             schedule = tuple(LayerCall(layer, cache_of) for layer, cache_of in cfg["schedule"])
@@ -207,15 +277,20 @@ def toy_plain_logits(cfg, tensors, tokens):
     for call, (layer, cache_of) in enumerate(cfg["schedule"]):
         p = f"model.layers.{layer}"
         x = plain.rms_norm(h, tensors[f"{p}.input_layernorm.weight"], cfg["eps"])
-        if cfg["mixers"][layer] == "attention":
+        if cfg["mixers"][layer].startswith("attention"):
             heads, kvh, dim = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
-            angles = plain.rope_angles(pos, dim, 1e4)
+            if cfg["mixers"][layer] == "attention":
+                angles = plain.rope_angles(pos, dim, 1e4)
+                encode = lambda t: plain.apply_rope(t, angles)
+            else:
+                table = tensors[f"{p}.self_attn.position_table"]
+                encode = lambda t: t + table[pos][:, None, :]
             q = (x @ tensors[f"{p}.self_attn.q_proj.weight"].T + tensors[f"{p}.self_attn.q_proj.bias"]).view(-1, heads, dim)
-            q = plain.apply_rope(q, angles)
+            q = encode(q)
             if cache_of is None:
                 k = (x @ tensors[f"{p}.self_attn.k_proj.weight"].T + tensors[f"{p}.self_attn.k_proj.bias"]).view(-1, kvh, dim)
                 v = (x @ tensors[f"{p}.self_attn.v_proj.weight"].T + tensors[f"{p}.self_attn.v_proj.bias"]).view(-1, kvh, dim)
-                kv_of_call[call] = (plain.apply_rope(k, angles), v)
+                kv_of_call[call] = (encode(k), v)
             k, v = kv_of_call[call if cache_of is None else cache_of]
             mixed = plain.attention(q, k, v, plain.attention_mask(pos, len(tokens), None), dim ** -0.5)
             mixed = mixed.reshape(len(tokens), -1) @ tensors[f"{p}.self_attn.o_proj.weight"].T
@@ -224,17 +299,27 @@ def toy_plain_logits(cfg, tensors, tokens):
             mixed = mean @ tensors[f"{p}.self_attn.mix.weight"].T
         h = h + mixed
         x = plain.rms_norm(h, tensors[f"{p}.post_attention_layernorm.weight"], cfg["eps"])
-        h = h + plain.swiglu_mlp(x, *(tensors[f"{p}.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        if cfg["feed_forwards"][layer] == "routed":
+            choice = (x @ tensors[f"{p}.mlp.router.weight"].T).argmax(dim=-1)
+            h = h + torch.stack([
+                plain.swiglu_mlp(x[t:t + 1], *(tensors[f"{p}.mlp.experts.{int(choice[t])}.{n}_proj.weight"]
+                                               for n in ("gate", "up", "down")))[0]
+                for t in range(len(tokens))])
+        else:
+            h = h + plain.swiglu_mlp(x, *(tensors[f"{p}.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
     h = plain.rms_norm(h, tensors["model.norm.weight"], cfg["eps"])
     return h @ tensors["model.embed_tokens.weight"].T
 
 
 TOY_CONFIG = {
     "architectures": ["ToyForCausalLM"], "hidden_size": 40, "intermediate_size": 56, "vocab_size": 97, "heads": 5,
-    "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "mixers": ["attention", "state", "attention"],
-    # layer 0, the stateful layer, layer 0 AGAIN (weights reused, a cache of its own), then
-    # layer 2 reading the cache of the first call instead of keeping one.
-    "schedule": [[0, None], [1, None], [0, None], [2, 0]],
+    "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "experts": 3,
+    "mixers": ["attention", "state", "attention", "attention_learned"],
+    "feed_forwards": ["swiglu", "routed", "swiglu", "routed"],
+    # layer 0, the stateful layer (with a routed feed-forward), layer 0 AGAIN (weights reused, a
+    # cache of its own), layer 2 reading the cache of the first call instead of keeping one, then
+    # a layer whose attention takes learned positions instead of rotation.
+    "schedule": [[0, None], [1, None], [0, None], [2, 0], [3, None]],
 }
 
 
@@ -252,10 +337,12 @@ def test_toy_model_is_data(toy_folder):
 
     _, model = describe_model(TOY_CONFIG)
     layout = CacheLayout.from_model(model)
-    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads"]
-    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2) and layout.state_entries[0][0] == 1
+    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads", "pages"]
+    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2, 4) and layout.state_entries[0][0] == 1
     names = list(model.tensor_specs())
     assert "model.layers.1.self_attn.mix.weight" in names and "model.layers.2.self_attn.q_proj.weight" in names
+    assert "model.layers.1.mlp.experts.2.down_proj.weight" in names and "model.layers.1.mlp.router.weight" in names
+    assert "model.layers.3.self_attn.position_table" in names and "model.layers.0.mlp.gate_proj.weight" in names
 
 
 @pytest.mark.parametrize("cut", ["whole", "prefix_then_single", "portions", "mixed"])
@@ -273,6 +360,30 @@ def test_toy_architecture_steps_like_its_plain_form(toy_folder, cut):
     for rid, toks in requests.items():
         want = toy_plain_logits(raw, tensors, toks)
         assert float((got[rid] - want).abs().max()) <= 1e-4, f"{cut} {rid}"
+
+
+def test_a_part_can_keep_the_model_out_of_graphs(toy_folder):
+    """A part that reads device data back on the host says `capturable = False`; the runner
+    then records no HIP graph and steps the model eagerly, with the same logits."""
+    from test_gpu_replay import run_trace
+    from turboserve_amd.engine.replay import TraceReplayer
+    from turboserve_amd.parts import registry as part_registry
+
+    register_toy_architecture()
+    routed = part_registry.FEED_FORWARDS["top1_experts"]
+    raw, tensors = tiny.read_model_dir(toy_folder)
+    requests = {"a": tiny.random_tokens(97, 20, 1), "b": tiny.random_tokens(97, 33, 2)}
+    steps = th.prefix_then_single(requests)
+    assert TraceReplayer(toy_folder, dtype="float32", max_tokens=128, page_size=8).runner.graphs is not None
+    recorded = th.collect(steps, run_trace(toy_folder, "float32", 8, steps), requests)
+    routed.capturable = False
+    try:
+        assert TraceReplayer(toy_folder, dtype="float32", max_tokens=128, page_size=8).runner.graphs is None
+        eager = th.collect(steps, run_trace(toy_folder, "float32", 8, steps), requests)
+    finally:
+        routed.capturable = True
+    for rid in requests:
+        assert torch.equal(recorded[rid], eager[rid])
 
 
 # -- long decoding, first tokens ----------------------------------------------------------------------

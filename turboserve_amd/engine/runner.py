@@ -31,9 +31,10 @@ class ModelRunner:
         self.views = storage.views()
         self.vocab_size = model.plan.vocab_size
         self.num_steps = 0
-        #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``).
+        #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``), unless a part
+        #: of the model says it cannot be recorded (``Part.capturable``).
         self.graphs: DecodeGraphs | None = None
-        if use_graphs:
+        if use_graphs and model.is_capturable():
             self.graphs = DecodeGraphs(
                 model, self.views, page_size=storage.page_size, num_groups=len(self.layout.groups),
                 pad_state_slot=storage.pad_state_slot, max_batch=max_graph_batch,

@@ -120,6 +120,11 @@ class DecoderModel:
 
     # -- caches -------------------------------------------------------------------------------
 
+    def is_capturable(self) -> bool:
+        """Whether single-token steps of this model may be recorded into HIP graphs: every
+        part says so (``Part.capturable``)."""
+        return all(block.is_capturable() for block in self.blocks) and self.final_norm.is_capturable()
+
     def cache_needs(self) -> list[CacheNeed]:
         """What each schedule entry needs a cache for (``None``: nothing, or it reads another's)."""
         needs: list[CacheNeed] = []

@@ -58,6 +58,9 @@ class GroupedQueryAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
+    def is_capturable(self) -> bool:
+        return self.capturable and self.position.is_capturable()
+
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs = {
             self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden_size)),

@@ -135,6 +135,11 @@ class Part:
 
     #: A part without weights whose instances with equal parameters may be one object.
     shareable = False
+    #: Whether a step through this part may be recorded into a HIP graph: it reads nothing back
+    #: to the host (no ``.item()``, ``.tolist()``, ``nonzero()``) and what it launches depends only
+    #: on the step's shape, not on device data.  A part that cannot promise this says False and
+    #: the runner then runs every step of the model eagerly.
+    capturable = True
 
     def __init__(self, prefix: str, runtime: Runtime) -> None:
         self.prefix = prefix
@@ -142,6 +147,10 @@ class Part:
 
     def name(self, suffix: str) -> str:
         return f"{self.prefix}.{suffix}" if self.prefix else suffix
+
+    def is_capturable(self) -> bool:
+        """``capturable`` of this part and of the parts it is made of."""
+        return self.capturable
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         return {}
@@ -212,6 +221,9 @@ class Block(Part):
 
     def forward(self, stream: ResidualStream, ctx: "StepContext", cache: CacheView) -> ResidualStream:
         raise NotImplementedError
+
+    def is_capturable(self) -> bool:
+        return self.capturable and all(part.is_capturable() for part in self.parts())
 
     def parts(self) -> list[Part]:
         raise NotImplementedError

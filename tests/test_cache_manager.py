@@ -191,3 +191,40 @@ def test_sizing():
     assert both.num_blocks[1] == window_pages_needed(16, scheduler) == 14
     assert both.num_blocks[0] == (10**5 - 14 * 512) // 512
     assert torch.cuda.is_available() or True
+
+
+def test_page_table_mirror_follows_the_list():
+    """The int32 mirror of a block table equals the list after appends, after an overwritten
+    entry that was reported, and after growth beyond its first capacity."""
+    import numpy as np
+
+    from turboserve_amd.cache.page_table import PageTable, table_array
+
+    table = PageTable()
+    assert table_array(table).size == 0 and table == []
+    for page in range(40):
+        table.append(100 + page)
+        if page % 7 == 0:
+            assert table_array(table).tolist() == list(table)
+    table[3] = -1
+    table.entry_changed(3)
+    table.append(7)
+    mirror = table_array(table)
+    assert mirror.dtype == np.int32 and mirror.tolist() == list(table) and mirror[3] == -1
+    assert table_array([4, 5, 6]).tolist() == [4, 5, 6]
+
+
+def test_manager_tables_report_released_pages():
+    """Pages a window has passed turn into PAD_PAGE in the list and in its int32 mirror."""
+    from turboserve_amd.cache.manager import PAD_PAGE, CacheManager
+    from turboserve_amd.cache.page_table import table_array
+
+    manager = CacheManager([None, 8], [16, 16], 4, 2)
+    held = manager.admit("r")
+    for _ in range(10):
+        manager.append("r", 3)
+        for table in held.tables:
+            assert table_array(table).tolist() == list(table)
+    assert held.tables[1][0] == PAD_PAGE and PAD_PAGE not in held.tables[0]
+    manager.free("r")
+    manager.check_invariants()

@@ -14,6 +14,7 @@ from collections.abc import Hashable, Sequence
 from dataclasses import dataclass, field
 
 from turboserve_amd.cache.allocator import OutOfPagesError, PageAllocator
+from turboserve_amd.cache.page_table import PageTable
 from turboserve_amd.cache.state_slots import StateSlotPool
 
 #: Fill value of unused block-table entries (src/turboserve/engine/core/types.py:64-65).
@@ -103,7 +104,7 @@ class CacheManager:
         if request in self._requests:
             raise ValueError(f"request {request!r} already holds a cache")
         entry = RequestCache(
-            tables=[[] for _ in self.pools],
+            tables=[PageTable() for _ in self.pools],
             state_slot=self.state_slots.allocate(),
             released=[0] * len(self.pools),
         )
@@ -150,6 +151,7 @@ class CacheManager:
             for index in range(entry.released[g], upto):
                 pool.decref(table[index])
                 table[index] = PAD_PAGE
+                table.entry_changed(index)
             entry.released[g] = max(entry.released[g], upto)
             while len(table) * self.page_size < end:
                 table.append(pool.allocate())

@@ -17,6 +17,7 @@ import numpy as np
 import torch
 
 from turboserve_amd.cache.manager import PAD_PAGE
+from turboserve_amd.cache.page_table import table_array
 
 
 #: Rows of one request that the prefill attention kernel handles per wavefront.
@@ -153,8 +154,8 @@ def build_context(
         pieces.append(np.fromiter((s for e in entries for s in e.slots[g]), dtype=np.int32, count=num_tokens))
         table = np.full((num_seqs, widths[g]), PAD_PAGE, dtype=np.int32)
         for i, e in enumerate(entries):
-            row = e.tables[g]
-            table[i, : len(row)] = row
+            row = table_array(e.tables[g])
+            table[i, : row.size] = row
         pieces.append(table.reshape(-1))
     sizes = [p.size for p in pieces]
     packed = torch.from_numpy(np.concatenate(pieces)).to(device)

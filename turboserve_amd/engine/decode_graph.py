@@ -23,6 +23,7 @@ from collections.abc import Sequence
 import numpy as np
 import torch
 
+from turboserve_amd.cache.page_table import table_array
 from turboserve_amd.engine.batch import StepContext, StepEntry
 
 
@@ -180,8 +181,8 @@ class DecodeGraphs:
             table = field(f"table{g}").reshape(batch, width)
             table[:] = 0  # padding (and the unused tail of a row) points at page 0: never read past the context
             for i, e in enumerate(entries):
-                row = e.tables[g]
-                table[i, : len(row)] = row
+                row = table_array(e.tables[g])
+                table[i, : row.size] = row
         return host
 
     # -- the step --------------------------------------------------------------------------------

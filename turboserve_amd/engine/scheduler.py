@@ -40,7 +40,7 @@ class ScheduledSeq:
     start: int
     token_ids: list[int]
     slots: list[list[int]]
-    tables: list[list[int]]
+    tables: list[list[int]]  # the cache manager's own tables, not copies: read before the next scheduling call
     state_slot: int
     is_prefill: bool
     is_chunk: bool  # a portion that does not reach the end of the prompt: no logits, no token
@@ -279,7 +279,7 @@ class Scheduler:
         is_prefill = start < seq.num_prompt_tokens
         item = ScheduledSeq(
             seq=seq, num_new_tokens=num_new, start=start, token_ids=seq.tokens_in_range(start, end),
-            slots=slots, tables=[list(table) for table in held.tables], state_slot=held.state_slot,
+            slots=slots, tables=held.tables, state_slot=held.state_slot,
             is_prefill=is_prefill, is_chunk=end < seq.num_tokens,
         )
         seq.advance_computed(num_new)

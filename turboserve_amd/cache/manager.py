@@ -134,14 +134,16 @@ class CacheManager:
     def can_append(self, request: Hashable, num_new: int) -> bool:
         return not any(self.pages_short(request, num_new))
 
-    def append(self, request: Hashable, num_new: int) -> list[list[int]]:
+    def append(self, request: Hashable, num_new: int, *, checked: bool = False) -> list[list[int]]:
         """Take pages for the request's next ``num_new`` tokens; returns their slots per group.
 
-        Pages a window has passed are given back first.  All-or-nothing over the groups."""
+        Pages a window has passed are given back first.  All-or-nothing over the groups.
+        ``checked``: the caller has just seen :meth:`can_append` say yes for the same arguments
+        (the scheduler's case, once per request per step), so the check is not repeated."""
         if num_new < 0:
             raise ValueError(f"num_new must be non-negative, got {num_new}")
         entry = self.get(request)
-        if any(self.pages_short(request, num_new)):
+        if not checked and any(self.pages_short(request, num_new)):
             raise OutOfPagesError(f"request {request!r} cannot grow by {num_new} tokens: pages are short")
         start, end = entry.num_tokens, entry.num_tokens + num_new
         slots: list[list[int]] = []
@@ -156,7 +158,10 @@ class CacheManager:
             while len(table) * self.page_size < end:
                 table.append(pool.allocate())
             size = self.page_size
-            slots.append([table[pos // size] * size + pos % size for pos in range(start, end)])
+            if num_new == 1:  # a decoded token: no loop
+                slots.append([table[start // size] * size + start % size])
+            else:
+                slots.append([table[pos // size] * size + pos % size for pos in range(start, end)])
         entry.num_tokens = end
         return slots
 

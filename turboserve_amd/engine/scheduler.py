@@ -231,7 +231,7 @@ class Scheduler:
                 continue
             if not self._make_room(seq, num_new, scheduled_ids, out, preempted_now):
                 continue
-            self._emit(seq, num_new, budget, scheduled_ids, prefills, decodes, out)
+            self._emit(seq, num_new, budget, scheduled_ids, prefills, decodes, out, checked=True)
 
         while budget[0] > 0 and budget[1] > 0:
             from_preempted = bool(self._preempted)
@@ -269,13 +269,13 @@ class Scheduler:
         self._num_decode_tokens += out.num_decode_tokens
         return out
 
-    def _emit(self, seq, num_new, budget, scheduled_ids, prefills, decodes, out) -> None:
+    def _emit(self, seq, num_new, budget, scheduled_ids, prefills, decodes, out, *, checked: bool = False) -> None:
         """Take the slots of ``num_new`` tokens, record the request in the step and advance its
-        computed count at once (scheduler.py:713-744)."""
+        computed count at once (scheduler.py:713-744).  ``checked``: room was just made."""
         start = seq.num_computed_tokens
         end = start + num_new
         held = self.cache.get(seq.seq_id)
-        slots = self.cache.append(seq.seq_id, num_new)
+        slots = self.cache.append(seq.seq_id, num_new, checked=checked)
         is_prefill = start < seq.num_prompt_tokens
         item = ScheduledSeq(
             seq=seq, num_new_tokens=num_new, start=start, token_ids=seq.tokens_in_range(start, end),

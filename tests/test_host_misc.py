@@ -150,3 +150,31 @@ def test_the_run_order_is_data():
         ModelPlan(10, 8, layers, (LayerCall(2),), norm, True)
     with pytest.raises(ValueError, match="owns none"):
         ModelPlan(10, 8, layers, (LayerCall(0), LayerCall(1, cache_of=0), LayerCall(0, cache_of=1)), norm, True)
+
+
+def test_bench_contract_on_the_host():
+    """What of bench.py can be checked without a GPU: more than one GPU is refused with one
+    line and exit code 2; the byte and flop counts behind `roofline` and `prefill.frac` are the
+    7B shape's by hand; the other shapes differ only where BASELINE's configurations do."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    sys.path.insert(0, str(root))
+    import bench
+    from turboserve_amd.config.registry import parse_model_config
+
+    refused = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert refused.returncode == 2 and len(refused.stdout.strip().splitlines()) == 1
+    config = parse_model_config(dict(bench.SHAPE_7B))
+    h, i, v, layers = 3584, 18944, 152064, 28
+    per_layer = h * 4608 + 4608 + h * h + 3 * h * i + 2 * h  # qkv + bias, o, gate/up/down, two norms
+    weights = layers * per_layer + h + v * h
+    assert bench.decode_bytes(config, layers, 0, 0, 2) == 2 * weights
+    cache_8 = 8 * 8192 * 2 * layers * 512 * 2  # batch 8, context 8192, K and V, 4 KV heads x 128, bf16
+    assert bench.decode_bytes(config, layers, 8, 8192, 2) == 2 * (weights + 8 * h) + cache_8
+    linear = layers * (h * 4608 + h * h + 3 * h * i)
+    assert bench.prefill_flops(config, layers, 2048) == 2.0 * 2048 * linear + layers * 4 * h * 2048 * 2048 / 2 + 2.0 * v * h
+    assert bench.SHAPES["14b"][1]["num_hidden_layers"] == 48 and bench.SHAPES["32b"][1]["intermediate_size"] == 27648
+    assert bench.PEAK_FLOPS["bf16"] == 2.5e15 and bench.PEAK_FLOPS["fp32"] == 157.3e12 and bench.HBM_PEAK_GBS == 8000.0

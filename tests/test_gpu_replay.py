@@ -14,6 +14,7 @@ import torch
 
 import tiny
 import trace_helpers as th
+from plain import qwen2_plain as plain
 
 pytestmark = pytest.mark.gpu
 
@@ -138,3 +139,40 @@ def test_trace_run_program(case, dtype, tmp_path):
         else:
             assert not path.exists()
     check(th.collect(steps, outputs, case["requests"]), case["expected"][dtype], dtype, "trace_run mixed")
+
+
+@pytest.mark.parametrize("trial", range(10))
+def test_random_configurations_replay_like_plain(trial, tmp_path):
+    """Seeded random configurations beyond the three fixed ones: head sizes that are and are not
+    multiples of 16 or 32, one to sixteen query heads per KV head (every attention kernel variant),
+    page sizes 8 to 64, windows, tied and untied heads; mixed and portion-wise cutting, both dtypes."""
+    import random
+
+    rng = random.Random(9000 + trial)
+    kv_heads = rng.choice([1, 1, 2, 3, 4])
+    group = rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 16])
+    heads = kv_heads * group if kv_heads * group <= 32 else kv_heads * (32 // kv_heads)
+    window = rng.choice([None, None, 12, 33, 70])
+    config = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": rng.choice([64, 72, 96, 136, 200]),
+        "num_hidden_layers": rng.choice([1, 2, 3]), "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+        "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 128, 256, 24, 40]),
+        "intermediate_size": rng.choice([64, 104, 200, 264]), "vocab_size": rng.choice([97, 256, 1000, 5003]),
+        "rope_theta": rng.choice([1e4, 1e6]), "rms_norm_eps": rng.choice([1e-6, 1e-5]),
+        "tie_word_embeddings": rng.random() < 0.5, "use_sliding_window": window is not None,
+        "max_position_embeddings": 512,
+    }
+    if window is not None:
+        config["sliding_window"] = window
+        config["max_window_layers"] = rng.choice([0, 1])
+    page = rng.choice([8, 16, 32, 64])
+    lengths = [rng.choice([3, 17, 40, 75, 130, 200]) for _ in range(rng.choice([2, 3, 5]))]
+    folder = tiny.make_model_dir(tmp_path, config, trial, torch.float32)
+    raw, tensors = tiny.read_model_dir(folder)
+    requests = {f"r{i}": tiny.random_tokens(config["vocab_size"], n, 500 + i) for i, n in enumerate(lengths)}
+    expected = {rid: plain.forward_logits(raw, plain.as_float32(tensors), toks) for rid, toks in requests.items()}
+    for cut in ("mixed", "portions"):
+        steps = CUTS[cut](requests)
+        for dtype in ("float32", "bfloat16"):
+            got = th.collect(steps, run_trace(folder, dtype, page, steps), requests)
+            check(got, expected, dtype, f"trial {trial} {config} page {page} {cut}")

@@ -176,3 +176,68 @@ def test_random_configurations_replay_like_plain(trial, tmp_path):
         for dtype in ("float32", "bfloat16"):
             got = th.collect(steps, run_trace(folder, dtype, page, steps), requests)
             check(got, expected, dtype, f"trial {trial} {config} page {page} {cut}")
+
+
+def test_7b_layer_sizes_float32_and_bfloat16_paths_agree():
+    """Two layers of the Qwen2.5-7B sizes (hidden 3584, 28 heads on 4 KV heads of 128, 18944
+    wide, 152064 tokens) holding the same bfloat16-rounded random weights, stepped by the
+    32-bit path (its own product and attention kernels) and by the bfloat16 path (skinny and
+    library products, matrix-core attention): a 300- and a 77-token prompt in one step, then
+    four decode steps of both.  The logits agree to bfloat16 accuracy and pick the same token."""
+    from turboserve_amd.cache.manager import CacheManager
+    from turboserve_amd.engine.batch import StepEntry
+    from turboserve_amd.engine.loading import build_model, build_storage, make_runtime
+    from turboserve_amd.engine.runner import ModelRunner
+
+    shape = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 3584, "num_hidden_layers": 2,
+        "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128, "intermediate_size": 18944,
+        "vocab_size": 152064, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+        "max_position_embeddings": 32768,
+    }
+    generator = torch.Generator().manual_seed(5)
+    requests = {name: torch.randint(0, shape["vocab_size"], (n,), generator=generator).tolist()
+                for name, n in (("a", 300), ("b", 77))}
+    logits = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        runtime = make_runtime(dtype, "cuda:0")
+        _, model = build_model(shape, runtime)
+        draw = torch.Generator(device="cuda:0")
+        draw.manual_seed(3)
+        tensors = {}
+        for name, spec in model.tensor_specs().items():
+            if spec.init == "ones":
+                values = torch.ones(spec.shape, device="cuda:0")
+            else:
+                values = torch.empty(spec.shape, device="cuda:0").normal_(0.0, 0.02, generator=draw)
+            tensors[name] = values.bfloat16().to(dtype)  # the same numbers in both runs
+        model.load(tensors)
+        del tensors
+        storage = build_storage(model, 64, 16, 4)
+        manager = CacheManager(storage.layout.windows(), 64, 16, 4)
+        runner = ModelRunner(model, storage)
+        rows = []
+        entries = []
+        for name, tokens in requests.items():
+            held = manager.admit(name)
+            slots = manager.append(name, len(tokens) - 4)
+            entries.append(StepEntry(request=name, tokens=tokens[:-4], start=0, tables=held.tables, slots=slots,
+                                     state_slot=held.state_slot, want=[len(tokens) - 5]))
+        rows.append(runner.step(entries).float().cpu())
+        for k in range(4):
+            entries = []
+            for name, tokens in requests.items():
+                held = manager.get(name)
+                start = held.num_tokens
+                slots = manager.append(name, 1)
+                entries.append(StepEntry(request=name, tokens=[tokens[len(tokens) - 4 + k]], start=start,
+                                         tables=held.tables, slots=slots, state_slot=held.state_slot, want=[0]))
+            rows.append(runner.step(entries).float().cpu())
+        logits[dtype] = torch.cat(rows)
+        runner.release()
+        del model, storage, runner
+        torch.cuda.empty_cache()
+    exact, fast = logits[torch.float32], logits[torch.bfloat16]
+    assert exact.shape == (10, shape["vocab_size"])
+    assert float((exact - fast).abs().max()) <= RTOL_BF16 * float(exact.abs().max())
+    assert torch.equal(exact.argmax(-1), fast.argmax(-1))

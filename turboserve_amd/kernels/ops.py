@@ -146,6 +146,11 @@ class Ops:
         self.core = load_module("core")
         for module in modules:
             load_module(module)
+        #: (row bucket, N, K, biased, 32-bit result) -> True where the BLAS library, not the skinny
+        #: product, runs a bfloat16 projection of 17 to 64 rows (filled by a timed choice at start-up).
+        self.library_products: dict[tuple[int, int, int, bool, bool], bool] = {}
+        #: While a list: every such projection that runs is noted here as (key, weight, bias).
+        self.product_log: list | None = None
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -570,6 +575,19 @@ class Ops:
                "ts_gemm_skinny")
         return partial
 
+    def _skinny_runs(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, float32_out: bool) -> bool:
+        """Whether the skinny product, not the library, runs this bfloat16 projection: always up
+        to 16 rows, never above 64, in between unless a timed choice gave the shape to the library."""
+        m = x.shape[0]
+        if not self.skinny_supported(x, weight) or m > self.skinny_max_rows:
+            return False
+        if m <= self.skinny_resident_rows:
+            return True
+        key = (1 << (m - 1).bit_length(), weight.shape[0], weight.shape[1], bias is not None, float32_out)
+        if self.product_log is not None:
+            self.product_log.append((key, weight, bias))
+        return not self.library_products.get(key, False)
+
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
         """The projection of the serving path.  32-bit runs use :meth:`gemm_plain` (no reduced
         matrix mode).  bfloat16 runs with decode-sized batches use :meth:`gemm_skinny` and
@@ -579,7 +597,7 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight, bias)
         _gpu(x, weight, bias)
-        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
+        if self._skinny_runs(x, weight, bias, False):
             return self.gemm_skinny(x, weight, bias)
         if bias is None:
             return torch.mm(x, weight.t())
@@ -591,7 +609,7 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight)
         _gpu(x, weight)
-        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
+        if self._skinny_runs(x, weight, None, True):
             return self.gemm_skinny(x, weight, max_splits=1)[0]
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
 

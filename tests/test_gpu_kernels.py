@@ -269,6 +269,48 @@ def test_rope_store(ops, dtype, heads, kv_heads, dim, page, theta, factor):
         ops.rope_store(dev, kp, vp, cos.to(DEV), sin.to(DEV), positions.to(DEV), None, heads, kv_heads, dim, page, 128)
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(7, 1, 128, 16), (3, 3, 48, 8), (4, 2, 32, 4), (2, 1, 96, 32)])
+def test_rope_store_of_many_tokens_equals_token_by_token(ops, heads, kv_heads, dim, page):
+    """Prompt portions of 32 tokens or more go through a kernel that handles 8 tokens per block
+    with 16-byte accesses (values of 8 consecutive slots leave as one store into the transposed
+    page).  It must write, bit for bit, what the per-token kernel writes when the same tokens
+    come in pieces of fewer than 32: slots in runs that start on and off a multiple of 8, runs
+    that cross pages, scattered slots, a token without a slot, a ragged last group."""
+    from turboserve_amd.parts.rope import rotary_tables
+
+    g = torch.Generator().manual_seed(dim + page)
+    tokens, num_pages = 75, 256 // page + 1
+    width = (heads + 2 * kv_heads) * dim
+    qkv = torch.randn(tokens, width, generator=g).to(torch.bfloat16)
+    positions = torch.cat([torch.arange(5, 45), torch.arange(0, 35)]).to(torch.int32)
+    slots = list(range(16, 56))            # a run from a multiple of 8, over page edges
+    slots += list(range(83, 83 + 19))      # a run that starts off a multiple of 8
+    scattered = [3, 150, 7, 201, 130, 9, 64, 249, 11, 70, 2, 255, 128, 140, 0, 77]
+    slots += scattered[: tokens - len(slots)]
+    slots[50] = -1
+    assert len(slots) == tokens and max(slots) < num_pages * page
+    live = [s for s in slots if s >= 0]
+    assert len(set(live)) == len(live)
+    cos, sin = rotary_tables(64, dim, 10000.0, 1.0)
+    cos, sin = cos.to(DEV), sin.to(DEV)
+    results = []
+    for piece in (tokens, 16):
+        kp = torch.zeros(num_pages, kv_heads, page, dim, dtype=torch.bfloat16, device=DEV)
+        vp = torch.zeros(num_pages, kv_heads, dim, page, dtype=torch.bfloat16, device=DEV)
+        dev = qkv.to(DEV)
+        for start in range(0, tokens, piece):
+            stop = min(tokens, start + piece)
+            ops.rope_store(dev[start:stop], kp, vp, cos, sin, positions[start:stop].to(DEV),
+                           torch.tensor(slots[start:stop], dtype=torch.int32, device=DEV), heads, kv_heads, dim, page, 63)
+        results.append((dev.cpu(), kp.cpu(), vp.cpu()))
+    for whole, pieces in zip(*results):
+        assert torch.equal(whole.view(torch.int16), pieces.view(torch.int16))
+    # and against the plain rotation, so that both are not wrong together
+    q = qkv.float()[:, : heads * dim].view(tokens, heads, dim)
+    want = plain.apply_rope(q, plain.rope_angles(positions, dim, 10000.0, 1.0))
+    torch.testing.assert_close(results[0][0].float()[:, : heads * dim].view(tokens, heads, dim), want, **tol(torch.bfloat16))
+
+
 # -- attention --------------------------------------------------------------------------------------
 
 

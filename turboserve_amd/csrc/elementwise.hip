@@ -310,6 +310,12 @@ extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits,
 // 16-byte load.  rotate == 0 skips the rotation (a position encoding that only stores).
 // slots == nullptr or a negative slot: nothing is stored for that token.
 // ---------------------------------------------------------------------------------------------
+// One rotation, written out so that every kernel rounds it the same way.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float& o1, float& o2) {
+  o1 = __builtin_fmaf(x1, c, -(x2 * s));
+  o2 = __builtin_fmaf(x2, c, x1 * s);
+}
+
 template <typename T, typename P>
 __global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int splits,
                                   size_t split_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
@@ -345,8 +351,10 @@ __global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int sp
         x1 += to_float(row[sp * split_stride + i]);
         x2 += to_float(row[sp * split_stride + i + half]);
       }
-      const T o1 = from_float<T>(rotate ? x1 * c[i] - x2 * s[i] : x1);
-      const T o2 = from_float<T>(rotate ? x2 * c[i] + x1 * s[i] : x2);
+      float r1 = x1, r2 = x2;
+      if (rotate) rotate_pair(x1, x2, c[i], s[i], r1, r2);
+      const T o1 = from_float<T>(r1);
+      const T o2 = from_float<T>(r2);
       if (qrow) {
         qrow[i] = o1;
         qrow[i + half] = o2;
@@ -365,6 +373,93 @@ __global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int sp
   }
 }
 
+// The same for many tokens at once (prompt portions): bfloat16 in and out, no partial sums, head
+// size a multiple of 16.  One block per (group of 8 consecutive tokens, head).  q and k heads: a
+// thread rotates 8 pairs with 16-byte loads and stores.  v heads: a thread collects one head
+// dimension of the 8 tokens; when the group's slots are 8 consecutive ones starting at a multiple
+// of 8 (the usual case inside a prompt: they lie in one page, block_size being a multiple of 8)
+// that is one 16-byte store into the transposed value page, else one 2-byte store per token.
+constexpr int ROPE_GROUP = 8;
+
+__global__ void __launch_bounds__(64)
+rope_store_group_kernel(bf16_t* q_out, long q_stride, const bf16_t* proj, bf16_t* __restrict__ k_pages,
+                        bf16_t* __restrict__ v_pages, const float* __restrict__ cos_table,
+                        const float* __restrict__ sin_table, const int* __restrict__ positions,
+                        const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim,
+                        int block_size, int rotate) {
+  typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  const int t0 = blockIdx.x * ROPE_GROUP;
+  const int h = blockIdx.y;
+  const int half = dim / 2;
+  const int width = (heads + 2 * kv_heads) * dim;
+  const int count = min(ROPE_GROUP, tokens - t0);
+  if (h < heads + kv_heads) {
+    const bool is_key = h >= heads;
+    const int kvh = h - heads;
+    const int vectors = half / 8;  // 16-byte pieces of a half row
+    for (int item = threadIdx.x; item < ROPE_GROUP * vectors; item += blockDim.x) {
+      const int j = item / vectors, i = (item % vectors) * 8;
+      if (j >= count) continue;
+      const int t = t0 + j;
+      const bf16_t* row = proj + (size_t)t * width + (size_t)h * dim;
+      const u16x8 a = *reinterpret_cast<const u16x8*>(row + i);
+      const u16x8 b = *reinterpret_cast<const u16x8*>(row + i + half);
+      u16x8 o1 = a, o2 = b;
+      if (rotate) {
+        const float* c = cos_table + (size_t)positions[t] * half + i;
+        const float* s = sin_table + (size_t)positions[t] * half + i;
+        const f32x4v c0 = *reinterpret_cast<const f32x4v*>(c), c1 = *reinterpret_cast<const f32x4v*>(c + 4);
+        const f32x4v s0 = *reinterpret_cast<const f32x4v*>(s), s1 = *reinterpret_cast<const f32x4v*>(s + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float cv = e < 4 ? c0[e & 3] : c1[e & 3], sv = e < 4 ? s0[e & 3] : s1[e & 3];
+          float r1, r2;
+          rotate_pair(to_float(bf16_t{a[e]}), to_float(bf16_t{b[e]}), cv, sv, r1, r2);
+          o1[e] = from_float<bf16_t>(r1).bits;
+          o2[e] = from_float<bf16_t>(r2).bits;
+        }
+      }
+      if (!is_key) {
+        bf16_t* qrow = q_out + (size_t)t * q_stride + (size_t)h * dim;
+        *reinterpret_cast<u16x8*>(qrow + i) = o1;
+        *reinterpret_cast<u16x8*>(qrow + i + half) = o2;
+      } else {
+        const int slot = slots ? slots[t] : -1;
+        if (slot < 0) continue;
+        bf16_t* page = k_pages + (((size_t)(slot / block_size) * kv_heads + kvh) * block_size + slot % block_size) * dim;
+        *reinterpret_cast<u16x8*>(page + i) = o1;
+        *reinterpret_cast<u16x8*>(page + i + half) = o2;
+      }
+    }
+    return;
+  }
+  if (!slots) return;
+  const int kvh = h - heads - kv_heads;
+  int slot[ROPE_GROUP];
+#pragma unroll
+  for (int j = 0; j < ROPE_GROUP; ++j) slot[j] = j < count ? slots[t0 + j] : -1;
+  bool run = count == ROPE_GROUP && slot[0] >= 0 && (slot[0] & 7) == 0 && (block_size & 7) == 0;
+#pragma unroll
+  for (int j = 1; j < ROPE_GROUP; ++j) run = run && slot[j] == slot[0] + j;
+  const bf16_t* column = proj + (size_t)t0 * width + (size_t)h * dim;
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    u16x8 v;
+#pragma unroll
+    for (int j = 0; j < ROPE_GROUP; ++j) v[j] = j < count ? column[(size_t)j * width + d].bits : (uint16_t)0;
+    if (run) {
+      bf16_t* dst = v_pages + (((size_t)(slot[0] / block_size) * kv_heads + kvh) * dim + d) * block_size + slot[0] % block_size;
+      *reinterpret_cast<u16x8*>(dst) = v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < ROPE_GROUP; ++j) {
+        if (slot[j] < 0) continue;
+        v_pages[(((size_t)(slot[j] / block_size) * kv_heads + kvh) * dim + d) * block_size + slot[j] % block_size] = bf16_t{v[j]};
+      }
+    }
+  }
+}
+
 extern "C" int ts_rope_store(void* q_out, long q_stride, const void* proj, int in_f32, int splits,
                              long split_stride, void* k_pages, void* v_pages, const float* cos_table,
                              const float* sin_table, const int* positions, const int* slots, int tokens,
@@ -377,6 +472,13 @@ extern "C" int ts_rope_store(void* q_out, long q_stride, const void* proj, int i
   if (rotate && (!cos_table || !sin_table)) return TS_ERR_ARG;
   if (slots && (!k_pages || !v_pages)) return TS_ERR_ARG;
   dim3 grid(tokens, heads + 2 * kv_heads), block(64);
+  const bool aligned = ((uintptr_t)q_out | (uintptr_t)proj | (uintptr_t)k_pages | (uintptr_t)v_pages |
+                        (uintptr_t)cos_table | (uintptr_t)sin_table) % 16 == 0 && q_stride % 8 == 0;
+  if (dtype == TS_BF16 && !in_f32 && splits == 1 && dim % 16 == 0 && tokens >= 4 * ROPE_GROUP && aligned) {
+    dim3 groups((tokens + ROPE_GROUP - 1) / ROPE_GROUP, heads + 2 * kv_heads);
+    hipLaunchKernelGGL(rope_store_group_kernel, groups, block, 0, stream, (bf16_t*)q_out, q_stride, (const bf16_t*)proj, (bf16_t*)k_pages, (bf16_t*)v_pages, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, block_size, rotate);
+    return ts_launch_status();
+  }
   if (dtype == TS_F32)
     hipLaunchKernelGGL((rope_store_kernel<float, float>), grid, block, 0, stream, (float*)q_out, q_stride, (const float*)proj, splits, (size_t)split_stride, (float*)k_pages, (float*)v_pages, cos_table, sin_table, positions, slots, heads, kv_heads, dim, block_size, rotate);
   else if (dtype == TS_BF16 && in_f32)

@@ -422,6 +422,32 @@ def test_attention_decode_mfma_far_key_and_subrange(ops):
     assert float(case.expected[1].abs().mean()) > 4.0  # the spike's value dominates
 
 
+def test_attention_decode_mfma_at_tens_of_thousands_of_keys(ops):
+    """One request with 40,000 keys (the most splits a launch makes) next to a short one; a far
+    key carries the long one's result."""
+    heads, kv_heads, dim, page = 14, 2, 128, 16
+    contexts = [40000, 700]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, [(c, 1) for c in contexts], None, seed=9, spike=23456)
+    out = torch.zeros(len(contexts), heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints(contexts), 0, len(contexts), heads, dim ** -0.5, None, max(contexts),
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+    assert float(case.expected[0].abs().mean()) > 4.0
+    # the same cache, its last 40 positions as a prompt portion
+    seqs = [(40000, 40)]
+    portion = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, None, seed=9, spike=23456)
+    blocks = [(0, off) for off in range(0, 40, 16)]
+    out = torch.zeros(40, heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, portion.dev(portion.q), heads * dim, portion.dev(portion.kp), portion.dev(portion.vp),
+        portion.dev(portion.table), portion.ints(portion.qsl), portion.ints([40000]), portion.ints(blocks), heads,
+        dim ** -0.5, None, 40000,
+    )
+    torch.testing.assert_close(out.float().cpu(), portion.expected, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_GEOMETRIES)
 @pytest.mark.parametrize("window", [None, 20, 300])
 def test_attention_prefill_mfma(ops, heads, kv_heads, dim, page, window):

@@ -5,7 +5,7 @@
 
 A "step" is one decode step of the whole engine path: the step function over a batch of
 single tokens against the paged cache, logits, greedy sampling, tokens back on the host.
-The default run has the 7B shape of BASELINE.json's configs[2], random weights
+The default run has the Qwen2.5-7B layer sizes (the benchmark's named configuration), random weights
 (N(0, 0.02), norm gains 1), a batch of 8 requests each holding a context of 8,192 tokens
 (cache filled with random keys and values; what is timed is real decode steps on top of it).
 One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times one
@@ -31,7 +31,7 @@ import time
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
-#: BASELINE.json configs[2]: Qwen2.5-7B shape.
+#: The benchmark's named configuration: Qwen2.5-7B layer sizes.
 SHAPE_7B = {
     "architectures": ["Qwen2ForCausalLM"],
     "model_type": "qwen2",
@@ -48,7 +48,7 @@ SHAPE_7B = {
     "use_sliding_window": False,
     "max_position_embeddings": 32768,
 }
-#: BASELINE.json configs[3] and configs[4]: the other layer shapes a run can be asked for.
+#: The 14B and 32B layer sizes of the same family: the other shapes a run can be asked for.
 SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
                  intermediate_size=13824, rms_norm_eps=1e-5)
 SHAPE_32B = dict(SHAPE_14B, num_hidden_layers=64, intermediate_size=27648)

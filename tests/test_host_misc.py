@@ -155,7 +155,7 @@ def test_the_run_order_is_data():
 def test_bench_contract_on_the_host():
     """What of bench.py can be checked without a GPU: more than one GPU is refused with one
     line and exit code 2; the byte and flop counts behind `roofline` and `prefill.frac` are the
-    7B shape's by hand; the other shapes differ only where BASELINE's configurations do."""
+    7B shape's by hand; the other shapes differ only where the 14B and 32B layer sizes do."""
     import subprocess
     import sys
     from pathlib import Path

@@ -86,12 +86,19 @@ __device__ __forceinline__ void swap_rows(float v, bool halves, float& a, float&
   a = __builtin_bit_cast(float, first);
   b = __builtin_bit_cast(float, second);
 }
+// The larger of two numbers that are known not to be NaN, as the one instruction (fmaxf would
+// first rewrite each operand that comes out of a swap, in case it were a signalling NaN).
+__device__ __forceinline__ float max_of_numbers(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 __device__ __forceinline__ float groups_max(float v) {
   float a, b;
   swap_rows(v, false, a, b);
-  v = fmaxf(a, b);
+  v = max_of_numbers(a, b);
   swap_rows(v, true, a, b);
-  return fmaxf(a, b);
+  return max_of_numbers(a, b);
 }
 __device__ __forceinline__ float groups_sum(float v) {
   float a, b;
@@ -758,13 +765,18 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
         {
           KeyFrags kf;
           read_keys(kf, ks + buf * K_TILE, lane16, group);
-          const bool inside = interior(w);
+          // One branch for all heads of the wavefront: the masks' comparisons are formed only
+          // where a window needs them, and neither path copies its scores to meet the other.
+          if (interior(w)) {
 #pragma unroll
-          for (int c = 0; c < CT; ++c) {
-            const f32x4 s0 = score_tile(kf, 0, qf[c]);
-            const f32x4 s1 = score_tile(kf, 1, qf[c]);
-            prob[c] = inside ? softmax_window<false>(st[c], s0, s1, w, group, lo_col, p_col, scale_log2, alpha[c])
-                             : softmax_window<true>(st[c], s0, s1, w, group, lo_col, p_col, scale_log2, alpha[c]);
+            for (int c = 0; c < CT; ++c)
+              prob[c] = softmax_window<false>(st[c], score_tile(kf, 0, qf[c]), score_tile(kf, 1, qf[c]), w, group,
+                                              lo_col, p_col, scale_log2, alpha[c]);
+          } else {
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+              prob[c] = softmax_window<true>(st[c], score_tile(kf, 0, qf[c]), score_tile(kf, 1, qf[c]), w, group,
+                                             lo_col, p_col, scale_log2, alpha[c]);
           }
         }
         ValueFrags vf;

@@ -62,7 +62,8 @@ def parse_args() -> argparse.Namespace:
     p = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=64)
-    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--warmup", type=int, default=40,
+                   help="untimed steps first; the clocks take some tens of milliseconds of load to settle")
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=CONTEXT)
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")

@@ -32,10 +32,13 @@
 #endif
 static_assert(TS_HEAD_DIM % 16 == 0 && TS_HEAD_DIM >= 16 && TS_HEAD_DIM <= 256, "head size: 16..256 in steps of 16");
 
-// Query heads of one KV head that share each loaded window in the prefill kernel.
+// Query heads of one KV head that share each loaded window in the prefill kernel, and
+// wavefronts per SIMD the register budgets are set for: the largest head sizes need the whole
+// register file of a SIMD for one wavefront (accumulators alone are D / 4 registers a head).
 #ifndef TS_PREFILL_HEADS
-#define TS_PREFILL_HEADS 2
+#define TS_PREFILL_HEADS (TS_HEAD_DIM > 128 ? 1 : 2)
 #endif
+#define TS_WAVES_PER_SIMD (TS_HEAD_DIM > 128 ? 1 : 2)
 
 #define TS_CAT2(a, b) a##b
 #define TS_CAT(a, b) TS_CAT2(a, b)
@@ -340,7 +343,7 @@ __device__ __forceinline__ float column_sum(float l) { return groups_sum(l); }
 // decode: grid (splits, kv_heads * head_tiles, requests); one wavefront each.
 // partial_acc [requests, heads, splits, D] float; partial_ml [requests, heads, splits, 2] float.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(TS_WAVES_PER_SIMD, TS_WAVES_PER_SIMD)))
 decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
               const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
               const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
@@ -679,7 +682,7 @@ __device__ __forceinline__ void read_values(ValueFrags& f, const uint16_t* vs, i
 }
 
 template <int CT>
-__global__ void __launch_bounds__(STAGE_WAVES * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(STAGE_WAVES * TS_WAVE) __attribute__((amdgpu_waves_per_eu(TS_WAVES_PER_SIMD, TS_WAVES_PER_SIMD)))
 prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
                       const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                       const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,

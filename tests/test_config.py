@@ -127,6 +127,9 @@ def test_kv_bytes_and_round_trip(tmp_path):
         assert Qwen2Config.from_dict(parsed.to_hf_dict()) == parsed, name
     (tmp_path / "config.json").write_text(json.dumps(QWEN2_RAW))
     assert read_config_json(tmp_path)["vocab_size"] == 512
+    from_folder = Qwen2Config.from_hf(tmp_path)
+    assert from_folder.name_or_path == str(tmp_path)
+    assert from_folder.to_hf_dict() == Qwen2Config.from_dict(QWEN2_RAW).to_hf_dict()
     with pytest.raises(UnsupportedModelError, match="no config.json"):
         read_config_json(tmp_path / "nowhere")
     (tmp_path / "config.json").write_text("[1, 2]")
@@ -153,6 +156,15 @@ def test_engine_and_sampling_options():
         SchedulerConfig(block_size=12)
     with pytest.raises(ValueError, match="at least one block"):
         SchedulerConfig(block_size=16, max_num_batched_tokens=8)
+    # What the reference has and this engine does not is accepted switched off, refused switched on.
+    assert SchedulerConfig(enable_prefix_caching=False, policy="fcfs").enable_prefix_caching is False
+    with pytest.raises(ValueError, match="no prefix cache"):
+        SchedulerConfig(enable_prefix_caching=True)
+    with pytest.raises(ValueError, match="fcfs"):
+        SchedulerConfig(policy="priority")
+    from turboserve_amd.engine.outputs import RequestOutput
+
+    assert RequestOutput(request_id="r").cached_prompt_tokens == 0
     config = EngineConfig(model="m")
     assert config.resolved_dtype() == "bfloat16" and config.resolved_device() == "cuda:0"
     assert config.gpu_memory_utilization == 0.9 and config.block_size == 16 and config.num_blocks is None

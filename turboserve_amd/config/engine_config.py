@@ -1,7 +1,9 @@
 """Options of the scheduler and of the engine (src/turboserve/engine/core/types.py:484-593).
 
-Names and defaults are the reference's where it has them; what it has and this engine does
-not (prefix caching, tenant policy, speculative and LoRA blocks) is absent.
+Names and defaults are the reference's where it has them.  What it has and this engine does
+not is either absent (speculative and LoRA blocks) or, where a caller of the reference is likely
+to pass it, accepted in its "off" value only: ``enable_prefix_caching`` (the reference's default
+is on; here it must be off) and ``policy`` (first come, first served).
 """
 
 from __future__ import annotations
@@ -18,8 +20,14 @@ class SchedulerConfig:
     block_size: int = 16
     num_blocks: int | None = None
     enable_chunked_prefill: bool = True
+    enable_prefix_caching: bool = False  # not built: every prompt is computed in full
+    policy: str = "fcfs"  # the only order of admission
 
     def __post_init__(self) -> None:
+        if self.enable_prefix_caching:
+            raise ValueError("enable_prefix_caching=True: this engine has no prefix cache; pass False")
+        if self.policy != "fcfs":
+            raise ValueError(f"policy {self.policy!r} is not built; the only policy is 'fcfs'")
         for name in ("max_num_seqs", "max_num_batched_tokens", "block_size"):
             value = getattr(self, name)
             if isinstance(value, bool) or not isinstance(value, int) or value < 1:

@@ -295,6 +295,11 @@ class Qwen2Config:
             name_or_path=name_or_path,
         )
 
+    @classmethod
+    def from_hf(cls, model_dir: str | Path) -> "Qwen2Config":
+        """The configuration of a model folder (model_config.py:316-339); local folders only."""
+        return cls.from_dict(read_config_json(model_dir), name_or_path=str(model_dir))
+
 
 def read_config_json(model_dir: str | Path) -> dict[str, Any]:
     """The parsed ``config.json`` of a model folder (model_config.py:334-339)."""

@@ -40,7 +40,11 @@ class LLMEngine:
         scheduler: Scheduler | None = None,
         runner: Any | None = None,
         sampler: Any | None = None,
+        local_files_only: bool = True,
     ) -> None:
+        # local_files_only: in the reference's signature (runtime/engine.py:125-146); this engine
+        # reads local folders only, whatever its value.
+        del local_files_only
         from turboserve_amd.cache.layout import CacheLayout
         from turboserve_amd.cache.storage import CacheStorage
         from turboserve_amd.engine.loading import load_model

@@ -21,4 +21,5 @@ class RequestOutput:
     timing: RequestTiming | None = None
     prompt_tokens: int = 0
     output_tokens: int = 0
+    cached_prompt_tokens: int = 0  # always 0: there is no prefix cache (types.py:596-634 has the field)
     logprobs: list[float] = field(default_factory=list)

@@ -136,6 +136,14 @@ def test_command_line_options_are_the_references():
     assert (kv.max_num_seqs, kv.gpu_memory_utilization, kv.max_model_len, kv.block_size) == (64, 0.9, None, 16)
     assert build_parser().parse_args(["hwinfo"]).indent == 2
     assert build_parser().parse_args(["version"]).command == "version"
+    # the reference's flags for what is not built: accepted switched off, refused switched on
+    off = build_parser().parse_args(["engine", "generate", "hi", "-m", "m", "--offline", "--no-prefix-caching"])
+    assert off.offline and off.prefix_caching is False
+    assert build_parser().parse_args(["engine", "kv-size", "-m", "m", "--offline"]).prefix_caching is False
+    from turboserve_amd.cli import main
+
+    with pytest.raises(ValueError, match="no prefix cache"):
+        main(["engine", "generate", "--prompt-ids", "1", "-m", "m", "--prefix-caching"])
 
 
 def test_the_run_order_is_data():

@@ -9,8 +9,9 @@ src/turboserve/engine/runtime/engine.py:515-641)::
 Option names, defaults and meanings are the reference's where it has them (``--max-tokens 64``,
 ``--temperature 0`` = greedy, ``--max-num-seqs 8`` for ``generate`` and 64 for ``kv-size``,
 ...).  Added here: ``--prompt-ids`` (prompts as comma-separated token ids, so no tokenizer is
-needed), ``--top-k``, ``--repetition-penalty`` and the ``random-model`` command.  Not here:
-``--prefix-caching`` and ``--offline`` (there is no prefix cache and no download).
+needed), ``--top-k``, ``--repetition-penalty`` and the ``random-model`` command.  The
+reference's ``--offline`` and ``--no-prefix-caching`` are accepted and change nothing (there is
+no download and no prefix cache); ``--prefix-caching`` is refused with that reason.
 """
 
 from __future__ import annotations
@@ -30,6 +31,11 @@ def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> Non
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--max-num-seqs", type=int, default=max_num_seqs)
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    p.add_argument("--offline", action="store_true", help="accepted for the reference's command lines: nothing is ever downloaded")
+    p.add_argument("--prefix-caching", dest="prefix_caching", action="store_true",
+                   help="refused: this engine has no prefix cache")
+    p.add_argument("--no-prefix-caching", dest="prefix_caching", action="store_false", help="accepted: the only mode")
+    p.set_defaults(prefix_caching=False)
     p.add_argument("--tune-gemm", action="store_true",
                    help="time the BLAS library's kernels for a full step of prompt tokens at start-up and keep the fastest")
 
@@ -89,7 +95,7 @@ def _generate(args: argparse.Namespace) -> int:
         tune_gemm_tokens=(args.max_num_batched_tokens,) if args.tune_gemm else (),
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
-            block_size=args.block_size, num_blocks=args.num_blocks,
+            block_size=args.block_size, num_blocks=args.num_blocks, enable_prefix_caching=args.prefix_caching,
         ),
     )
     sampling = SamplingParams(
@@ -125,7 +131,7 @@ def _kv_size(args: argparse.Namespace) -> int:
         gpu_memory_utilization=args.gpu_memory_utilization, max_model_len=args.max_model_len,
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
-            block_size=args.block_size,
+            block_size=args.block_size, enable_prefix_caching=args.prefix_caching,
         ),
     )
     model_config, model = describe_model(read_config_json(config.model))

@@ -64,6 +64,13 @@ def test_preemption_keeps_the_tokens(model):
         assert [o.new_token_ids for o in outputs] == want
         assert engine.stats()["num_preemptions"] > 0
         engine.scheduler.check_invariants()
+        # the structured snapshot of the reference (engine.py:80-115), merged into the flat one
+        snapshot = engine.engine_stats()
+        assert snapshot.num_finished == len(model["prompts"]) and snapshot.num_unfinished == 0
+        assert snapshot.num_generated_tokens == new * len(model["prompts"])
+        assert snapshot.kv_utilization == 0.0 and snapshot.prefix_hit_rate == 0.0
+        assert engine.stats()["num_generated_tokens"] == snapshot.num_generated_tokens
+        assert str(engine.device) == "cuda:0" and engine.dtype == torch.float32
 
 
 def test_temperature_sampling_follows_the_rule(model):

@@ -8,10 +8,12 @@ tiny pool or a stand-in runner.
 
 from __future__ import annotations
 
-import logging
 import contextlib
+import dataclasses
+import logging
 import time
 from collections.abc import Sequence as SequenceABC
+from dataclasses import dataclass
 from typing import Any
 
 import torch
@@ -26,6 +28,28 @@ from turboserve_amd.engine.sequence import Sequence
 from turboserve_amd.sampling.params import FinishReason, SamplingParams
 
 logger = logging.getLogger(__name__)
+
+
+@dataclass(frozen=True)
+class EngineStats:
+    """A snapshot of engine health (engine.py:80-115).  The two prefix-cache fields are in the
+    reference's record and always zero here: there is no prefix cache."""
+
+    num_running: int
+    num_waiting: int
+    num_preempted: int
+    num_unfinished: int
+    num_finished: int
+    num_preemptions: int
+    num_steps: int
+    kv_utilization: float  # fraction of cache pages held by requests, the fullest group's
+    prefix_hit_rate: float
+    num_prompt_tokens: int
+    num_generated_tokens: int
+    num_cached_prompt_tokens: int
+
+    def to_dict(self) -> dict[str, int | float]:
+        return dataclasses.asdict(self)
 
 
 class LLMEngine:
@@ -296,11 +320,34 @@ class LLMEngine:
 
     # -- observability --------------------------------------------------------------------------
 
+    @property
+    def device(self) -> torch.device:
+        return self.model.runtime.device
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.model.runtime.dtype
+
+    def engine_stats(self) -> EngineStats:
+        """Structured snapshot (engine.py:452-468)."""
+        raw = self.scheduler.stats()
+        utilization = 0.0
+        for pool in self.scheduler.cache.pools:
+            if pool.num_pages:
+                utilization = max(utilization, pool.num_in_use / pool.num_pages)
+        return EngineStats(
+            num_running=int(raw["num_running"]), num_waiting=int(raw["num_waiting"]),
+            num_preempted=int(raw["num_preempted"]), num_unfinished=int(raw["num_unfinished"]),
+            num_finished=int(raw["num_finished"]), num_preemptions=int(raw["num_preemptions"]),
+            num_steps=int(raw["num_steps"]), kv_utilization=utilization, prefix_hit_rate=0.0,
+            num_prompt_tokens=self._num_prompt_tokens, num_generated_tokens=self._num_generated_tokens,
+            num_cached_prompt_tokens=0,
+        )
+
     def stats(self) -> dict[str, int | float | str]:
-        """Flat, JSON-safe counters (engine.py:452-484)."""
+        """Flat, JSON-safe counters (engine.py:470-484)."""
         out: dict[str, int | float | str] = dict(self.scheduler.stats())
-        out["num_prompt_tokens"] = self._num_prompt_tokens
-        out["num_generated_tokens"] = self._num_generated_tokens
+        out.update(self.engine_stats().to_dict())
         out["model"] = self.config.model
         runtime = getattr(self.model, "runtime", None)
         if runtime is not None:

@@ -165,6 +165,16 @@ def test_engine_and_sampling_options():
     from turboserve_amd.engine.outputs import RequestOutput
 
     assert RequestOutput(request_id="r").cached_prompt_tokens == 0
+    with pytest.raises(ValueError, match="not built"):
+        EngineConfig(model="m", speculative={"model": "draft"})
+    env = {"TURBOSERVE_MODEL": "/models/q", "TURBOSERVE_DTYPE": "float32", "TURBOSERVE_MAX_NUM_SEQS": "12",
+           "TURBOSERVE_BLOCK_SIZE": "32", "TURBOSERVE_ENABLE_CHUNKED_PREFILL": "false", "TURBOSERVE_NUM_BLOCKS": ""}
+    from_env = EngineConfig.from_env(env, seed=7)
+    assert (from_env.model, from_env.dtype, from_env.seed) == ("/models/q", "float32", 7)
+    assert (from_env.scheduler.max_num_seqs, from_env.block_size, from_env.num_blocks) == (12, 32, None)
+    assert from_env.scheduler.enable_chunked_prefill is False and from_env.scheduler.max_num_batched_tokens == 2048
+    with pytest.raises(ValueError, match="TURBOSERVE_MODEL"):
+        EngineConfig.from_env({})
     config = EngineConfig(model="m")
     assert config.resolved_dtype() == "bfloat16" and config.resolved_device() == "cuda:0"
     assert config.gpu_memory_utilization == 0.9 and config.block_size == 16 and config.num_blocks is None

@@ -8,7 +8,10 @@ is on; here it must be off) and ``policy`` (first come, first served).
 
 from __future__ import annotations
 
+import os
+from collections.abc import Mapping
 from dataclasses import dataclass, field
+from typing import Any
 
 
 @dataclass
@@ -55,6 +58,10 @@ class EngineConfig:
     max_model_len: int | None = None
     seed: int | None = None
     scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
+    #: In the reference's record (types.py:543-547) for subsystems that are not built here:
+    #: only ``None`` is accepted.
+    speculative: dict | None = None
+    lora: dict | None = None
     #: Step sizes (tokens) at which the BLAS library's kernels for this model's projections are
     #: timed at start-up and the fastest kept (bfloat16 only; a few seconds per size).  Empty:
     #: the library's own heuristic picks.  No counterpart in the reference.
@@ -67,6 +74,8 @@ class EngineConfig:
     choose_products: bool = True
 
     def __post_init__(self) -> None:
+        if self.speculative is not None or self.lora is not None:
+            raise ValueError("speculative decoding and LoRA are not built: leave `speculative` and `lora` at None")
         if self.dtype not in ("auto", "bfloat16", "float32"):
             raise ValueError(f"unsupported dtype {self.dtype!r}; expected auto, bfloat16 or float32")
         if self.device != "auto" and not self.device.startswith("cuda"):
@@ -78,6 +87,45 @@ class EngineConfig:
         self.tune_gemm_tokens = tuple(self.tune_gemm_tokens)
         if any(isinstance(t, bool) or not isinstance(t, int) or t < 1 for t in self.tune_gemm_tokens):
             raise ValueError(f"tune_gemm_tokens must be ints >= 1, got {self.tune_gemm_tokens!r}")
+
+    @classmethod
+    def from_env(cls, environ: Mapping[str, str] | None = None, **overrides: Any) -> "EngineConfig":
+        """An engine configuration from the process-wide ``TURBOSERVE_*`` variables the
+        reference's settings read (src/turboserve/config.py:38-64, types.py:575-593): MODEL,
+        DTYPE, DEVICE, GPU_MEMORY_UTILIZATION, MAX_NUM_SEQS, MAX_NUM_BATCHED_TOKENS, BLOCK_SIZE,
+        NUM_BLOCKS, ENABLE_CHUNKED_PREFILL.  Unset variables keep this class's defaults;
+        ``overrides`` win over the environment."""
+        env = os.environ if environ is None else environ
+
+        def get(name: str, convert):
+            raw = env.get(f"TURBOSERVE_{name}")
+            return None if raw is None or raw == "" else convert(raw)
+
+        def truth(raw: str) -> bool:
+            if raw.strip().lower() in ("1", "true", "yes", "on"):
+                return True
+            if raw.strip().lower() in ("0", "false", "no", "off"):
+                return False
+            raise ValueError(f"not a boolean: {raw!r}")
+
+        scheduler = {k: v for k, v in {
+            "max_num_seqs": get("MAX_NUM_SEQS", int),
+            "max_num_batched_tokens": get("MAX_NUM_BATCHED_TOKENS", int),
+            "block_size": get("BLOCK_SIZE", int),
+            "num_blocks": get("NUM_BLOCKS", int),
+            "enable_chunked_prefill": get("ENABLE_CHUNKED_PREFILL", truth),
+        }.items() if v is not None}
+        fields = {k: v for k, v in {
+            "model": get("MODEL", str),
+            "dtype": get("DTYPE", str),
+            "device": get("DEVICE", str),
+            "gpu_memory_utilization": get("GPU_MEMORY_UTILIZATION", float),
+        }.items() if v is not None}
+        fields["scheduler"] = SchedulerConfig(**scheduler)
+        fields.update(overrides)
+        if "model" not in fields:
+            raise ValueError("no model: set TURBOSERVE_MODEL or pass model=")
+        return cls(**fields)
 
     @property
     def block_size(self) -> int:

@@ -127,6 +127,12 @@ class LLMEngine:
 
     # -- helpers --------------------------------------------------------------------------------
 
+    @classmethod
+    def from_env(cls, environ=None, **kwargs: Any) -> "LLMEngine":
+        """An engine built from the ``TURBOSERVE_*`` variables (engine.py:218-221 builds one
+        from the reference's settings object, which reads the same variables)."""
+        return cls(EngineConfig.from_env(environ), **kwargs)
+
     def _tune_library_products(self) -> None:
         """Time the BLAS library's kernels for this model's projections at the configured step
         sizes (dry steps that leave the cache alone) and keep the fastest."""

@@ -12,11 +12,8 @@ One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` time
 2,048-token prompt; ``roofline`` prices the decode step against HBM bandwidth; ``points``
 holds decode at batch 1 and 64.  The prefill's projections are BLAS-library products; which
 of the library's kernels runs each is timed once before the measurement
-(``--no-gemm-tuning`` leaves it to the library's heuristic).  At batch 64 each projection shape
-runs on the faster of this engine's product kernel and the library, timed once as an engine does
-at start-up (``product_choice`` in the line says which; ``--no-product-choice`` keeps the engine's
-kernel everywhere).  Peaks are the published MI355X figures: HBM 8 TB/s, dense bf16 MFMA
-2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+(``--no-gemm-tuning`` leaves it to the library's heuristic).  Peaks are the published MI355X
+figures: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
 """
 
 from __future__ import annotations
@@ -72,8 +69,6 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--no-gemm-tuning", action="store_true",
                    help="leave the choice of the BLAS library's prefill kernels to its heuristic")
-    p.add_argument("--no-product-choice", action="store_true",
-                   help="batches above 16: keep this engine's product kernel for every shape (no timed choice)")
     p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     p.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (the default run is 7b)")
     p.add_argument("--fill-hbm", action="store_true",
@@ -264,7 +259,6 @@ def main() -> int:
     dtype_key = "bf16" if dtype == torch.bfloat16 else "fp32"
 
     pool_tokens = 0
-    product_notes: dict[int, str] = {}
 
     def decode_rate(batch: int, steps: int, warmup: int) -> tuple[float, float]:
         nonlocal pool_tokens
@@ -276,20 +270,6 @@ def main() -> int:
 
             with LibraryGemmTuning(os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")):
                 bench.runner.dry_run(args.mixed_prefill + batch)
-        if 16 < batch <= 64 and not args.mixed_prefill and not args.no_product_choice and dtype == torch.bfloat16:
-            # As an engine does at start-up: own product kernel or library, per shape, by timing.
-            import contextlib
-
-            from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
-            from turboserve_amd.kernels.product_choice import choose_products, product_bucket
-
-            tuning = (contextlib.nullcontext() if args.no_gemm_tuning else LibraryGemmTuning(
-                os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")))
-            with tuning:
-                timings = choose_products(runtime.ops, lambda m: bench.runner.dry_run(m, want_all=True),
-                                          [product_bucket(batch)])
-            product_notes[batch] = ", ".join(
-                f"{t.out_features}x{t.in_features}:{'library' if t.library_chosen else 'own'}" for t in timings)
         seconds = bench.run(steps, warmup, args.mixed_prefill)
         bench.close()
         return batch * steps / seconds, seconds / steps
@@ -376,8 +356,6 @@ def main() -> int:
             rate, _ = decode_rate(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
             points[f"decode_b{batch}"] = round(rate, 2)
         result["points"] = points
-    if product_notes:
-        result["product_choice"] = {f"b{b}": note for b, note in product_notes.items()}
     info = collect()
     result["hw"] = {"gpu": info["gpu_name"], "torch": info["torch"]["version"], "hip": info["torch"]["hip_version"],
                     "git": (info["git"]["sha"] or "")[:12]}

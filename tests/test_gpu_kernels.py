@@ -117,60 +117,71 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(7, 8), (130, 104), (320, 96), (3584, 1000), (301, 2056), (4608, 3584)])
+@pytest.mark.parametrize("n,k", [(7, 8), (130, 104), (320, 96), (3584, 1000), (301, 2056), (4608, 3584), (33000, 136)])
 def test_gemm_skinny(ops, m, n, k):
     """The decode-sized product: 32-bit partial sums over ranges of K whose sum is the product,
-    for row counts around the 16-row tiles, N that is no multiple of 64 or 4, K that is no
-    multiple of the 256-wide chunk, one split and many."""
+    for row counts around the 16-row tiles, N that is no multiple of a tile or of 4, K that is
+    no multiple of the kernels' depth (128 and 256), one split and many, a matrix wide enough
+    for the resident kernel to take the fewest rows."""
     g = torch.Generator().manual_seed(m * n + k)
     x = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
     b = torch.randn(n, generator=g).bfloat16()
     want = x.double() @ w.double().T + b.double()
-    for max_splits in (None, 1):
-        partial = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV), max_splits=max_splits)
-        assert partial.dtype == torch.float32 and partial.shape[1:] == (m, n)
-        if max_splits == 1:
-            assert partial.shape[0] == 1
-        got = partial.double().sum(0).cpu()
-        assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1)
+    bound = 2e-5 * math.sqrt(k) * float(want.abs().max() + 1)
+    products = [lambda **kw: ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV), **kw),
+                lambda **kw: ops.gemm_tiled(x.to(DEV), w.to(DEV), b.to(DEV), **kw)]
+    if m <= 16:
+        products.append(lambda **kw: ops.gemm_resident(x.to(DEV), w.to(DEV), b.to(DEV), **kw))
+    for product in products:
+        for max_splits in (None, 1):
+            partial = product(max_splits=max_splits)
+            assert partial.dtype == torch.float32 and partial.shape[1:] == (m, n)
+            if max_splits == 1:
+                assert partial.shape[0] == 1
+            assert float((partial.double().sum(0).cpu() - want).abs().max()) <= bound
     none = ops.gemm_skinny(x.to(DEV), torch.zeros_like(w).to(DEV), b.to(DEV)).sum(0).cpu()
     torch.testing.assert_close(none, b.float().expand(m, n), rtol=0, atol=0)  # the bias, once
 
 
+@pytest.mark.parametrize("tile", [2, 4, 5])
+@pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (40, 64, 40)])
+def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
+    """The tiled product with its grid given by hand: every tile size, ranges of K of one
+    iteration and of several, a last range that is shorter, a last tile of rows that is partly
+    beyond N, a K below one iteration."""
+    g = torch.Generator().manual_seed(tile * 1000 + n)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    want = x.double() @ w.double().T
+    iters = -(-k // 128)
+    for per_split in sorted({1, 2, iters, max(1, iters - 1)}):
+        splits = -(-iters // per_split)
+        partial = ops.gemm_tiled(x.to(DEV), w.to(DEV), plan=(per_split, splits, tile))
+        assert partial.shape == (splits, m, n)
+        got = partial.double().sum(0).cpu()
+        assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1), per_split
+
+
 def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):
-    """A row's sums are the same bits whatever else is in the batch, within each of the two
-    variants (up to 16 rows with resident activations, up to 64 staged chunk by chunk); between
-    the variants the ranges of K may differ, so only the rounding of 32-bit sums does."""
+    """A row's sums are the same bits whatever else is in the batch, for a given grid of the
+    tiled kernel and within the resident kernel; between grids the ranges of K differ, so only
+    the rounding of 32-bit sums does."""
     g = torch.Generator().manual_seed(4)
     x = torch.randn(40, 1000, generator=g).bfloat16()
     w = torch.randn(200, 1000, generator=g).bfloat16()
-    full = ops.gemm_skinny(x.to(DEV), w.to(DEV)).cpu()
-    some = ops.gemm_skinny(x[10:30].to(DEV), w.to(DEV)).cpu()
-    assert torch.equal(full[:, 17:18], some[:, 7:8])
-    small = ops.gemm_skinny(x[5:21].to(DEV), w.to(DEV)).cpu()
-    nine = ops.gemm_skinny(x[12:21].to(DEV), w.to(DEV)).cpu()
-    one = ops.gemm_skinny(x[17:18].to(DEV), w.to(DEV)).cpu()
-    assert torch.equal(small[:, 12:13], one) and torch.equal(nine[:, 5:6], one)
-    torch.testing.assert_close(full.sum(0)[17:18], one.sum(0), rtol=1e-5, atol=1e-3)
-
-
-@pytest.mark.parametrize("m", [1, 7, 16])
-@pytest.mark.parametrize("hidden,inter", [(96, 200), (320, 2056), (3584, 18944)])
-def test_swiglu_inside_the_down_product(ops, m, hidden, inter):
-    """The down projection that applies SwiGLU to the gate|up partial sums while staging them
-    gives, bit for bit, what the stand-alone SwiGLU kernel followed by the product gives."""
-    g = torch.Generator().manual_seed(m + inter)
-    gate_up = torch.randn(3, m, 2 * inter, generator=g).to(DEV)
-    w = (torch.randn(hidden, inter, generator=g) * 0.05).bfloat16().to(DEV)
-    assert ops.swiglu_linear_possible(gate_up, w)
-    fused = ops.swiglu_linear(gate_up, w)
-    plain_way = ops.gemm_skinny(ops.swiglu(gate_up, torch.bfloat16), w)
-    assert torch.equal(fused, plain_way)
-    total = gate_up.sum(0).double().cpu()
-    act = torch.nn.functional.silu(total[:, :inter]) * total[:, inter:]
-    want = act.bfloat16().double() @ w.double().cpu().T
-    assert float((fused.sum(0).double().cpu() - want).abs().max()) <= 2e-2 * float(want.abs().max() + 1)
+    plan = (3, 3, 2)
+    full = ops.gemm_tiled(x.to(DEV), w.to(DEV), plan=plan).cpu()
+    some = ops.gemm_tiled(x[10:30].to(DEV), w.to(DEV), plan=plan).cpu()
+    one = ops.gemm_tiled(x[17:18].to(DEV), w.to(DEV), plan=plan).cpu()
+    assert torch.equal(full[:, 17:18], some[:, 7:8]) and torch.equal(full[:, 17:18], one)
+    small = ops.gemm_resident(x[5:21].to(DEV), w.to(DEV)).cpu()
+    nine = ops.gemm_resident(x[12:21].to(DEV), w.to(DEV)).cpu()
+    alone = ops.gemm_resident(x[17:18].to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(small[:, 12:13], alone) and torch.equal(nine[:, 5:6], alone)
+    torch.testing.assert_close(full.sum(0)[17:18], alone.sum(0), rtol=1e-5, atol=1e-3)
+    other = ops.gemm_skinny(x.to(DEV), w.to(DEV)).cpu()  # the grid the engine would choose
+    torch.testing.assert_close(full.sum(0), other.sum(0), rtol=1e-5, atol=1e-3)
 
 
 def test_consumers_add_up_partial_sums(ops):

@@ -68,10 +68,6 @@ class EngineConfig:
     tune_gemm_tokens: tuple[int, ...] = ()
     #: Where the timed choices are kept between runs; None is a per-user cache file.
     gemm_tuning_file: str | None = None
-    #: Time this engine's product kernel against the BLAS library for decode steps of 17 to 64
-    #: requests at start-up and let each projection shape run on the faster (bfloat16 only, under
-    #: a second; skipped when ``max_num_seqs`` is at most 16).  No counterpart in the reference.
-    choose_products: bool = True
 
     def __post_init__(self) -> None:
         if self.speculative is not None or self.lora is not None:

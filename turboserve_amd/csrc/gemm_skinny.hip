@@ -1,21 +1,20 @@
-// Weight-streaming product for decode-sized batches:
+// Weight-streaming product for a few rows, activations resident in LDS:
 //   partial[s][m][n] = sum over the k-range of split s of  X[m][k] * W[n][k]   (+ bias[n] in split 0)
-// for M <= 64 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
+// for M <= 16 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
 // them (F.linear's layout, src/turboserve/engine/model/layers.py:142), 32-bit accumulation on
 // the matrix cores and 32-bit partial sums out.  The consumer (norm, rotary/cache write,
 // SwiGLU, or nobody when splits == 1) adds the splits up, so no rounding happens between the
-// product and its consumer.
+// product and its consumer.  (gemm_tiled.hip holds the product for up to 64 rows; this one
+// serves small matrices, whose product lasts a few microseconds and gains from many small
+// workgroups that start quickly, and the widest matrices at up to four rows.)
 //
-// At these batch sizes the product is bound by reading W once from HBM.  Layout of the work:
+// The product is bound by reading W once from HBM.  Layout of the work:
 //   * a workgroup of 4 or 8 wavefronts owns 64 or 128 consecutive weight rows (16 per
 //     wavefront) and one k-range; the grid is (row blocks, splits);
 //   * the k-range is walked in chunks of 256: eight loads per lane, each of which has the four
 //     lane groups of a weight row cover 64 contiguous bytes (so a load instruction touches 16
 //     rows x 64 bytes, and the eight of a chunk 512 contiguous bytes per row), issued one chunk
 //     ahead of the matrix cores;
-//   * the chunk's activations are staged once per workgroup in LDS (rows padded against bank
-//     conflicts) and read as B operands by all four wavefronts; they are fetched from global
-//     memory into registers two chunks ahead and written to LDS one chunk ahead;
 //   * v_mfma_f32_16x16x32_bf16 with A = 16 weight rows, B = 16 activation rows, step j of a
 //     chunk covering k = chunk + 32 j .. + 31.
 #include "common.hpp"
@@ -29,7 +28,6 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int CHUNK = 256;          // k per iteration
 constexpr int STEPS = CHUNK / 32;   // matrix-core steps per chunk
 constexpr int ROWS_PER_WAVE = 16;
-constexpr int X_ROW = CHUNK + 8;    // LDS row stride in elements (16 bytes of padding)
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
@@ -53,156 +51,16 @@ __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row
   }
 }
 
-// The activations of one chunk, X[0..m-1][k0 .. k0+255], travel in two hops: global memory to
-// registers (issued a whole iteration before they are needed), registers to LDS.  A thread
-// carries 2 MT pieces of 16 bytes; rows >= m and k >= K are zeros.
-template <int MT, int WAVES>
-struct ActivationRegs {
-  static constexpr int PIECES = (MT * 16 * (CHUNK / 8) + WAVES * TS_WAVE - 1) / (WAVES * TS_WAVE);
-  u32x4 piece[PIECES];
-};
-
-template <int MT, int WAVES>
-__device__ __forceinline__ void fetch_activations(ActivationRegs<MT, WAVES>& r, const uint16_t* __restrict__ x,
-                                                  long x_stride, int m, int k0, int k_limit) {
-#pragma unroll
-  for (int i = 0; i < ActivationRegs<MT, WAVES>::PIECES; ++i) {
-    const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
-    const int row = idx / (CHUNK / 8);
-    const int k = k0 + 8 * (idx % (CHUNK / 8));
-    r.piece[i] = (row < m && k < k_limit) ? *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + k)
-                                          : u32x4{0u, 0u, 0u, 0u};
-  }
-}
-
-template <int MT, int WAVES>
-__device__ __forceinline__ void store_activations(uint16_t* lds, const ActivationRegs<MT, WAVES>& r) {
-#pragma unroll
-  for (int i = 0; i < ActivationRegs<MT, WAVES>::PIECES; ++i) {
-    const int idx = threadIdx.x + i * (WAVES * TS_WAVE);
-    if (idx < MT * 16 * (CHUNK / 8))
-      *reinterpret_cast<u32x4*>(lds + (idx / (CHUNK / 8)) * X_ROW + 8 * (idx % (CHUNK / 8))) = r.piece[i];
-  }
-}
-
-template <int MT>
-__device__ __forceinline__ void multiply_chunk(f32x4 (&acc)[MT], const WeightChunk& w, const uint16_t* xs,
-                                               int lane16, int group) {
-#pragma unroll
-  for (int j = 0; j < STEPS; ++j) {
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const u32x4 b = *reinterpret_cast<const u32x4*>(xs + (16 * t + lane16) * X_ROW + 8 * group + 32 * j);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w.piece[j]), as_bf16x8(b), acc[t], 0, 0, 0);
-    }
-  }
-}
-
-template <int MT, int WAVES>
-__global__ void __launch_bounds__(WAVES * TS_WAVE)
-gemm_skinny_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
-                   const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
-                   int chunks_per_split) {
-  __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16 * X_ROW];
-  const int lane = threadIdx.x & (TS_WAVE - 1);
-  const int wave = threadIdx.x / TS_WAVE;
-  const int lane16 = lane & 15;
-  const int group = lane >> 4;
-  const int split = blockIdx.y;
-  const int n0 = (blockIdx.x * WAVES + wave) * ROWS_PER_WAVE;
-  const int total_chunks = (k + CHUNK - 1) / CHUNK;
-  const int first = split * chunks_per_split;
-  const int last = min(first + chunks_per_split, total_chunks);  // exclusive
-
-  // Rows beyond N repeat the last row; their sums are never stored.
-  const int row_index = min(n0 + lane16, n - 1);
-  const uint16_t* wrow = w + (size_t)row_index * k;
-
-  f32x4 acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  if (first < last) {
-    // Invariant at the top of a round for chunk c: xs[buf] holds chunk c (complete, behind a
-    // barrier), `xr` holds chunk c + 1's activations (loads issued a round ago), and the
-    // weight registers of this round hold chunk c.
-    WeightChunk wa, wb;
-    ActivationRegs<MT, WAVES> xr;
-    load_weights(wa, wrow, first * CHUNK, group, k);
-    fetch_activations<MT, WAVES>(xr, x, x_stride, m, first * CHUNK, k);
-    store_activations<MT, WAVES>(xs[0], xr);
-    if (first + 1 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (first + 1) * CHUNK, k);
-    __syncthreads();
-    int c = first;
-    int buf = 0;
-    while (true) {
-      if (c + 1 < last) {
-        store_activations<MT, WAVES>(xs[buf ^ 1], xr);  // free since the last barrier
-        load_weights(wb, wrow, (c + 1) * CHUNK, group, k);
-        if (c + 2 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
-      }
-      multiply_chunk<MT>(acc, wa, xs[buf], lane16, group);
-      __syncthreads();
-      if (++c >= last) break;
-      buf ^= 1;
-      if (c + 1 < last) {
-        store_activations<MT, WAVES>(xs[buf ^ 1], xr);
-        load_weights(wa, wrow, (c + 1) * CHUNK, group, k);
-        if (c + 2 < last) fetch_activations<MT, WAVES>(xr, x, x_stride, m, (c + 2) * CHUNK, k);
-      }
-      multiply_chunk<MT>(acc, wb, xs[buf], lane16, group);
-      __syncthreads();
-      if (++c >= last) break;
-      buf ^= 1;
-    }
-  }
-
-  // acc[t][i] = sum for weight row n0 + 4 g + i and activation row 16 t + lane16.
-  const int nrow = n0 + 4 * group;
-  if (nrow < n) {
-    f32x4 b = {0.f, 0.f, 0.f, 0.f};
-    if (bias && split == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (nrow + i < n) b[i] = to_float(bf16_t{bias[nrow + i]});
-    }
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int row = 16 * t + lane16;
-      if (row >= m) continue;
-      float* dst = partial + ((size_t)split * m + row) * n + nrow;
-      const f32x4 v = acc[t] + b;
-      if (nrow + 3 < n && (n & 3) == 0) {
-        *reinterpret_cast<f32x4*>(dst) = v;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (nrow + i < n) dst[i] = v[i];
-      }
-    }
-  }
-}
-
-
 // The same product for M <= 16 with the activations resident in LDS: a workgroup stages its
 // split's activations X[0..mpad-1][k-range] once (in stretches of `stage_chunks` chunks when
 // the range is longer than LDS should hold) and its wavefronts then stream their weight rows
 // without meeting at a barrier again, two chunks of loads in flight each.  mpad is 8 or 16;
 // lanes whose activation row is beyond mpad read a real row again and drop the result.
-//
-// GATED: the activations do not exist yet.  `x` then points at the 32-bit partial sums
-// [gated_splits, m, 2 k] of a fused gate|up projection (row stride x_stride, splits
-// gated_stride elements apart) and the staging computes silu(gate) * up from them, rounded to
-// bfloat16 once, exactly as the stand-alone SwiGLU kernel does: one kernel and one pass over
-// that intermediate fewer per layer.
-template <int WAVES, bool GATED>
+template <int WAVES>
 __global__ void __launch_bounds__(WAVES * TS_WAVE)
-gemm_skinny_resident_kernel(float* __restrict__ partial, const void* __restrict__ x_any, long x_stride,
-                            int gated_splits, long gated_stride, const uint16_t* __restrict__ w,
-                            const uint16_t* __restrict__ bias, int m, int mpad, int n, int k, int chunks_per_split,
-                            int stage_chunks) {
-  const uint16_t* x = static_cast<const uint16_t*>(x_any);
-  const float* xg = static_cast<const float*>(x_any);
+gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
+                            const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int mpad,
+                            int n, int k, int chunks_per_split, int stage_chunks) {
   extern __shared__ __attribute__((aligned(16))) uint16_t xs_resident[];
   const int lane = threadIdx.x & (TS_WAVE - 1);
   const int wave = threadIdx.x / TS_WAVE;
@@ -237,32 +95,7 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const void* __restrict_
         if (piece >= live_pieces) continue;
         const int kk = k_begin + 8 * piece;
         u32x4 v = {0u, 0u, 0u, 0u};
-        if (row < m && kk < k) {
-          if (GATED) {
-            float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            for (int sp = 0; sp < gated_splits; ++sp) {
-              const float* src = xg + (size_t)sp * gated_stride + (size_t)row * x_stride + kk;
-#pragma unroll
-              for (int h = 0; h < 2; ++h) {
-                const f32x4 a = *reinterpret_cast<const f32x4*>(src + 4 * h);
-                const f32x4 b = *reinterpret_cast<const f32x4*>(src + k + 4 * h);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  g[4 * h + e] += a[e];
-                  u[4 * h + e] += b[e];
-                }
-              }
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float lo = g[2 * e] / (1.f + expf(-g[2 * e])) * u[2 * e];
-              const float hi = g[2 * e + 1] / (1.f + expf(-g[2 * e + 1])) * u[2 * e + 1];
-              v[e] = (uint32_t)from_float<bf16_t>(lo).bits | ((uint32_t)from_float<bf16_t>(hi).bits << 16);
-            }
-          } else {
-            v = *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + kk);
-          }
-        }
+        if (row < m && kk < k) v = *reinterpret_cast<const u32x4*>(x + (size_t)row * x_stride + kk);
         *reinterpret_cast<u32x4*>(xs_resident + row * x_row + 8 * piece) = v;
       }
       __syncthreads();
@@ -309,56 +142,18 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const void* __restrict_
 
 }  // namespace
 
-template <int WAVES>
-static int launch_skinny(float* partial, const uint16_t* x, long x_stride, const uint16_t* w, const uint16_t* bias,
-                         int m, int n, int k, int chunks_per_split, int splits, hipStream_t stream) {
-  const int rows_per_block = WAVES * ROWS_PER_WAVE;
-  dim3 grid((n + rows_per_block - 1) / rows_per_block, splits), block(WAVES * TS_WAVE);
-  if (grid.y > 65535) return TS_ERR_SHAPE;
-  if (m <= 16)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
-  else if (m <= 32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
-  else if (m <= 48)
-    hipLaunchKernelGGL((gemm_skinny_kernel<3, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
-  else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, WAVES>), grid, block, 0, stream, partial, x, x_stride, w, bias, m, n, k, chunks_per_split);
-  return ts_launch_status();
-}
-
-// partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
-// w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
-// chunks_per_split 256-wide chunks of k go to each of `splits` = ceil(ceil(k / 256) / chunks_per_split).
-// waves: wavefronts (16 weight rows each) per workgroup, 4 or 8.
-extern "C" int ts_gemm_skinny(float* partial, const void* x, long x_stride, const void* w, const void* bias,
-                              int m, int n, int k, int chunks_per_split, int splits, int waves, hipStream_t stream) {
-  if (m == 0 || n == 0) return TS_OK;
-  if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
-  if (m > 64 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
-  const int total_chunks = (k + CHUNK - 1) / CHUNK;
-  if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
-  if (waves == 4)
-    return launch_skinny<4>(partial, (const uint16_t*)x, x_stride, (const uint16_t*)w, (const uint16_t*)bias, m, n, k, chunks_per_split, splits, stream);
-  if (waves == 8)
-    return launch_skinny<8>(partial, (const uint16_t*)x, x_stride, (const uint16_t*)w, (const uint16_t*)bias, m, n, k, chunks_per_split, splits, stream);
-  return TS_ERR_SHAPE;
-}
-
-// The variant for m <= 16 that keeps a split's activations in LDS (see the kernel).  stage_chunks:
-// chunks staged at a time, an even number unless it covers a whole split; the LDS it needs,
+// partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride; w [n, k]
+// bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 16, k % 8 == 0.  chunks_per_split
+// 256-wide chunks of k go to each of `splits` = ceil(ceil(k / 256) / chunks_per_split).  waves:
+// wavefronts (16 weight rows each) per workgroup, 4 or 8.  stage_chunks: chunks staged at a time,
+// an even number unless it covers a whole split; the LDS it needs,
 // mpad * (min(stage_chunks, chunks_per_split) * 256 + 8) * 2 bytes with mpad = 8 or 16, must be <= 64 KiB.
-// gated_splits == 0: x is bfloat16 [m, k].  gated_splits >= 1: x is float [gated_splits, m, 2 k]
-// (splits gated_stride elements apart), the partial sums of a gate|up projection, and the
-// product's left operand is silu(gate) * up (k % 8 == 0, x_stride >= 2 k, no bias).
-static int skinny_resident(float* partial, const void* x, long x_stride, int gated_splits, long gated_stride,
-                           const void* w, const void* bias, int m, int n, int k, int chunks_per_split, int splits,
-                           int waves, int stage_chunks, hipStream_t stream) {
+extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
+                                       int m, int n, int k, int chunks_per_split, int splits, int waves,
+                                       int stage_chunks, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
-  const bool gated = gated_splits > 0;
-  if (m > 16 || (k & 7) != 0 || x_stride < (gated ? 2L * k : (long)k) || (x_stride & (gated ? 3 : 7)) != 0)
-    return TS_ERR_SHAPE;
-  if (gated && (bias || (gated_stride & 3) != 0)) return TS_ERR_ARG;
+  if (m > 16 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
   const int total_chunks = (k + CHUNK - 1) / CHUNK;
   if (chunks_per_split < 1 || splits != (total_chunks + chunks_per_split - 1) / chunks_per_split) return TS_ERR_SHAPE;
   if (stage_chunks < 1 || (stage_chunks < chunks_per_split && (stage_chunks & 1) != 0)) return TS_ERR_SHAPE;
@@ -366,33 +161,17 @@ static int skinny_resident(float* partial, const void* x, long x_stride, int gat
   const int stage = stage_chunks < chunks_per_split ? stage_chunks : chunks_per_split;
   const size_t lds = (size_t)mpad * (stage * CHUNK + 8) * sizeof(uint16_t);
   if (lds > 64 * 1024 || splits > 65535) return TS_ERR_SHAPE;
+  const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (waves != 4 && waves != 8) return TS_ERR_SHAPE;
   dim3 grid((n + 16 * waves - 1) / (16 * waves), splits), block(waves * TS_WAVE);
-#define TS_LAUNCH_RESIDENT(W, G)                                                                                   \
-  hipLaunchKernelGGL((gemm_skinny_resident_kernel<W, G>), grid, block, lds, stream, partial, x, x_stride,         \
-                     gated_splits, gated_stride, wp, bp, m, mpad, n, k, chunks_per_split, stage_chunks)
-  if (waves == 4 && !gated) TS_LAUNCH_RESIDENT(4, false);
-  else if (waves == 8 && !gated) TS_LAUNCH_RESIDENT(8, false);
-  else if (waves == 4) TS_LAUNCH_RESIDENT(4, true);
-  else TS_LAUNCH_RESIDENT(8, true);
-#undef TS_LAUNCH_RESIDENT
+  if (waves == 4)
+    hipLaunchKernelGGL((gemm_skinny_resident_kernel<4>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m,
+                       mpad, n, k, chunks_per_split, stage_chunks);
+  else if (waves == 8)
+    hipLaunchKernelGGL((gemm_skinny_resident_kernel<8>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m,
+                       mpad, n, k, chunks_per_split, stage_chunks);
+  else
+    return TS_ERR_SHAPE;
   return ts_launch_status();
-}
-
-extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
-                                       int m, int n, int k, int chunks_per_split, int splits, int waves,
-                                       int stage_chunks, hipStream_t stream) {
-  return skinny_resident(partial, x, x_stride, 0, 0, w, bias, m, n, k, chunks_per_split, splits, waves, stage_chunks,
-                         stream);
-}
-
-extern "C" int ts_gemm_skinny_resident_gated(float* partial, const float* gate_up, long row_stride, int gated_splits,
-                                             long gated_stride, const void* w, int m, int n, int k,
-                                             int chunks_per_split, int splits, int waves, int stage_chunks,
-                                             hipStream_t stream) {
-  if (gated_splits < 1) return TS_ERR_ARG;
-  return skinny_resident(partial, gate_up, row_stride, gated_splits, gated_stride, w, nullptr, m, n, k,
-                         chunks_per_split, splits, waves, stage_chunks, stream);
 }

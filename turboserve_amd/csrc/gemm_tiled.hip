@@ -1,0 +1,219 @@
+// Weight-streaming product for decode-sized batches, tiled through LDS:
+//   partial[s][m][n] = sum over the k-range of split s of  X[m][k] * W[n][k]   (+ bias[n] in split 0)
+// for M <= 64 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
+// them (F.linear's layout, src/turboserve/engine/model/layers.py:142), 32-bit accumulation on
+// the matrix cores and 32-bit partial sums out; the consumer adds the splits up.
+//
+// The product is bound by reading W once from HBM, and what decides its rate is how the reading
+// is spread over the device, not how much of it is in flight:
+//   * a workgroup of four wavefronts (2 x 2) owns a tile of NT = 32 TN weight rows (TN = 2, 4
+//     or 5) by all 64 activation rows and one range of K; the host sizes tiles and ranges so that
+//     the grid is about one workgroup per compute unit (two for the smallest tile): every
+//     compute unit then streams one contiguous block of each of its rows, start to end;
+//   * the range is walked 128 deep: both operands travel global memory -> registers (16-byte
+//     pieces; consecutive threads take consecutive pieces of a row, 256 contiguous bytes per row)
+//     -> LDS (two buffers, rows padded by 16 bytes against bank conflicts) -> matrix cores.  The
+//     loads of an iteration are issued one iteration ahead; more in flight measured slower;
+//   * every load is issued on every path (rows beyond N or M repeat the last row, iterations
+//     beyond the range repeat its last one), so the compiler can count the loads in flight and
+//     waits only for those it needs; pieces beyond K are cleared on their way into LDS;
+//   * a wavefront computes TN x 2 tiles of v_mfma_f32_16x16x32_bf16 (A = 16 weight rows, B = 16
+//     activation rows): each weight fragment it reads from LDS serves two products, each
+//     activation fragment TN.
+#include "common.hpp"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int DEPTH = 128;            // k per iteration
+constexpr int LDS_ROW = DEPTH + 8;    // LDS row stride in elements
+constexpr int M_TILE = 64;            // activation rows a workgroup covers (rows beyond M are repeats)
+constexpr int THREADS = 256;
+constexpr int ROW_PIECES = DEPTH / 8; // 16-byte pieces of a row of an iteration
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+template <int TN>
+struct TileRegs {
+  static constexpr int W_PIECES = 32 * TN * ROW_PIECES / THREADS;  // 2 TN
+  static constexpr int X_PIECES = M_TILE * ROW_PIECES / THREADS;   // 4
+  u32x4 w[W_PIECES];
+  u32x4 x[X_PIECES];
+};
+
+template <int TN>
+__global__ void __launch_bounds__(THREADS)
+gemm_tiled_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
+                  const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
+                  int iters_per_split) {
+  constexpr int NT = 32 * TN;
+  constexpr int STAGE = (NT + M_TILE) * LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
+  typedef TileRegs<TN> Regs;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [2][STAGE]
+  const int tid = threadIdx.x;
+  const int lane = tid & (TS_WAVE - 1);
+  const int wave = tid / TS_WAVE;
+  const int lane16 = lane & 15;
+  const int group = lane >> 4;
+  const int wave_n = wave >> 1;  // which half of the tile's weight rows
+  const int wave_m = wave & 1;   // which half of the activation rows
+  const int n_base = blockIdx.x * NT;
+  const int split = blockIdx.y;
+  const int total = (k + DEPTH - 1) / DEPTH;
+  const int first = split * iters_per_split;
+  const int last = min(first + iters_per_split, total);  // exclusive
+  if (first >= last) return;                              // the whole workgroup leaves together
+
+  // This thread's pieces: piece p = tid + 256 i of a tile is row p / 16, bytes 16 (p % 16) of the
+  // iteration's 256.  Source pointers are at k = 0; destinations are offsets inside a buffer.
+  const uint16_t* wsrc[Regs::W_PIECES];
+  const uint16_t* xsrc[Regs::X_PIECES];
+  const int piece_k = 8 * (tid % ROW_PIECES);
+  const int piece_row = tid / ROW_PIECES;  // rows advance by 16 per i
+#pragma unroll
+  for (int i = 0; i < Regs::W_PIECES; ++i)
+    wsrc[i] = w + (size_t)min(n_base + piece_row + 16 * i, n - 1) * k;
+#pragma unroll
+  for (int i = 0; i < Regs::X_PIECES; ++i)
+    xsrc[i] = x + (size_t)min(piece_row + 16 * i, m - 1) * x_stride;
+  const int dst = piece_row * LDS_ROW + piece_k;  // + 16 i rows
+
+  auto fetch = [&](Regs& r, int it) {
+    // Iterations beyond the range repeat its last one; a piece beyond K reads the last piece of
+    // the row instead (cleared in `stage`).
+    const int k0 = min(min(it, last - 1) * DEPTH + piece_k, k - 8);
+#pragma unroll
+    for (int i = 0; i < Regs::X_PIECES; ++i) r.x[i] = *reinterpret_cast<const u32x4*>(xsrc[i] + k0);
+#pragma unroll
+    for (int i = 0; i < Regs::W_PIECES; ++i) r.w[i] = *reinterpret_cast<const u32x4*>(wsrc[i] + k0);
+  };
+  auto stage = [&](const Regs& r, int buf, int it) {
+    uint16_t* base = lds + buf * STAGE + dst;
+    if ((it + 1) * DEPTH <= k) {  // the same in every thread; the usual case, kept free of selects
+#pragma unroll
+      for (int i = 0; i < Regs::X_PIECES; ++i) *reinterpret_cast<u32x4*>(base + (NT + 16 * i) * LDS_ROW) = r.x[i];
+#pragma unroll
+      for (int i = 0; i < Regs::W_PIECES; ++i) *reinterpret_cast<u32x4*>(base + 16 * i * LDS_ROW) = r.w[i];
+    } else {  // the last iteration of a K that is no multiple of 128 (or one past the end, never read)
+      const bool beyond = it * DEPTH + piece_k >= k;
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int i = 0; i < Regs::X_PIECES; ++i)
+        *reinterpret_cast<u32x4*>(base + (NT + 16 * i) * LDS_ROW) = beyond ? zero : r.x[i];
+#pragma unroll
+      for (int i = 0; i < Regs::W_PIECES; ++i)
+        *reinterpret_cast<u32x4*>(base + 16 * i * LDS_ROW) = beyond ? zero : r.w[i];
+    }
+  };
+
+  f32x4 acc[TN][2];
+#pragma unroll
+  for (int a = 0; a < TN; ++a) acc[a][0] = acc[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](int buf) {
+    const uint16_t* base = lds + buf * STAGE + lane16 * LDS_ROW + 8 * group;
+#pragma unroll
+    for (int step = 0; step < DEPTH / 32; ++step) {
+      u32x4 xf[2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 32 * wave_m + 16 * b) * LDS_ROW + 32 * step);
+#pragma unroll
+      for (int a = 0; a < TN; ++a) {
+        const u32x4 wf = *reinterpret_cast<const u32x4*>(base + (wave_n * TN + a) * 16 * LDS_ROW + 32 * step);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wf), as_bf16x8(xf[b]), acc[a][b], 0, 0, 0);
+      }
+    }
+  };
+
+  // Invariant at the top of a round for iteration `it`: LDS buffer (it - first) % 2 holds it
+  // (complete, behind a barrier) and `regs` holds iteration it + 1 (its loads were issued a
+  // round ago).
+  Regs regs;
+  fetch(regs, first);
+  stage(regs, 0, first);
+  fetch(regs, first + 1);
+  __syncthreads();
+  for (int it = first; it < last; ++it) {
+    const int buf = (it - first) & 1;
+    stage(regs, buf ^ 1, it + 1);  // that buffer was last read a round ago, before the barrier
+    fetch(regs, it + 2);
+    multiply(buf);
+    __syncthreads();
+  }
+
+  // acc[a][b][i] = sum for weight row n_base + 16 (wave_n TN + a) + 4 g + i and activation row
+  // 32 wave_m + 16 b + lane16.
+#pragma unroll
+  for (int a = 0; a < TN; ++a) {
+    const int nrow = n_base + (wave_n * TN + a) * 16 + 4 * group;
+    if (nrow >= n) continue;
+    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+    if (bias && split == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nrow + i < n) bv[i] = to_float(bf16_t{bias[nrow + i]});
+    }
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int row = 32 * wave_m + 16 * b + lane16;
+      if (row >= m) continue;
+      float* out = partial + ((size_t)split * m + row) * n + nrow;
+      const f32x4 v = acc[a][b] + bv;
+      if (nrow + 3 < n && (n & 3) == 0) {
+        *reinterpret_cast<f32x4*>(out) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nrow + i < n) out[i] = v[i];
+      }
+    }
+  }
+}
+
+template <int TN>
+int launch_tiled(float* partial, const uint16_t* x, long x_stride, const uint16_t* w, const uint16_t* bias, int m,
+                 int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+  constexpr int NT = 32 * TN;
+  constexpr size_t lds_bytes = (size_t)2 * (NT + M_TILE) * LDS_ROW * sizeof(uint16_t);
+  if (lds_bytes > 48 * 1024) {
+    static bool raised = false;  // per process; the attribute belongs to the kernel
+    if (!raised) {
+      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds_bytes) != hipSuccess)
+        return TS_ERR_LAUNCH;
+      raised = true;
+    }
+  }
+  dim3 grid((n + NT - 1) / NT, splits);
+  hipLaunchKernelGGL((gemm_tiled_kernel<TN>), grid, dim3(THREADS), lds_bytes, stream, partial, x, x_stride, w, bias,
+                     m, n, k, iters_per_split);
+  return ts_launch_status();
+}
+
+}  // namespace
+
+// partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
+// w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
+// iters_per_split iterations of 128 of k go to each of `splits` = ceil(ceil(k / 128) / iters_per_split).
+// tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows).
+extern "C" int ts_gemm_tiled(float* partial, const void* x, long x_stride, const void* w, const void* bias, int m,
+                             int n, int k, int iters_per_split, int splits, int tile, hipStream_t stream) {
+  if (m == 0 || n == 0) return TS_OK;
+  if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
+  if (m > M_TILE || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
+  const int total = (k + DEPTH - 1) / DEPTH;
+  if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split || splits > 65535)
+    return TS_ERR_SHAPE;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* bp = (const uint16_t*)bias;
+  if (tile == 2) return launch_tiled<2>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 4) return launch_tiled<4>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 5) return launch_tiled<5>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  return TS_ERR_SHAPE;
+}

@@ -10,8 +10,7 @@ Shapes are bucketed so that few graphs serve every batch: the number of requests
 to a power of two (the extra rows are padding: position 0, context 1, no cache write, results
 dropped) and each cache group's block-table width to a power of two.  The kernels read the
 true context lengths from the device, so one graph serves every length up to its width.  The
-graphs hold this engine's own kernels and, for batches above 16, the library products that a
-timed choice preferred after checking that they replay exactly (``kernels/product_choice.py``).
+graphs hold only this engine's own kernels (no library call, no memset node).
 
 The reference has no counterpart: it launches eager torch ops every step
 (src/turboserve/engine/runtime/worker.py:221-233).

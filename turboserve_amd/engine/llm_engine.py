@@ -8,7 +8,6 @@ tiny pool or a stand-in runner.
 
 from __future__ import annotations
 
-import contextlib
 import dataclasses
 import logging
 import time
@@ -117,8 +116,6 @@ class LLMEngine:
         self.sampler = sampler if sampler is not None else Sampler(model.runtime.ops)
         if config.tune_gemm_tokens and runner is None:
             self._tune_library_products()
-        if config.choose_products and runner is None:
-            self._choose_products()
         self._decoders: dict[str, StreamingDecoder] = {}
         self._seed = config.seed if config.seed is not None else time.time_ns() & 0xFFFFFFFF
         self._num_generated_tokens = 0
@@ -148,27 +145,6 @@ class LLMEngine:
         logger.info("library products timed for steps of %s tokens in %.1f s (%d choices kept in %s)",
                     list(self.config.tune_gemm_tokens), time.perf_counter() - started, tuning.num_results(),
                     tuning.results_file)
-
-    def _choose_products(self) -> None:
-        """For decode steps of 17 to 64 requests: time this engine's product kernel against the
-        library on every projection of the model and keep the faster per shape."""
-        if self.model.runtime.dtype != torch.bfloat16:
-            return
-        from turboserve_amd.kernels.product_choice import MEASURED_ROWS, choose_products
-
-        limit = min(self.config.scheduler.max_num_seqs, self.config.scheduler.max_num_batched_tokens)
-        rows = [m for m in MEASURED_ROWS if m // 2 < limit]
-        if not rows:
-            return
-        started = time.perf_counter()
-        with contextlib.ExitStack() as stack:
-            if self.config.tune_gemm_tokens:  # the library's candidates are timed at these sizes too
-                from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
-
-                stack.enter_context(LibraryGemmTuning(self.config.gemm_tuning_file))
-            timings = choose_products(self.model.runtime.ops, lambda m: self.runner.dry_run(m, want_all=True), rows)
-        logger.info("products of 17 to 64 rows: %d of %d shapes go to the library (%.2f s)",
-                    sum(t.library_chosen for t in timings), len(timings), time.perf_counter() - started)
 
     def _resolve_eos_token_ids(self) -> frozenset[int]:
         """The checkpoint's end-of-sequence ids (engine.py:223-237)."""

@@ -36,6 +36,7 @@ MODULES: dict[str, tuple[str, ...]] = {
         "attention_generic.hip",
         "gemm_plain.hip",
         "gemm_skinny.hip",
+        "gemm_tiled.hip",
         "sampling.hip",
     ),
 }

@@ -52,12 +52,10 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                        c_float, c_int, c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
-        "ts_gemm_skinny": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p],
+        "ts_gemm_tiled": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                          c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_void_p],
-        "ts_gemm_skinny_resident_gated": [c_void_p, c_void_p, c_long, c_int, c_long, c_void_p, c_int, c_int, c_int,
-                                          c_int, c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -146,11 +144,6 @@ class Ops:
         self.core = load_module("core")
         for module in modules:
             load_module(module)
-        #: (row bucket, N, K, biased, 32-bit result) -> True where the BLAS library, not the skinny
-        #: product, runs a bfloat16 projection of 17 to 64 rows (filled by a timed choice at start-up).
-        self.library_products: dict[tuple[int, int, int, bool, bool], bool] = {}
-        #: While a list: every such projection that runs is noted here as (key, weight, bias).
-        self.product_log: list | None = None
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -478,16 +471,12 @@ class Ops:
                "ts_gemm_plain")
         return y
 
-    #: Workgroups a skinny product aims for (four per compute unit of a 256-CU device).
-    skinny_target_blocks = int(os.environ.get("TS_SKINNY_TB", "1024"))
-    #: Most ranges of K a skinny product is split into (its consumer adds them up).
+    #: Most ranges of K the resident product is split into (its consumer adds them up).
     skinny_max_splits = int(os.environ.get("TS_SKINNY_MAXS", "8"))
-    #: Wavefronts (16 weight rows each) per workgroup of the skinny product: 4 or 8.
-    skinny_waves = int(os.environ.get("TS_SKINNY_WAVES", "4"))
-    #: Largest batch the skinny product serves; above it the BLAS library is used.
+    #: Largest batch the weight-streaming products serve; above it the BLAS library is used.
     skinny_max_rows = 64
-    #: Up to this many rows the skinny product keeps a split's activations resident in LDS.
-    skinny_resident_rows = int(os.environ.get("TS_SKINNY_RROWS", "16"))
+    #: Most rows the resident product takes (a split's activations stay in LDS).
+    skinny_resident_rows = 16
     #: Wavefronts (16 weight rows x one range of K each) the resident variant aims for: 16 per compute unit.
     skinny_resident_waves = int(os.environ.get("TS_SKINNY_RW", "4096"))
     #: Wavefronts per workgroup of the resident variant (4 or 8); 0 chooses by the grid's size.
@@ -511,82 +500,98 @@ class Ops:
         waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 1024) else 4)
         return per_split, splits, waves, self.skinny_stage_chunks[0 if m <= 8 else 1]
 
-    #: Up to this many rows a feed-forward hands the gate|up partial sums straight to the down
-    #: product, which applies SwiGLU while staging its activations (one kernel fewer per layer).
-    #: Every workgroup of that product redoes the activation for its range of K, which at 8 rows
-    #: already costs more than the kernel it saves (measured at the 7B shape).
-    swiglu_fuse_rows = int(os.environ.get("TS_FUSE_SWIGLU_ROWS", "4"))
+    #: Compute units the tiled product sizes its grid for.
+    tiled_compute_units = int(os.environ.get("TS_TILED_CUS", "256"))
+    #: Up to this many rows a product of a wide matrix (at least 200 tiles of 160 rows) stays with
+    #: the resident-activation kernel, which is a little faster there; everything else up to 64
+    #: rows runs the tiled kernel.
+    resident_wide_rows = int(os.environ.get("TS_RESIDENT_WIDE_ROWS", "4"))
+    #: Matrices smaller than this many bytes stay with the resident kernel up to 16 rows: the product
+    #: lasts a few microseconds and the resident kernel's many small workgroups start faster.
+    resident_small_bytes = int(os.environ.get("TS_RESIDENT_SMALL_BYTES", str(64 << 20)))
 
-    def swiglu_linear_possible(self, gate_up: torch.Tensor, weight: torch.Tensor) -> bool:
-        """Whether :meth:`swiglu_linear` takes these operands at all."""
-        return (gate_up.dim() == 3 and gate_up.dtype == torch.float32 and weight.dtype == torch.bfloat16
-                and gate_up.shape[1] <= self.skinny_resident_rows and gate_up.shape[2] == 2 * weight.shape[1]
-                and weight.shape[1] % 8 == 0 and gate_up.is_contiguous())
+    def _tiled_plan(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int]:
+        """(iterations of 128 per split, splits, tile) of the tiled product.  The cost of a
+        choice is what the busiest compute unit has to stream: workgroups it is handed (one at
+        a time for the larger tiles, whose LDS fills a compute unit; two for the smallest) x
+        rows of a tile x iterations, one more iteration per workgroup for starting up, with
+        small corrections fitted to measurements at the 7B sizes."""
+        iters = -(-k // 128)
+        limit = min(iters, max_splits or 32)
+        best = None
+        for tile in (5, 4, 2):
+            rows = 32 * tile
+            tiles = -(-n // rows)
+            for want in range(1, limit + 1):
+                per_split = -(-iters // want)
+                splits = -(-iters // per_split)
+                if splits != want:
+                    continue  # the same grid as a smaller `want`
+                groups = -(-tiles * splits // self.tiled_compute_units)
+                cost = groups * rows * (per_split + 1)
+                cost *= 1.0 + splits * m / k        # partial sums written here and read by the consumer
+                cost *= 1.0 + 0.12 * m / rows       # activations a workgroup stages, relative to its weights
+                if tile == 2:
+                    cost *= 0.95                    # two workgroups share a compute unit and fill each other's waits
+                resident = self.tiled_compute_units * (2 if tile == 2 else 1)
+                cost *= 1.0 + 0.1 * (-(-tiles * splits // resident) - 1)  # later rounds start on a busy device, unevenly
+                if best is None or cost < best[0] * 0.999:
+                    best = (cost, per_split, splits, tile)
+        return best[1], best[2], best[3]
 
-    def swiglu_linear_supported(self, gate_up: torch.Tensor, weight: torch.Tensor) -> bool:
-        """Whether a feed-forward should use :meth:`swiglu_linear` for these operands."""
-        return self.swiglu_linear_possible(gate_up, weight) and gate_up.shape[1] <= self.swiglu_fuse_rows
+    def gemm_tiled(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                   *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None) -> torch.Tensor:
+        """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
+        K (bias in the first) by the LDS-tiled kernel: M up to 64, K a multiple of 8.  ``plan``
+        overrides the grid (iterations per split, splits, tile) for measurements."""
+        _gpu(x, weight, bias)
+        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
+              and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
+        _need(self.skinny_supported(x, weight), "the tiled product takes bfloat16, M <= 64 and K % 8 == 0")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
+        per_split, splits, tile = plan or self._tiled_plan(m, n, k, max_splits)
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
+        _check(self.core.ts_gemm_tiled(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
+                                       per_split, splits, tile, self.stream()), "ts_gemm_tiled")
+        return partial
 
-    def swiglu_linear(self, gate_up: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-        """``[S', M, N]`` 32-bit partial sums of ``(silu(gate) * up) @ weight^T`` from the 32-bit
-        partial sums ``gate_up [S, M, 2 I]`` of a fused gate|up projection: what :meth:`swiglu`
-        followed by :meth:`gemm_skinny` gives, bit for bit, in one kernel."""
-        _gpu(gate_up, weight)
-        _need(self.swiglu_linear_possible(gate_up, weight) and weight.is_contiguous(),
-              "swiglu_linear takes contiguous 32-bit partial sums [S, M <= 16, 2 I] and a bfloat16 weight [N, I]")
-        gated_splits, m, width = gate_up.shape
-        n, k = weight.shape
-        per_split, splits, waves, stage = self._resident_plan(m, n, -(-k // 256), None)
-        partial = torch.empty((splits, m, n), dtype=torch.float32, device=gate_up.device)
-        _check(self.core.ts_gemm_skinny_resident_gated(_ptr(partial), _ptr(gate_up), width, gated_splits, m * width,
-                                                       _ptr(weight), m, n, k, per_split, splits, waves, stage,
-                                                       self.stream()), "ts_gemm_skinny_resident_gated")
+    def gemm_resident(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                      *, max_splits: int | None = None) -> torch.Tensor:
+        """The same partial sums by the kernel that keeps a split's activations resident in LDS and
+        streams the weights through registers: M up to 16."""
+        _gpu(x, weight, bias)
+        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
+              and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
+        _need(self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_resident_rows,
+              "the resident product takes bfloat16, M <= 16 and K % 8 == 0")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
+        x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
+        per_split, splits, waves, stage = self._resident_plan(m, n, -(-k // 256), max_splits)
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        _check(self.core.ts_gemm_skinny_resident(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias),
+                                                 m, n, k, per_split, splits, waves, stage, self.stream()),
+               "ts_gemm_skinny_resident")
         return partial
 
     def gemm_skinny(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                     *, max_splits: int | None = None) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
-        K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``."""
-        _gpu(x, weight, bias)
-        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
-              and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
-        _need(self.skinny_supported(x, weight), "the skinny product takes bfloat16, M <= 64 and K % 8 == 0")
-        m, k = x.shape
-        n = weight.shape[0]
-        if bias is not None:
-            _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
-        chunks = -(-k // 256)
-        x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
-        if m <= self.skinny_resident_rows:
-            per_split, splits, waves, stage = self._resident_plan(m, n, chunks, max_splits)
-            partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-            _check(self.core.ts_gemm_skinny_resident(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias),
-                                                     m, n, k, per_split, splits, waves, stage, self.stream()),
-                   "ts_gemm_skinny_resident")
-            return partial
-        waves = self.skinny_waves
-        row_blocks = -(-n // (16 * waves))
-        want = max(1, min(chunks, -(-self.skinny_target_blocks // row_blocks), max_splits or self.skinny_max_splits))
-        per_split = -(-chunks // want)
-        splits = -(-chunks // per_split)
-        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-        _check(self.core.ts_gemm_skinny(_ptr(partial), _ptr(x), x_stride,
-                                        _ptr(weight), _ptr(bias), m, n, k, per_split, splits, waves, self.stream()),
-               "ts_gemm_skinny")
-        return partial
-
-    def _skinny_runs(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, float32_out: bool) -> bool:
-        """Whether the skinny product, not the library, runs this bfloat16 projection: always up
-        to 16 rows, never above 64, in between unless a timed choice gave the shape to the library."""
-        m = x.shape[0]
-        if not self.skinny_supported(x, weight) or m > self.skinny_max_rows:
-            return False
-        if m <= self.skinny_resident_rows:
-            return True
-        key = (1 << (m - 1).bit_length(), weight.shape[0], weight.shape[1], bias is not None, float32_out)
-        if self.product_log is not None:
-            self.product_log.append((key, weight, bias))
-        return not self.library_products.get(key, False)
+        K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``: the
+        tiled kernel, except for a few rows against a wide matrix (the resident kernel is a
+        little faster there)."""
+        m, (n, k) = x.shape[0], weight.shape
+        if m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes:
+            return self.gemm_resident(x, weight, bias, max_splits=max_splits)
+        if m <= self.resident_wide_rows and -(-n // 160) >= 200:
+            return self.gemm_resident(x, weight, bias, max_splits=max_splits)
+        return self.gemm_tiled(x, weight, bias, max_splits=max_splits)
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
         """The projection of the serving path.  32-bit runs use :meth:`gemm_plain` (no reduced
@@ -597,7 +602,7 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight, bias)
         _gpu(x, weight, bias)
-        if self._skinny_runs(x, weight, bias, False):
+        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             return self.gemm_skinny(x, weight, bias)
         if bias is None:
             return torch.mm(x, weight.t())
@@ -609,7 +614,7 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight)
         _gpu(x, weight)
-        if self._skinny_runs(x, weight, None, True):
+        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             return self.gemm_skinny(x, weight, max_splits=1)[0]
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
 

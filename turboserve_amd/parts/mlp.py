@@ -38,6 +38,4 @@ class SwiGLU(FeedForward):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
         gate_up = ops.linear(x, self.gate_up_weight)
-        if ops.swiglu_linear_supported(gate_up, self.down_weight):
-            return ops.swiglu_linear(gate_up, self.down_weight)  # the activation is applied inside the product
         return ops.linear(ops.swiglu(gate_up, self.runtime.dtype), self.down_weight)

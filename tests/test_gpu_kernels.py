@@ -84,6 +84,14 @@ def test_embed_swiglu_gather(ops, dtype):
     zero_up = gu.clone()
     zero_up[:, 200:] = 0
     assert float(ops.swiglu(zero_up.to(DEV)).abs().max()) == 0.0
+    # the same values with gate and up alternating, for a width that takes the 4-wide kernel and one that does not
+    for inter in (200, 201):
+        gu = torch.randn(7, 2 * inter, generator=g).to(dtype)
+        want = torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]
+        pairs = torch.stack([gu[:, :inter], gu[:, inter:]], dim=2).reshape(7, 2 * inter).contiguous()
+        halves = ops.swiglu(gu.to(DEV)).cpu()
+        torch.testing.assert_close(halves.float(), want, **tol(dtype))
+        assert torch.equal(ops.swiglu(pairs.to(DEV), paired=True).cpu(), halves)
 
     rows = torch.tensor([6, 0, 3], dtype=torch.int32)
     torch.testing.assert_close(ops.gather_rows(gu.to(DEV), rows.to(DEV)).cpu(), gu[rows.long()], rtol=0, atol=0)
@@ -161,6 +169,34 @@ def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
         assert partial.shape == (splits, m, n)
         got = partial.double().sum(0).cpu()
         assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1), per_split
+
+
+@pytest.mark.parametrize("tile", [2, 4, 5])
+@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (33, 1000, 40)])
+def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
+    """A gate|up matrix with alternating rows through the tiled product with the activation in
+    its epilogue gives, bit for bit, what the product's partial sums followed by the SwiGLU
+    kernel give; and the plain value of silu(x Wg^T) * (x Wu^T).  `linear_swiglu` takes that
+    path when the product is one range of K, the two-kernel path otherwise, 32-bit included."""
+    g = torch.Generator().manual_seed(tile + inter)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    gate = (torch.randn(inter, k, generator=g) * 0.2).bfloat16()
+    up = (torch.randn(inter, k, generator=g) * 0.2).bfloat16()
+    w = torch.stack([gate, up], dim=1).reshape(2 * inter, k).contiguous()
+    plan = (-(-k // 128), 1, tile)
+    fused = ops.gemm_tiled(x.to(DEV), w.to(DEV), plan=plan, gated=True)
+    two_steps = ops.swiglu(ops.gemm_tiled(x.to(DEV), w.to(DEV), plan=plan), torch.bfloat16, paired=True)
+    assert fused.shape == (m, inter) and torch.equal(fused, two_steps)
+    want = torch.nn.functional.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    assert float((fused.double().cpu() - want).abs().max()) <= 1e-2 * float(want.abs().max() + 1)
+    either = ops.linear_swiglu(x.to(DEV), w.to(DEV))
+    assert float((either.double().cpu() - want).abs().max()) <= 1e-2 * float(want.abs().max() + 1)
+    exact = ops.linear_swiglu(x.float().to(DEV), w.float().to(DEV))
+    assert exact.dtype == torch.float32
+    assert float((exact.double().cpu() - want).abs().max()) <= 1e-5 * float(want.abs().max() + 1) * math.sqrt(k)
+    with pytest.raises(Exception, match="one range of K"):
+        ops.gemm_tiled(x.to(DEV), w.to(DEV), plan=(1, -(-k // 128), tile), gated=True) if k > 128 else ops.gemm_tiled(
+            x.to(DEV), w.to(DEV), torch.zeros(2 * inter).bfloat16().to(DEV), plan=plan, gated=True)
 
 
 def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):

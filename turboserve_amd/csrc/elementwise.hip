@@ -224,20 +224,24 @@ extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int
 }
 
 // ---------------------------------------------------------------------------------------------
-// SwiGLU over the fused gate|up projection: out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+// SwiGLU over the fused gate|up projection [T, 2 I]: out[t, i] = silu(gate[t, i]) * up[t, i], with
+// gate in the first I columns and up in the last (paired == 0), or alternating: gate i in column
+// 2 i, up i in column 2 i + 1 (paired != 0).
 // ---------------------------------------------------------------------------------------------
 // P: type of the projection output: T, or float for `splits` partial sums to be added up.
 template <typename T, typename P>
 __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
-                              size_t split_stride, int inter, size_t total) {
+                              size_t split_stride, int inter, size_t total, int paired) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t t = idx / inter;
   const int i = (int)(idx - t * inter);
+  const size_t gate_at = t * 2 * inter + (paired ? 2 * i : i);
+  const size_t up_at = paired ? gate_at + 1 : gate_at + inter;
   float g = 0.f, u = 0.f;
   for (int sp = 0; sp < splits; ++sp) {
-    g += to_float(gate_up[sp * split_stride + t * 2 * inter + i]);
-    u += to_float(gate_up[sp * split_stride + t * 2 * inter + inter + i]);
+    g += to_float(gate_up[sp * split_stride + gate_at]);
+    u += to_float(gate_up[sp * split_stride + up_at]);
   }
   const float act = g / (1.f + expf(-g));
   out[idx] = from_float<T>(act * u);
@@ -246,7 +250,7 @@ __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up
 // Four outputs per thread with 8- or 16-byte loads: for I a multiple of 4.
 template <typename T, typename P>
 __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
-                                   size_t split_stride, int inter, size_t quads) {
+                                   size_t split_stride, int inter, size_t quads, int paired) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= quads) return;
   const int per_row = inter / 4;
@@ -255,6 +259,13 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
   float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
   for (int sp = 0; sp < splits; ++sp) {
     float a[4], b[4];
+    if (paired) {  // eight consecutive columns: g0 u0 g1 u1 | g2 u2 g3 u3
+      Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + 2 * i, a);
+      Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + 2 * i + 4, b);
+      g[0] += a[0]; u[0] += a[1]; g[1] += a[2]; u[1] += a[3];
+      g[2] += b[0]; u[2] += b[1]; g[3] += b[2]; u[3] += b[3];
+      continue;
+    }
     Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + i, a);
     Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + inter + i, b);
 #pragma unroll
@@ -271,28 +282,28 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
 
 template <typename T, typename P>
 static void launch_swiglu(void* out, const void* gate_up, int splits, long split_stride, int tokens, int inter,
-                          hipStream_t stream) {
+                          int paired, hipStream_t stream) {
   if (inter % 4 == 0) {
     const size_t quads = (size_t)tokens * (inter / 4);
     hipLaunchKernelGGL((swiglu_vec4_kernel<T, P>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
-                       (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads);
+                       (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads, paired);
   } else {
     const size_t total = (size_t)tokens * inter;
     hipLaunchKernelGGL((swiglu_kernel<T, P>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (T*)out,
-                       (const P*)gate_up, splits, (size_t)split_stride, inter, total);
+                       (const P*)gate_up, splits, (size_t)split_stride, inter, total, paired);
   }
 }
 
 extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits, long split_stride,
-                         int tokens, int inter, int dtype, hipStream_t stream) {
+                         int tokens, int inter, int paired, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !gate_up || inter < 1 || splits < 1) return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, stream);
+    launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
   else if (dtype == TS_BF16 && in_f32)
-    launch_swiglu<bf16_t, float>(out, gate_up, splits, split_stride, tokens, inter, stream);
+    launch_swiglu<bf16_t, float>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
   else if (dtype == TS_BF16)
-    launch_swiglu<bf16_t, bf16_t>(out, gate_up, splits, split_stride, tokens, inter, stream);
+    launch_swiglu<bf16_t, bf16_t>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -46,9 +46,9 @@ struct TileRegs {
 
 template <int TN>
 __global__ void __launch_bounds__(THREADS)
-gemm_tiled_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
-                  const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
-                  int iters_per_split) {
+gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, const uint16_t* __restrict__ x,
+                  long x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n,
+                  int k, int iters_per_split) {
   constexpr int NT = 32 * TN;
   constexpr int STAGE = (NT + M_TILE) * LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
   typedef TileRegs<TN> Regs;
@@ -162,6 +162,22 @@ gemm_tiled_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, l
     for (int b = 0; b < 2; ++b) {
       const int row = 32 * wave_m + 16 * b + lane16;
       if (row >= m) continue;
+      if (gated) {
+        // The matrix is a gate|up projection with rows alternating gate, up (one range of K, no
+        // bias): the lane holds two such pairs and writes silu(gate) * up for both, rounded once,
+        // by the formula of the stand-alone SwiGLU kernel.
+        const f32x4 s = acc[a][b];
+        const float lo = s[0] / (1.f + expf(-s[0])) * s[1];
+        const float hi = s[2] / (1.f + expf(-s[2])) * s[3];
+        uint16_t* out = gated + (size_t)row * (n / 2) + nrow / 2;
+        if (nrow + 3 < n) {
+          *reinterpret_cast<uint32_t*>(out) =
+              (uint32_t)from_float<bf16_t>(lo).bits | ((uint32_t)from_float<bf16_t>(hi).bits << 16);
+        } else if (nrow + 1 < n) {
+          out[0] = from_float<bf16_t>(lo).bits;
+        }
+        continue;
+      }
       float* out = partial + ((size_t)split * m + row) * n + nrow;
       const f32x4 v = acc[a][b] + bv;
       if (nrow + 3 < n && (n & 3) == 0) {
@@ -176,8 +192,8 @@ gemm_tiled_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, l
 }
 
 template <int TN>
-int launch_tiled(float* partial, const uint16_t* x, long x_stride, const uint16_t* w, const uint16_t* bias, int m,
-                 int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
+                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
   constexpr int NT = 32 * TN;
   constexpr size_t lds_bytes = (size_t)2 * (NT + M_TILE) * LDS_ROW * sizeof(uint16_t);
   if (lds_bytes > 48 * 1024) {
@@ -190,8 +206,8 @@ int launch_tiled(float* partial, const uint16_t* x, long x_stride, const uint16_
     }
   }
   dim3 grid((n + NT - 1) / NT, splits);
-  hipLaunchKernelGGL((gemm_tiled_kernel<TN>), grid, dim3(THREADS), lds_bytes, stream, partial, x, x_stride, w, bias,
-                     m, n, k, iters_per_split);
+  hipLaunchKernelGGL((gemm_tiled_kernel<TN>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride, w,
+                     bias, m, n, k, iters_per_split);
   return ts_launch_status();
 }
 
@@ -201,19 +217,24 @@ int launch_tiled(float* partial, const uint16_t* x, long x_stride, const uint16_
 // w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
 // iters_per_split iterations of 128 of k go to each of `splits` = ceil(ceil(k / 128) / iters_per_split).
 // tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows).
-extern "C" int ts_gemm_tiled(float* partial, const void* x, long x_stride, const void* w, const void* bias, int m,
-                             int n, int k, int iters_per_split, int splits, int tile, hipStream_t stream) {
+// gated (bfloat16 [m, n / 2], contiguous) instead of partial: w is a gate|up projection whose rows
+// alternate gate, up, and the kernel writes silu(gate) * up; needs splits == 1, no bias, n even.
+extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_stride, const void* w,
+                             const void* bias, int m, int n, int k, int iters_per_split, int splits, int tile,
+                             hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
-  if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
+  if (!x || !w || m < 0 || n < 0 || k < 8 || (partial == nullptr) == (gated == nullptr)) return TS_ERR_ARG;
   if (m > M_TILE || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
   const int total = (k + DEPTH - 1) / DEPTH;
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split || splits > 65535)
     return TS_ERR_SHAPE;
+  if (gated && (splits != 1 || bias || (n & 1) != 0)) return TS_ERR_ARG;
+  uint16_t* gp = (uint16_t*)gated;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (tile == 2) return launch_tiled<2>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
-  if (tile == 4) return launch_tiled<4>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
-  if (tile == 5) return launch_tiled<5>(partial, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 2) return launch_tiled<2>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 4) return launch_tiled<4>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 5) return launch_tiled<5>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
   return TS_ERR_SHAPE;
 }

@@ -43,7 +43,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
         "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
                            c_int, c_int, c_int, c_void_p],
-        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p],
+        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p],
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -52,8 +52,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                        c_float, c_int, c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
-        "ts_gemm_tiled": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                          c_void_p],
+        "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                          c_int, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -220,9 +220,11 @@ class Ops:
                                         self.stream()), "ts_add_rmsnorm")
         return y
 
-    def swiglu(self, gate_up: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+    def swiglu(self, gate_up: torch.Tensor, dtype: torch.dtype | None = None, *, paired: bool = False) -> torch.Tensor:
         """``silu(gate) * up`` of the fused ``[T, 2 I]`` projection (or its ``[S, T, 2 I]`` 32-bit
-        partial sums) -> ``[T, I]`` of ``dtype`` (the projection's own if it is not partial)."""
+        partial sums) -> ``[T, I]`` of ``dtype`` (the projection's own if it is not partial).
+        Gate fills the first ``I`` columns and up the last, or, with ``paired``, they alternate
+        (gate ``i`` in column ``2 i``, up ``i`` in column ``2 i + 1``)."""
         _gpu(gate_up)
         tokens, width = gate_up.shape[-2], gate_up.shape[-1]
         _need(width % 2 == 0, "gate_up must be [T, 2 I]")
@@ -233,7 +235,7 @@ class Ops:
         inter = width // 2
         out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
         _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
-                                   dtype_code(out_dtype), self.stream()), "ts_swiglu")
+                                   1 if paired else 0, dtype_code(out_dtype), self.stream()), "ts_swiglu")
         return out
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
@@ -540,10 +542,13 @@ class Ops:
         return best[1], best[2], best[3]
 
     def gemm_tiled(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-                   *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None) -> torch.Tensor:
+                   *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None,
+                   gated: bool = False) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
         K (bias in the first) by the LDS-tiled kernel: M up to 64, K a multiple of 8.  ``plan``
-        overrides the grid (iterations per split, splits, tile) for measurements."""
+        overrides the grid (iterations per split, splits, tile) for measurements.  ``gated``:
+        the weight is a gate|up projection whose rows alternate gate, up, and the result is
+        ``silu(gate) * up`` as bfloat16 ``[M, N / 2]`` (one range of K only)."""
         _gpu(x, weight, bias)
         _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
               and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
@@ -553,9 +558,16 @@ class Ops:
         if bias is not None:
             _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
         per_split, splits, tile = plan or self._tiled_plan(m, n, k, max_splits)
-        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
-        _check(self.core.ts_gemm_tiled(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
+        if gated:
+            _need(splits == 1 and bias is None and n % 2 == 0,
+                  "the gated result needs one range of K, no bias and an even number of weight rows")
+            out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+            _check(self.core.ts_gemm_tiled(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k,
+                                           per_split, splits, tile, self.stream()), "ts_gemm_tiled")
+            return out
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        _check(self.core.ts_gemm_tiled(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
                                        per_split, splits, tile, self.stream()), "ts_gemm_tiled")
         return partial
 
@@ -586,12 +598,29 @@ class Ops:
         K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``: the
         tiled kernel, except for a few rows against a wide matrix (the resident kernel is a
         little faster there)."""
-        m, (n, k) = x.shape[0], weight.shape
-        if m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes:
-            return self.gemm_resident(x, weight, bias, max_splits=max_splits)
-        if m <= self.resident_wide_rows and -(-n // 160) >= 200:
+        if self._resident_runs(x.shape[0], weight.shape[0], weight.shape[1]):
             return self.gemm_resident(x, weight, bias, max_splits=max_splits)
         return self.gemm_tiled(x, weight, bias, max_splits=max_splits)
+
+    def _resident_runs(self, m: int, n: int, k: int) -> bool:
+        """Whether the resident kernel, not the tiled one, runs a decode-sized product: small
+        matrices up to 16 rows, the widest ones up to four."""
+        if m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes:
+            return True
+        return m <= self.resident_wide_rows and -(-n // 160) >= 200
+
+    def linear_swiglu(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """``silu(gate) * up`` of the projection of ``x`` by a gate|up matrix ``[2 I, K]`` whose rows
+        alternate gate, up -> ``[T, I]`` in the dtype of ``x``.  Decode-sized bfloat16 batches whose
+        product runs as one range of K get the activation in the product's own kernel; every other
+        case is the projection followed by :meth:`swiglu`."""
+        if (x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows
+                and not self._resident_runs(x.shape[0], weight.shape[0], weight.shape[1])):
+            _gpu(x, weight)
+            plan = self._tiled_plan(x.shape[0], weight.shape[0], weight.shape[1], None)
+            if plan[1] == 1 and weight.shape[0] % 2 == 0 and weight.is_contiguous() and x.stride(1) == 1:
+                return self.gemm_tiled(x, weight, plan=plan, gated=True)
+        return self.swiglu(self.linear(x, weight), x.dtype, paired=True)
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
         """The projection of the serving path.  32-bit runs use :meth:`gemm_plain` (no reduced

@@ -13,7 +13,9 @@ from turboserve_amd.parts.registry import register_feed_forward
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     """``down(silu(gate(x)) * up(x))`` (layers.py:437-440).  Gate and up are held as one
-    ``[2 I, H]`` matrix (concatenated at load), so a step does one product for both."""
+    ``[2 I, H]`` matrix whose rows alternate gate, up (interleaved at load; the checkpoint keeps
+    them apart): a step does one product for both, and the product's kernel has each gate
+    value next to its up value, so it can apply the activation itself."""
 
     def __init__(self, prefix: str, runtime: Runtime, *, hidden_size: int, intermediate_size: int) -> None:
         super().__init__(prefix, runtime)
@@ -30,12 +32,10 @@ class SwiGLU(FeedForward):
         }
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.gate_up_weight = torch.cat(
-            [tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]], dim=0
-        ).contiguous()
+        gate, up = tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]
+        self.gate_up_weight = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         self.down_weight = tensors[self.name("down_proj.weight")].contiguous()
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
-        gate_up = ops.linear(x, self.gate_up_weight)
-        return ops.linear(ops.swiglu(gate_up, self.runtime.dtype), self.down_weight)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up_weight), self.down_weight)

@@ -531,7 +531,7 @@ class Ops:
                     continue  # the same grid as a smaller `want`
                 groups = -(-tiles * splits // self.tiled_compute_units)
                 cost = groups * rows * (per_split + 1)
-                cost *= 1.0 + splits * m / k        # partial sums written here and read by the consumer
+                cost *= 1.0 + 2.0 * splits * m / k  # partial sums written here and read by the consumer
                 cost *= 1.0 + 0.12 * m / rows       # activations a workgroup stages, relative to its weights
                 if tile == 2:
                     cost *= 0.95                    # two workgroups share a compute unit and fill each other's waits
@@ -614,8 +614,7 @@ class Ops:
         alternate gate, up -> ``[T, I]`` in the dtype of ``x``.  Decode-sized bfloat16 batches whose
         product runs as one range of K get the activation in the product's own kernel; every other
         case is the projection followed by :meth:`swiglu`."""
-        if (x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows
-                and not self._resident_runs(x.shape[0], weight.shape[0], weight.shape[1])):
+        if x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             _gpu(x, weight)
             plan = self._tiled_plan(x.shape[0], weight.shape[0], weight.shape[1], None)
             if plan[1] == 1 and weight.shape[0] % 2 == 0 and weight.is_contiguous() and x.stride(1) == 1:

@@ -30,8 +30,13 @@ def model(request, tmp_path_factory):
     raw, tensors = tiny.read_model_dir(folder)
     lengths = [5, 17, 33] if request.param == "A" else [1, 9, 24, 40]
     prompts = [tiny.random_tokens(config["vocab_size"], n, 50 + n) for n in lengths]
+    # The same architecture with a wider spread of weights, for the 32-bit token-for-token tests:
+    # its greedy continuations do not settle on one token, so every step's logits matter.
+    wide = tiny.make_model_dir(tmp_path_factory.mktemp(f"engine{request.param}_wide"), config, seed + 1, torch.float32,
+                               std=tiny.WIDE_STD)
+    wide_raw, wide_tensors = tiny.read_model_dir(wide)
     return {"name": request.param, "folder": folder, "page": page, "raw": raw, "tensors": tensors, "prompts": prompts,
-            "vocab": config["vocab_size"]}
+            "vocab": config["vocab_size"], "wide_folder": wide, "wide_raw": wide_raw, "wide_tensors": wide_tensors}
 
 
 def test_greedy_generation_equals_plain(model):
@@ -40,9 +45,10 @@ def test_greedy_generation_equals_plain(model):
     from turboserve_amd.sampling.params import SamplingParams
 
     new = 8 if model["name"] == "A" else 12
-    want = [plain.greedy_generate(model["raw"], model["tensors"], p, new) for p in model["prompts"]]
+    want = [plain.greedy_generate(model["wide_raw"], model["wide_tensors"], p, new) for p in model["prompts"]]
+    assert all(len(set(tokens)) > 2 for tokens in want), "the continuations should not repeat one token"
     for budget, blocks in ((2048, 64), (16, 64), (7 if model["page"] <= 7 else model["page"], 64)):
-        with make_engine(model["folder"], "float32", model["page"], num_blocks=blocks, budget=budget) as engine:
+        with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=blocks, budget=budget) as engine:
             outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
             assert [o.new_token_ids for o in outputs] == want, f"budget {budget}"
             assert all(o.finish_reason == "length" and o.output_tokens == new for o in outputs)
@@ -56,10 +62,10 @@ def test_preemption_keeps_the_tokens(model):
     from turboserve_amd.sampling.params import SamplingParams
 
     new = 20
-    want = [plain.greedy_generate(model["raw"], model["tensors"], p, new) for p in model["prompts"]]
+    want = [plain.greedy_generate(model["wide_raw"], model["wide_tensors"], p, new) for p in model["prompts"]]
     longest = max(len(p) for p in model["prompts"]) + new
     blocks = -(-longest // model["page"])  # the longest request just fits alone; together they do not
-    with make_engine(model["folder"], "float32", model["page"], num_blocks=blocks, budget=64) as engine:
+    with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=blocks, budget=64) as engine:
         outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
         assert [o.new_token_ids for o in outputs] == want
         assert engine.stats()["num_preemptions"] > 0

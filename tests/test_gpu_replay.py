@@ -42,7 +42,8 @@ def case(request, tmp_path_factory):
     config, seed, page = tiny.TINY[name]
     folders = {}
     for dtype_name, dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
-        folders[dtype_name] = tiny.make_model_dir(tmp_path_factory.mktemp(f"tiny{name}_{dtype_name}"), config, seed, dtype)
+        folders[dtype_name] = tiny.make_model_dir(tmp_path_factory.mktemp(f"tiny{name}_{dtype_name}"), config, seed, dtype,
+                                                  std=tiny.WIDE_STD if dtype == torch.float32 else 0.02)
     requests = {f"r{i}": tiny.random_tokens(config["vocab_size"], n, 100 + i) for i, n in enumerate(lengths_for(name))}
     expected = {d: {rid: tiny.plain_logits(folders[d], toks) for rid, toks in requests.items()} for d in folders}
     return {"name": name, "page": page, "folders": folders, "requests": requests, "expected": expected}

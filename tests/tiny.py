@@ -76,10 +76,17 @@ PAGE_C = 32
 TINY = {"A": (CONFIG_A, 0, PAGE_A), "B": (CONFIG_B, 1, PAGE_B), "C": (CONFIG_C, 2, PAGE_C)}
 
 
-def make_model_dir(folder: Path, config: dict, seed: int, dtype: torch.dtype = torch.float32) -> Path:
+#: A wider spread of the weights for 32-bit comparisons.  With the usual 0.02 a model this small
+#: hardly mixes its inputs (greedy generation repeats one token, attention weights are near
+#: uniform); with 0.15 every layer matters to the next token, so a fault in any of them shows.
+#: bfloat16 runs keep 0.02: their rounding error grows with the spread, the bounds do not.
+WIDE_STD = 0.15
+
+
+def make_model_dir(folder: Path, config: dict, seed: int, dtype: torch.dtype = torch.float32, std: float = 0.02) -> Path:
     from turboserve_amd.weights.random_init import write_random_model
 
-    return write_random_model(config, folder, seed=seed, dtype=dtype)
+    return write_random_model(config, folder, seed=seed, dtype=dtype, std=std)
 
 
 def read_model_dir(folder: Path) -> tuple[dict, dict[str, torch.Tensor]]:

@@ -179,26 +179,34 @@ def test_decode_graphs_replay_like_eager(model):
             assert torch.equal(eager, graph), f"{dtype}: a graph replay differs from the eager step"
 
 
-def test_timed_library_products_and_the_dry_step(model, tmp_path):
-    """An engine asked to time the BLAS library's kernels at start-up: the dry step it runs for
-    that leaves every cache page as it was, the choices are written to the given file, and a
-    prompt longer than the skinny product's 64 rows (so that the library computes its
-    projections) still gives the plain implementation's log-probabilities."""
+def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
+    """An engine asked to time the BLAS library's kernels at start-up: the choices are written
+    to the given file, nothing is timed once the engine serves, products below the size worth
+    timing keep the library's default kernel, and the dry step the timing runs in leaves every
+    cache page as it was.  A prompt longer than the 128 rows the engine's own products take (so
+    that the library computes its projections) gives the plain implementation's
+    log-probabilities."""
     from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
     from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.kernels.ops import Ops
     from turboserve_amd.sampling.params import SamplingParams
 
-    results = tmp_path / "choices.csv"
-    prompt = tiny.random_tokens(model["vocab"], 100, 77)
-    engine = LLMEngine(EngineConfig(
-        model=str(model["folder"]), dtype="bfloat16", tune_gemm_tokens=(100,), gemm_tuning_file=str(results),
-        scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=128, block_size=model["page"], num_blocks=32),
-    ))
+    prompt = tiny.random_tokens(model["vocab"], 200, 77)
+
+    def engine_with_tuning(results):
+        return LLMEngine(EngineConfig(
+            model=str(model["folder"]), dtype="bfloat16", tune_gemm_tokens=(200,), gemm_tuning_file=str(results),
+            scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=256, block_size=model["page"], num_blocks=64),
+        ))
+
+    # This model's products are all below the size worth timing: nothing is chosen, nothing written.
+    untouched = tmp_path / "none.csv"
+    engine = engine_with_tuning(untouched)
     try:
-        assert results.exists() and "Gemm" in results.read_text()
-        assert not torch.cuda.tunable.tuning_is_enabled()  # nothing is timed once the engine serves
+        assert torch.cuda.tunable.is_enabled() and not torch.cuda.tunable.tuning_is_enabled()
+        assert not untouched.exists() or "Gemm" not in untouched.read_text()
         before = [t.clone() for t in engine.storage.pages]
-        engine.runner.dry_run(70)
+        engine.runner.dry_run(150)
         assert all(torch.equal(a, b) for a, b in zip(before, engine.storage.pages))
         out = engine.generate([prompt], SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True, logprobs=True))[0]
     finally:
@@ -209,21 +217,32 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
     for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
         want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
         assert abs(got - want) <= 0.05, (i, got, want)
+    # With the size limit lifted the same start-up times them and keeps its choices.
+    monkeypatch.setattr(Ops, "library_tuning_min_work", 0)
+    results = tmp_path / "choices.csv"
+    engine = engine_with_tuning(results)
+    try:
+        assert results.exists() and "Gemm" in results.read_text()
+        assert not torch.cuda.tunable.tuning_is_enabled()
+    finally:
+        engine.close()
+        torch.cuda.tunable.enable(False)
 
 
-def test_many_requests_decode_together(model):
-    """40 requests decoding in one batch (recorded steps of 64 rows, the tiled product at its
-    largest size) give the plain implementation's log-probabilities."""
+@pytest.mark.parametrize("count", [40, 100])
+def test_many_requests_decode_together(model, count):
+    """40 and 100 requests decoding in one batch (recorded steps of 64 and 128 rows, the tiled
+    product at both of its heights) give the plain implementation's log-probabilities."""
     from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
     from turboserve_amd.engine.llm_engine import LLMEngine
     from turboserve_amd.sampling.params import SamplingParams
 
-    prompts = [tiny.random_tokens(model["vocab"], 3 + i % 9, 300 + i) for i in range(40)]
+    prompts = [tiny.random_tokens(model["vocab"], 3 + i % 9, 300 + i) for i in range(count)]
     sampling = SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True, logprobs=True)
     weights = plain.as_float32(model["tensors"])
     engine = LLMEngine(EngineConfig(
         model=str(model["folder"]), dtype="bfloat16",
-        scheduler=SchedulerConfig(max_num_seqs=64, max_num_batched_tokens=2048, block_size=model["page"], num_blocks=256),
+        scheduler=SchedulerConfig(max_num_seqs=128, max_num_batched_tokens=2048, block_size=model["page"], num_blocks=512),
     ))
     try:
         outs = engine.generate(prompts, sampling)

@@ -124,7 +124,7 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops):
     assert torch.equal(full[40:41], one)
 
 
-@pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64, 65, 100, 128])
 @pytest.mark.parametrize("n,k", [(7, 8), (130, 104), (320, 96), (3584, 1000), (301, 2056), (4608, 3584), (33000, 136)])
 def test_gemm_skinny(ops, m, n, k):
     """The decode-sized product: 32-bit partial sums over ranges of K whose sum is the product,
@@ -153,7 +153,7 @@ def test_gemm_skinny(ops, m, n, k):
 
 
 @pytest.mark.parametrize("tile", [2, 4, 5])
-@pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (40, 64, 40)])
+@pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (40, 64, 40), (128, 330, 520), (77, 1000, 264)])
 def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
     """The tiled product with its grid given by hand: every tile size, ranges of K of one
     iteration and of several, a last range that is shorter, a last tile of rows that is partly
@@ -172,7 +172,7 @@ def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
 
 
 @pytest.mark.parametrize("tile", [2, 4, 5])
-@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (33, 1000, 40)])
+@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (33, 1000, 40), (128, 250, 264), (90, 81, 128)])
 def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
     """A gate|up matrix with alternating rows through the tiled product with the activation in
     its epilogue gives, bit for bit, what the product's partial sums followed by the SwiGLU

@@ -1,13 +1,14 @@
 // Weight-streaming product for decode-sized batches, tiled through LDS:
 //   partial[s][m][n] = sum over the k-range of split s of  X[m][k] * W[n][k]   (+ bias[n] in split 0)
-// for M <= 64 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
+// for M <= 128 rows of bfloat16 activations, bfloat16 weights [N, K] as the checkpoint stores
 // them (F.linear's layout, src/turboserve/engine/model/layers.py:142), 32-bit accumulation on
 // the matrix cores and 32-bit partial sums out; the consumer adds the splits up.
 //
 // The product is bound by reading W once from HBM, and what decides its rate is how the reading
 // is spread over the device, not how much of it is in flight:
 //   * a workgroup of four wavefronts (2 x 2) owns a tile of NT = 32 TN weight rows (TN = 2, 4
-//     or 5) by all 64 activation rows and one range of K; the host sizes tiles and ranges so that
+//     or 5) by all activation rows (64 of them, or 128 when M > 64) and one range of K; the host
+//     sizes tiles and ranges so that
 //     the grid is about one workgroup per compute unit (two for the smallest tile): every
 //     compute unit then streams one contiguous block of each of its rows, start to end;
 //   * the range is walked 128 deep: both operands travel global memory -> registers (16-byte
@@ -17,9 +18,9 @@
 //   * every load is issued on every path (rows beyond N or M repeat the last row, iterations
 //     beyond the range repeat its last one), so the compiler can count the loads in flight and
 //     waits only for those it needs; pieces beyond K are cleared on their way into LDS;
-//   * a wavefront computes TN x 2 tiles of v_mfma_f32_16x16x32_bf16 (A = 16 weight rows, B = 16
-//     activation rows): each weight fragment it reads from LDS serves two products, each
-//     activation fragment TN.
+//   * a wavefront computes TN x MB tiles of v_mfma_f32_16x16x32_bf16 (A = 16 weight rows, B = 16
+//     activation rows; MB = 2, or 4 for M > 64): each weight fragment it reads from LDS serves MB
+//     products, each activation fragment TN.
 #include "common.hpp"
 
 namespace {
@@ -30,28 +31,29 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int DEPTH = 128;            // k per iteration
 constexpr int LDS_ROW = DEPTH + 8;    // LDS row stride in elements
-constexpr int M_TILE = 64;            // activation rows a workgroup covers (rows beyond M are repeats)
+constexpr int M_MAX = 128;            // most activation rows (a workgroup covers 32 MB: rows beyond M are repeats)
 constexpr int THREADS = 256;
 constexpr int ROW_PIECES = DEPTH / 8; // 16-byte pieces of a row of an iteration
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <int TN>
+template <int TN, int MB>
 struct TileRegs {
   static constexpr int W_PIECES = 32 * TN * ROW_PIECES / THREADS;  // 2 TN
-  static constexpr int X_PIECES = M_TILE * ROW_PIECES / THREADS;   // 4
+  static constexpr int X_PIECES = 32 * MB * ROW_PIECES / THREADS;  // 2 MB
   u32x4 w[W_PIECES];
   u32x4 x[X_PIECES];
 };
 
-template <int TN>
+template <int TN, int MB>
 __global__ void __launch_bounds__(THREADS)
 gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, const uint16_t* __restrict__ x,
                   long x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n,
                   int k, int iters_per_split) {
   constexpr int NT = 32 * TN;
+  constexpr int M_TILE = 32 * MB;
   constexpr int STAGE = (NT + M_TILE) * LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
-  typedef TileRegs<TN> Regs;
+  typedef TileRegs<TN, MB> Regs;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [2][STAGE]
   const int tid = threadIdx.x;
   const int lane = tid & (TS_WAVE - 1);
@@ -109,22 +111,25 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
     }
   };
 
-  f32x4 acc[TN][2];
+  f32x4 acc[TN][MB];
 #pragma unroll
-  for (int a = 0; a < TN; ++a) acc[a][0] = acc[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int a = 0; a < TN; ++a) {
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
   auto multiply = [&](int buf) {
     const uint16_t* base = lds + buf * STAGE + lane16 * LDS_ROW + 8 * group;
 #pragma unroll
     for (int step = 0; step < DEPTH / 32; ++step) {
-      u32x4 xf[2];
+      u32x4 xf[MB];
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
-        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 32 * wave_m + 16 * b) * LDS_ROW + 32 * step);
+      for (int b = 0; b < MB; ++b)
+        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 16 * MB * wave_m + 16 * b) * LDS_ROW + 32 * step);
 #pragma unroll
       for (int a = 0; a < TN; ++a) {
         const u32x4 wf = *reinterpret_cast<const u32x4*>(base + (wave_n * TN + a) * 16 * LDS_ROW + 32 * step);
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < MB; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wf), as_bf16x8(xf[b]), acc[a][b], 0, 0, 0);
       }
     }
@@ -147,7 +152,7 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
   }
 
   // acc[a][b][i] = sum for weight row n_base + 16 (wave_n TN + a) + 4 g + i and activation row
-  // 32 wave_m + 16 b + lane16.
+  // 16 MB wave_m + 16 b + lane16.
 #pragma unroll
   for (int a = 0; a < TN; ++a) {
     const int nrow = n_base + (wave_n * TN + a) * 16 + 4 * group;
@@ -159,8 +164,8 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
         if (nrow + i < n) bv[i] = to_float(bf16_t{bias[nrow + i]});
     }
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const int row = 32 * wave_m + 16 * b + lane16;
+    for (int b = 0; b < MB; ++b) {
+      const int row = 16 * MB * wave_m + 16 * b + lane16;
       if (row >= m) continue;
       if (gated) {
         // The matrix is a gate|up projection with rows alternating gate, up (one range of K, no
@@ -191,30 +196,40 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
   }
 }
 
-template <int TN>
-int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
-                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+template <int TN, int MB>
+int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
+                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits,
+                      hipStream_t stream) {
   constexpr int NT = 32 * TN;
-  constexpr size_t lds_bytes = (size_t)2 * (NT + M_TILE) * LDS_ROW * sizeof(uint16_t);
+  constexpr size_t lds_bytes = (size_t)2 * (NT + 32 * MB) * LDS_ROW * sizeof(uint16_t);
+  static_assert(lds_bytes <= 160 * 1024, "two buffers must fit the LDS of a compute unit");
   if (lds_bytes > 48 * 1024) {
     static bool raised = false;  // per process; the attribute belongs to the kernel
     if (!raised) {
-      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN, MB>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)lds_bytes) != hipSuccess)
         return TS_ERR_LAUNCH;
       raised = true;
     }
   }
   dim3 grid((n + NT - 1) / NT, splits);
-  hipLaunchKernelGGL((gemm_tiled_kernel<TN>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride, w,
-                     bias, m, n, k, iters_per_split);
+  hipLaunchKernelGGL((gemm_tiled_kernel<TN, MB>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride,
+                     w, bias, m, n, k, iters_per_split);
   return ts_launch_status();
+}
+
+template <int TN>
+int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
+                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+  if (m <= 64)
+    return launch_tiled_rows<TN, 2>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+  return launch_tiled_rows<TN, 4>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
 }
 
 }  // namespace
 
 // partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
-// w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 64, k % 8 == 0.
+// w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 128, k % 8 == 0.
 // iters_per_split iterations of 128 of k go to each of `splits` = ceil(ceil(k / 128) / iters_per_split).
 // tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows).
 // gated (bfloat16 [m, n / 2], contiguous) instead of partial: w is a gate|up projection whose rows
@@ -224,7 +239,7 @@ extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_
                              hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || (partial == nullptr) == (gated == nullptr)) return TS_ERR_ARG;
-  if (m > M_TILE || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
+  if (m > M_MAX || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
   const int total = (k + DEPTH - 1) / DEPTH;
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split || splits > 65535)
     return TS_ERR_SHAPE;

@@ -48,7 +48,7 @@ class _Graph:
 
 class DecodeGraphs:
     def __init__(self, model, views, *, page_size: int, num_groups: int, pad_state_slot: int,
-                 max_batch: int = 64) -> None:
+                 max_batch: int = 128) -> None:
         self.model = model
         self.views = views
         self.page_size = page_size

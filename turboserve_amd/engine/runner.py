@@ -23,7 +23,7 @@ from turboserve_amd.models.decoder import DecoderModel
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, storage: CacheStorage, *, check: bool = True,
-                 use_graphs: bool = True, max_graph_batch: int = 64) -> None:
+                 use_graphs: bool = True, max_graph_batch: int = 128) -> None:
         self.model = model
         self.storage = storage
         self.layout: CacheLayout = storage.layout

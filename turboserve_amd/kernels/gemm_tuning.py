@@ -11,7 +11,10 @@ module drives it:
 * ``with LibraryGemmTuning(path):`` times every product shape that runs inside the block; the
   winners are kept in memory and appended to ``path`` (read again by the next process);
 * after the block the winners stay in use, and shapes that were not timed fall back to the
-  library's heuristic at no cost (no timing outside the block, so no surprise stalls).
+  library's heuristic at no cost (no timing outside the block, so no surprise stalls);
+* a candidate has to reproduce the default kernel's result (within bfloat16 rounding) to be
+  eligible, and products too small to be worth timing never leave the default kernel
+  (``Ops.library_tuning_min_work``).
 
 An engine runs the block over one dry step of its usual prefill size at start-up when asked to
 (``EngineConfig.tune_gemm_tokens``).  The choice changes which library kernel computes a product,
@@ -67,11 +70,15 @@ class LibraryGemmTuning:
                 pass  # a file of another library version: its entries are ignored and replaced
         tunable.set_max_tuning_duration(self.max_ms_per_candidate)
         tunable.set_max_tuning_iterations(self.max_iterations)
+        # A candidate is only eligible if its result agrees with the library's default kernel up
+        # to bfloat16 rounding: the fastest kernel for a shape is of no use if it is a broken one.
+        tunable.set_numerical_check_tolerances(True, 2e-2, 2e-2)
         tunable.tuning_enable(True)
         return self
 
     def __exit__(self, *exc) -> None:
         torch.cuda.tunable.tuning_enable(False)
+        torch.cuda.tunable.set_numerical_check_tolerances(False)
 
     @staticmethod
     def num_results() -> int:

@@ -476,7 +476,7 @@ class Ops:
     #: Most ranges of K the resident product is split into (its consumer adds them up).
     skinny_max_splits = int(os.environ.get("TS_SKINNY_MAXS", "8"))
     #: Largest batch the weight-streaming products serve; above it the BLAS library is used.
-    skinny_max_rows = 64
+    skinny_max_rows = 128
     #: Most rows the resident product takes (a split's activations stay in LDS).
     skinny_resident_rows = 16
     #: Wavefronts (16 weight rows x one range of K each) the resident variant aims for: 16 per compute unit.
@@ -488,8 +488,8 @@ class Ops:
 
     @staticmethod
     def skinny_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-        """bfloat16, at most 64 rows, K a multiple of 8."""
-        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= 64
+        """bfloat16, at most 128 rows, K a multiple of 8."""
+        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= 128
                 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0)
 
     def _resident_plan(self, m: int, n: int, chunks: int, max_splits: int | None) -> tuple[int, int, int, int]:
@@ -545,14 +545,14 @@ class Ops:
                    *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None,
                    gated: bool = False) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
-        K (bias in the first) by the LDS-tiled kernel: M up to 64, K a multiple of 8.  ``plan``
+        K (bias in the first) by the LDS-tiled kernel: M up to 128, K a multiple of 8.  ``plan``
         overrides the grid (iterations per split, splits, tile) for measurements.  ``gated``:
         the weight is a gate|up projection whose rows alternate gate, up, and the result is
         ``silu(gate) * up`` as bfloat16 ``[M, N / 2]`` (one range of K only)."""
         _gpu(x, weight, bias)
         _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
               and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
-        _need(self.skinny_supported(x, weight), "the tiled product takes bfloat16, M <= 64 and K % 8 == 0")
+        _need(self.skinny_supported(x, weight), "the tiled product takes bfloat16, M <= 128 and K % 8 == 0")
         m, k = x.shape
         n = weight.shape[0]
         if bias is not None:
@@ -609,6 +609,29 @@ class Ops:
             return True
         return m <= self.resident_wide_rows and -(-n // 160) >= 200
 
+    #: Products with fewer multiply-adds than this never use a timed choice of the BLAS library's
+    #: kernels, only its default: timing them is noise, and one of the library's candidates for
+    #: such a shape ([200, 64] x [256, 64]) returned garbage once in about eight processes.
+    library_tuning_min_work = 1 << 24
+
+    def _library_product(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
+                         out_dtype: torch.dtype | None) -> torch.Tensor:
+        """``x @ weight^T (+ bias)`` by the BLAS library behind torch."""
+        tunable = torch.cuda.tunable
+        small = x.shape[0] * weight.shape[0] * weight.shape[1] < self.library_tuning_min_work
+        paused = small and tunable.is_enabled()
+        if paused:
+            tunable.enable(False)
+        try:
+            if out_dtype is not None:
+                return torch.mm(x, weight.t(), out_dtype=out_dtype)
+            if bias is None:
+                return torch.mm(x, weight.t())
+            return torch.addmm(bias, x, weight.t())
+        finally:
+            if paused:
+                tunable.enable(True)
+
     def linear_swiglu(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """``silu(gate) * up`` of the projection of ``x`` by a gate|up matrix ``[2 I, K]`` whose rows
         alternate gate, up -> ``[T, I]`` in the dtype of ``x``.  Decode-sized bfloat16 batches whose
@@ -632,9 +655,7 @@ class Ops:
         _gpu(x, weight, bias)
         if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             return self.gemm_skinny(x, weight, bias)
-        if bias is None:
-            return torch.mm(x, weight.t())
-        return torch.addmm(bias, x, weight.t())
+        return self._library_product(x, weight, bias, None)
 
     def linear_float32_out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """``x @ weight^T`` with a 32-bit result (the head: logits are 32-bit,
@@ -644,7 +665,7 @@ class Ops:
         _gpu(x, weight)
         if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             return self.gemm_skinny(x, weight, max_splits=1)[0]
-        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+        return self._library_product(x, weight, None, torch.float32)
 
     # -- sampling -----------------------------------------------------------------------------
 

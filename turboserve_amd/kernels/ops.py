@@ -144,6 +144,7 @@ class Ops:
         self.core = load_module("core")
         for module in modules:
             load_module(module)
+        self._tiled_plans: dict[tuple, tuple[int, int, int]] = {}  # (m, n, k, max_splits) -> grid of the tiled product
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -505,7 +506,7 @@ class Ops:
     #: Compute units the tiled product sizes its grid for.
     tiled_compute_units = int(os.environ.get("TS_TILED_CUS", "256"))
     #: Up to this many rows a product of a wide matrix (at least 200 tiles of 160 rows) stays with
-    #: the resident-activation kernel, which is a little faster there; everything else up to 64
+    #: the resident-activation kernel, which is a little faster there; everything else up to 128
     #: rows runs the tiled kernel.
     resident_wide_rows = int(os.environ.get("TS_RESIDENT_WIDE_ROWS", "4"))
     #: Matrices smaller than this many bytes stay with the resident kernel up to 16 rows: the product
@@ -518,6 +519,10 @@ class Ops:
         a time for the larger tiles, whose LDS fills a compute unit; two for the smallest) x
         rows of a tile x iterations, one more iteration per workgroup for starting up, with
         small corrections fitted to measurements at the 7B sizes."""
+        key = (m, n, k, max_splits)
+        known = self._tiled_plans.get(key)
+        if known is not None:
+            return known
         iters = -(-k // 128)
         limit = min(iters, max_splits or 32)
         best = None
@@ -539,7 +544,8 @@ class Ops:
                 cost *= 1.0 + 0.1 * (-(-tiles * splits // resident) - 1)  # later rounds start on a busy device, unevenly
                 if best is None or cost < best[0] * 0.999:
                     best = (cost, per_split, splits, tile)
-        return best[1], best[2], best[3]
+        self._tiled_plans[key] = (best[1], best[2], best[3])
+        return self._tiled_plans[key]
 
     def gemm_tiled(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                    *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None,

@@ -459,8 +459,21 @@ decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ parti
   const int d4 = 4 * (tid % LANES_PER_GROUP);
   if (g < GROUPS) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = g; sp < splits; sp += GROUPS)
-      acc += *reinterpret_cast<const f32x4*>(partial_acc + (base + sp) * D + d4) * weights[sp];
+    // Four splits' loads are issued together and added in split order: one trip to memory
+    // for every four splits of a group instead of one per split.
+    for (int sp0 = g; sp0 < splits; sp0 += 4 * GROUPS) {
+      f32x4 part[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int sp = sp0 + j * GROUPS;
+        part[j] = *reinterpret_cast<const f32x4*>(partial_acc + (base + (sp < splits ? sp : sp0)) * D + d4);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int sp = sp0 + j * GROUPS;
+        if (sp < splits) acc += part[j] * weights[sp];
+      }
+    }
     *reinterpret_cast<f32x4*>(&sums[g][d4]) = acc;
   }
   __syncthreads();

@@ -64,6 +64,25 @@ __global__ void rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x, const
   }
 }
 
+// `init` plus the `splits` values that lie `stride` elements apart, added in split order; the loads
+// of up to eight splits are in flight together (see add_splits4).
+template <typename P>
+__device__ __forceinline__ float add_splits(const P* p, int splits, size_t stride, float init) {
+  float s = init;
+  if (splits == 1) return s + to_float(p[0]);
+  int sp0 = 0;
+  do {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = to_float(p[(size_t)min(sp0 + j, splits - 1) * stride]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (sp0 + j < splits) s += v[j];
+    sp0 += 8;
+  } while (sp0 < splits);
+  return s;
+}
+
 // P is the type of `pending`: T, or float for `splits` partial sums of a product that are
 // `split_stride` elements apart and are added up here.
 template <typename T, typename P>
@@ -79,7 +98,7 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residu
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
     if (pending) {
-      for (int sp = 0; sp < splits; ++sp) s += to_float(pending[sp * split_stride + in_base + i]);
+      s = add_splits(pending + in_base + i, splits, split_stride, s);
       if (!rows) residual[in_base + i] = s;  // re-read below by this same thread
     }
     ss += s * s;
@@ -88,8 +107,7 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residu
   const float rstd = rsqrtf(ss / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
-    if (rows && pending)
-      for (int sp = 0; sp < splits; ++sp) s += to_float(pending[sp * split_stride + in_base + i]);
+    if (rows && pending) s = add_splits(pending + in_base + i, splits, split_stride, s);
     const float n = round_to<T>(s * rstd);
     y[out_base + i] = from_float<T>(to_float(w[i]) * n);
   }
@@ -140,6 +158,37 @@ struct Vec4Of<bf16_t> {
   }
 };
 
+// Partial sums of a product lie `stride` elements apart.  The loads of up to SPLIT_BATCH splits
+// are issued together and only then added, in split order: a loop that loads and adds one split
+// at a time makes every split wait a full trip to memory, and these kernels are nothing but
+// such trips.  A value that is not split (splits == 1) takes the one load.
+constexpr int SPLIT_BATCH = 8;
+
+template <typename P>
+__device__ __forceinline__ void add_splits4(const P* p, int splits, size_t stride, float (&s)[4]) {
+  if (splits == 1) {
+    float v[4];
+    Vec4Of<P>::load(p, v);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] += v[e];
+    return;
+  }
+  int sp0 = 0;
+  do {  // the first batch is issued before anything waits for `s` (the caller's own load)
+    float v[SPLIT_BATCH][4];
+#pragma unroll
+    for (int j = 0; j < SPLIT_BATCH; ++j) Vec4Of<P>::load(p + (size_t)min(sp0 + j, splits - 1) * stride, v[j]);
+#pragma unroll
+    for (int j = 0; j < SPLIT_BATCH; ++j) {
+      if (sp0 + j < splits) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] += v[j][e];
+      }
+    }
+    sp0 += SPLIT_BATCH;
+  } while (sp0 < splits);
+}
+
 #define NORM_ITEMS 4
 
 template <typename T, typename P>
@@ -160,12 +209,7 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
     if (qd < quads) {
       Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
       if (pending) {
-        for (int sp = 0; sp < splits; ++sp) {
-          float v[4];
-          Vec4Of<P>::load(pending + sp * split_stride + in_base + 4 * qd, v);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) s[it][e] += v[e];
-        }
+        add_splits4(pending + in_base + 4 * qd, splits, split_stride, s[it]);
         if (!rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
       }
 #pragma unroll
@@ -238,11 +282,8 @@ __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up
   const int i = (int)(idx - t * inter);
   const size_t gate_at = t * 2 * inter + (paired ? 2 * i : i);
   const size_t up_at = paired ? gate_at + 1 : gate_at + inter;
-  float g = 0.f, u = 0.f;
-  for (int sp = 0; sp < splits; ++sp) {
-    g += to_float(gate_up[sp * split_stride + gate_at]);
-    u += to_float(gate_up[sp * split_stride + up_at]);
-  }
+  const float g = add_splits(gate_up + gate_at, splits, split_stride, 0.f);
+  const float u = add_splits(gate_up + up_at, splits, split_stride, 0.f);
   const float act = g / (1.f + expf(-g));
   out[idx] = from_float<T>(act * u);
 }
@@ -256,22 +297,20 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
   const int per_row = inter / 4;
   const size_t t = idx / per_row;
   const int i = (int)(idx - t * per_row) * 4;
-  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int sp = 0; sp < splits; ++sp) {
-    float a[4], b[4];
-    if (paired) {  // eight consecutive columns: g0 u0 g1 u1 | g2 u2 g3 u3
-      Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + 2 * i, a);
-      Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + 2 * i + 4, b);
-      g[0] += a[0]; u[0] += a[1]; g[1] += a[2]; u[1] += a[3];
-      g[2] += b[0]; u[2] += b[1]; g[3] += b[2]; u[3] += b[3];
-      continue;
-    }
-    Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + i, a);
-    Vec4Of<P>::load(gate_up + sp * split_stride + t * 2 * inter + inter + i, b);
+  float g[4], u[4];
+  float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+  if (paired) {  // eight consecutive columns: g0 u0 g1 u1 | g2 u2 g3 u3
+    add_splits4(gate_up + t * 2 * inter + 2 * i, splits, split_stride, a);
+    add_splits4(gate_up + t * 2 * inter + 2 * i + 4, splits, split_stride, b);
+    g[0] = a[0]; u[0] = a[1]; g[1] = a[2]; u[1] = a[3];
+    g[2] = b[0]; u[2] = b[1]; g[3] = b[2]; u[3] = b[3];
+  } else {
+    add_splits4(gate_up + t * 2 * inter + i, splits, split_stride, a);
+    add_splits4(gate_up + t * 2 * inter + inter + i, splits, split_stride, b);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      g[e] += a[e];
-      u[e] += b[e];
+      g[e] = a[e];
+      u[e] = b[e];
     }
   }
   float o[4];
@@ -357,11 +396,8 @@ __global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int sp
     const float* c = cos_table + (size_t)pos * half;
     const float* s = sin_table + (size_t)pos * half;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      float x1 = 0.f, x2 = 0.f;
-      for (int sp = 0; sp < splits; ++sp) {
-        x1 += to_float(row[sp * split_stride + i]);
-        x2 += to_float(row[sp * split_stride + i + half]);
-      }
+      float x1 = add_splits(row + i, splits, split_stride, 0.f);
+      float x2 = add_splits(row + i + half, splits, split_stride, 0.f);
       float r1 = x1, r2 = x2;
       if (rotate) rotate_pair(x1, x2, c[i], s[i], r1, r2);
       const T o1 = from_float<T>(r1);
@@ -377,8 +413,7 @@ __global__ void rope_store_kernel(T* q_out, long q_stride, const P* proj, int sp
     }
   } else if (vpage) {
     for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-      float x = 0.f;
-      for (int sp = 0; sp < splits; ++sp) x += to_float(row[sp * split_stride + i]);
+      const float x = add_splits(row + i, splits, split_stride, 0.f);
       vpage[(size_t)i * block_size] = from_float<T>(x);
     }
   }

@@ -436,6 +436,19 @@ decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ parti
   const int tid = threadIdx.x;
   const int wave = tid / TS_WAVE;
   const size_t base = ((size_t)blockIdx.x * heads + head) * splits;
+  const int token = query_start_loc[seq];  // the row of the result; fetched with everything else
+
+  // The first four splits of this thread's group are fetched before anything else: their loads
+  // travel while the weights of the splits are worked out, instead of after two barriers.
+  const int g = tid / LANES_PER_GROUP;
+  const int d4 = 4 * (tid % LANES_PER_GROUP);
+  const bool sums_here = g < GROUPS;
+  f32x4 part[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int sp = g + j * GROUPS;
+    part[j] = *reinterpret_cast<const f32x4*>(partial_acc + (base + ((sums_here && sp < splits) ? sp : 0)) * D + d4);
+  }
 
   const bool owns = tid < splits;
   const float m = owns ? partial_ml[(base + tid) * 2] : -INFINITY;
@@ -455,14 +468,15 @@ decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ parti
 #pragma unroll
   for (int i = 0; i < REDUCE_THREADS / TS_WAVE; ++i) den += wave_part[1][i];
 
-  const int g = tid / LANES_PER_GROUP;
-  const int d4 = 4 * (tid % LANES_PER_GROUP);
-  if (g < GROUPS) {
+  if (sums_here) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    // Four splits' loads are issued together and added in split order: one trip to memory
-    // for every four splits of a group instead of one per split.
-    for (int sp0 = g; sp0 < splits; sp0 += 4 * GROUPS) {
-      f32x4 part[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int sp = g + j * GROUPS;
+      if (sp < splits) acc += part[j] * weights[sp];
+    }
+    // Further splits, four loads at a time, added in split order.
+    for (int sp0 = g + 4 * GROUPS; sp0 < splits; sp0 += 4 * GROUPS) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int sp = sp0 + j * GROUPS;
@@ -481,7 +495,6 @@ decode_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ parti
     float num = 0.f;
 #pragma unroll
     for (int i = 0; i < GROUPS; ++i) num += sums[i][tid];
-    const int token = query_start_loc[seq];
     out[((size_t)token * heads + head) * D + tid] = (uint16_t)bf16_bits(num / den);
   }
 }

@@ -158,35 +158,39 @@ struct Vec4Of<bf16_t> {
   }
 };
 
-// Partial sums of a product lie `stride` elements apart.  The loads of up to SPLIT_BATCH splits
-// are issued together and only then added, in split order: a loop that loads and adds one split
-// at a time makes every split wait a full trip to memory, and these kernels are nothing but
-// such trips.  A value that is not split (splits == 1) takes the one load.
-constexpr int SPLIT_BATCH = 8;
+// Partial sums of a product lie `stride` elements apart.  The loads of a batch of splits are
+// issued together and only then added, in split order: a loop that loads and adds one split at a
+// time makes every split wait a full trip to memory, and these kernels are nothing but such
+// trips.  Up to 16 splits are one batch in straight-line code (so that the caller's own loads,
+// issued before, are waited for only where they are used); more go in batches of 8.  A value
+// that is not split (splits == 1) takes the one load.
+template <int N, typename P>
+__device__ __forceinline__ void add_split_batch4(const P* p, int first, int splits, size_t stride, float (&s)[4]) {
+  float v[N][4];
+#pragma unroll
+  for (int j = 0; j < N; ++j) Vec4Of<P>::load(p + (size_t)min(first + j, splits - 1) * stride, v[j]);
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    if (first + j < splits) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += v[j][e];
+    }
+  }
+}
 
 template <typename P>
 __device__ __forceinline__ void add_splits4(const P* p, int splits, size_t stride, float (&s)[4]) {
   if (splits == 1) {
-    float v[4];
-    Vec4Of<P>::load(p, v);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) s[e] += v[e];
-    return;
+    add_split_batch4<1>(p, 0, 1, stride, s);
+  } else if (splits <= 4) {
+    add_split_batch4<4>(p, 0, splits, stride, s);
+  } else if (splits <= 8) {
+    add_split_batch4<8>(p, 0, splits, stride, s);
+  } else if (splits <= 16) {
+    add_split_batch4<16>(p, 0, splits, stride, s);
+  } else {
+    for (int first = 0; first < splits; first += 8) add_split_batch4<8>(p, first, splits, stride, s);
   }
-  int sp0 = 0;
-  do {  // the first batch is issued before anything waits for `s` (the caller's own load)
-    float v[SPLIT_BATCH][4];
-#pragma unroll
-    for (int j = 0; j < SPLIT_BATCH; ++j) Vec4Of<P>::load(p + (size_t)min(sp0 + j, splits - 1) * stride, v[j]);
-#pragma unroll
-    for (int j = 0; j < SPLIT_BATCH; ++j) {
-      if (sp0 + j < splits) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s[e] += v[j][e];
-      }
-    }
-    sp0 += SPLIT_BATCH;
-  } while (sp0 < splits);
 }
 
 #define NORM_ITEMS 4
@@ -201,13 +205,14 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
   const size_t in_base = (size_t)src * hidden;
   const size_t out_base = (size_t)blockIdx.x * hidden;
   const int quads = hidden / 4;
-  float s[NORM_ITEMS][4];
+  float s[NORM_ITEMS][4], g[NORM_ITEMS][4];
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < NORM_ITEMS; ++it) {
     const int qd = threadIdx.x + it * blockDim.x;
     if (qd < quads) {
       Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
+      Vec4Of<T>::load(w + 4 * qd, g[it]);  // with the other loads, not behind the reduction's barriers
       if (pending) {
         add_splits4(pending + in_base + 4 * qd, splits, split_stride, s[it]);
         if (!rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
@@ -222,10 +227,9 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
   for (int it = 0; it < NORM_ITEMS; ++it) {
     const int qd = threadIdx.x + it * blockDim.x;
     if (qd < quads) {
-      float g[4], o[4];
-      Vec4Of<T>::load(w + 4 * qd, g);
+      float o[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = g[e] * round_to<T>(s[it][e] * rstd);
+      for (int e = 0; e < 4; ++e) o[e] = g[it][e] * round_to<T>(s[it][e] * rstd);
       Vec4Of<T>::store(y + out_base + 4 * qd, o);
     }
   }

@@ -220,28 +220,39 @@ def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):
     torch.testing.assert_close(full.sum(0), other.sum(0), rtol=1e-5, atol=1e-3)
 
 
-def test_consumers_add_up_partial_sums(ops):
+@pytest.mark.parametrize("splits", [2, 3, 5, 8, 9, 16, 17, 29])
+@pytest.mark.parametrize("hidden", [200, 201])
+def test_consumers_add_up_partial_sums(ops, splits, hidden):
     """Norm, SwiGLU and rotary/cache write take the skinny product's 32-bit partial sums and
-    give what they give for the summed tensor."""
+    give what they give for the summed tensor.  The kernels fetch the splits in batches (of 4,
+    8, 16, and 8 at a time beyond that) and add them in split order: the residual they leave is,
+    bit for bit, the residual plus the splits added one after the other.  Widths that are and
+    are not a multiple of 4 take the kernels with and without 16-byte accesses."""
     from turboserve_amd.parts.rope import rotary_tables
 
-    g = torch.Generator().manual_seed(8)
-    tokens, hidden, splits = 6, 200, 3
+    g = torch.Generator().manual_seed(8 + splits)
+    tokens = 6
     parts = torch.randn(splits, tokens, hidden, generator=g)
     total = parts.sum(0)
     w = (1 + 0.1 * torch.randn(hidden, generator=g)).bfloat16()
     residual = torch.randn(tokens, hidden, generator=g)
     res_dev = residual.to(DEV)
     got = ops.add_rmsnorm(res_dev, parts.to(DEV), w.to(DEV), 1e-6).float().cpu()
-    torch.testing.assert_close(res_dev.cpu(), residual + total, rtol=0, atol=1e-5)
+    in_order = residual.clone()
+    for part in parts:
+        in_order += part
+    assert torch.equal(res_dev.cpu(), in_order)
     torch.testing.assert_close(got, plain.rms_norm(residual + total, w.float(), 1e-6), **tol(torch.bfloat16))
     rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
     got = ops.add_rmsnorm(residual.to(DEV), parts.to(DEV), w.to(DEV), 1e-6, rows).float().cpu()
     torch.testing.assert_close(got, plain.rms_norm(residual + total, w.float(), 1e-6)[[4, 1]], **tol(torch.bfloat16))
 
-    gu = torch.randn(splits, tokens, 2 * 72, generator=g)
-    want = torch.nn.functional.silu(gu.sum(0)[:, :72]) * gu.sum(0)[:, 72:]
+    inter = 72 if hidden % 4 == 0 else 73
+    gu = torch.randn(splits, tokens, 2 * inter, generator=g)
+    want = torch.nn.functional.silu(gu.sum(0)[:, :inter]) * gu.sum(0)[:, inter:]
     torch.testing.assert_close(ops.swiglu(gu.to(DEV), torch.bfloat16).float().cpu(), want, **tol(torch.bfloat16))
+    want = torch.nn.functional.silu(gu.sum(0)[:, 0::2]) * gu.sum(0)[:, 1::2]
+    torch.testing.assert_close(ops.swiglu(gu.to(DEV), torch.bfloat16, paired=True).float().cpu(), want, **tol(torch.bfloat16))
 
     heads, kv_heads, dim, page = 3, 1, 32, 8
     proj = torch.randn(splits, tokens, (heads + 2 * kv_heads) * dim, generator=g)

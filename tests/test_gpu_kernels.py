@@ -539,6 +539,51 @@ def test_attention_prefill_mfma_far_key(ops):
     assert float(case.expected[:40].abs().mean()) > 4.0
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [(14, 2, 128, 16), (3, 1, 32, 8)])
+@pytest.mark.parametrize("window", [40, 64, 97])
+def test_attention_at_the_windows_edge(ops, heads, kv_heads, dim, page, window):
+    """One key that would carry the result lies just outside the window of a single-token
+    request's query, then just inside; and inside the window of some rows of a prompt portion
+    and outside that of others.  A kernel that is one key off at either edge returns that key's
+    value (5.0) where the plain attention does not, or the other way round."""
+    ctx = 300
+    for spike, carried in ((ctx - 1 - window, False), (ctx - window, True), (ctx - 1, True)):
+        case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, [(ctx, 1)], window, seed=spike, spike=spike)
+        assert (float(case.expected.abs().mean()) > 4.0) == carried
+        out = torch.zeros(1, heads * dim, dtype=torch.bfloat16, device=DEV)
+        ops.attention_decode(
+            out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+            case.ints(case.qsl), case.ints([ctx]), 0, 1, heads, dim ** -0.5, window, ctx,
+        )
+        torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+        for dtype in (torch.float32, torch.bfloat16):
+            exact = PagedCase(dtype, heads, kv_heads, dim, page, [(ctx, 1)], window, seed=spike, spike=spike)
+            got = ops.paged_attention_generic(
+                exact.dev(exact.q), heads * dim, exact.dev(exact.kp), exact.dev(exact.vp), exact.dev(exact.table),
+                exact.ints(exact.token_seq), exact.ints(exact.positions), heads, dim ** -0.5, window,
+            ).float().cpu()
+            torch.testing.assert_close(got, exact.expected, **tol(dtype))
+    # a portion of 70 rows (positions 230..299): the key at 250 is seen by rows 250 .. 249 + window
+    # only, so some rows of one 16-row block see it and others do not, at both edges
+    qlen, spike = 70, 250
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, [(ctx, qlen)], window, seed=7, spike=spike)
+    rows = case.expected.view(qlen, -1).abs().mean(1) > 4.0
+    positions = torch.arange(ctx - qlen, ctx)
+    assert torch.equal(rows, (positions >= spike) & (positions <= spike + window - 1))
+    blocks = [(0, off) for off in range(0, qlen, 16)]
+    out = torch.zeros(qlen, heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints([ctx]), case.ints(blocks), heads, dim ** -0.5, window, ctx,
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+    got = ops.paged_attention_generic(
+        case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.token_seq), case.ints(case.positions), heads, dim ** -0.5, window,
+    ).float().cpu()
+    torch.testing.assert_close(got, case.expected, **tol(torch.bfloat16))
+
+
 # -- sampling ---------------------------------------------------------------------------------------
 
 

@@ -12,12 +12,12 @@ from plain import qwen2_plain as plain
 pytestmark = pytest.mark.gpu
 
 
-def make_engine(folder, dtype, page, *, num_blocks, budget=2048, max_num_seqs=8, seed=None):
+def make_engine(folder, dtype, page, *, num_blocks, budget=2048, max_num_seqs=8, seed=None, run_ahead=False):
     from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
     from turboserve_amd.engine.llm_engine import LLMEngine
 
     return LLMEngine(EngineConfig(
-        model=str(folder), dtype=dtype, seed=seed,
+        model=str(folder), dtype=dtype, seed=seed, run_ahead=run_ahead,
         scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget, block_size=page,
                                   num_blocks=num_blocks),
     ))
@@ -255,6 +255,47 @@ def test_many_requests_decode_together(model, count):
         for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
             want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
             assert abs(got - want) <= 0.05, (i, got, want)
+
+
+def test_steps_launched_ahead_give_the_same_tokens(model):
+    """With `run_ahead` every decode step is launched before the tokens of the step before it
+    have been read (they are copied on the device into the recorded step's input): greedy in
+    32-bit gives the plain implementation's tokens, with plenty of pages and with so few that
+    requests are preempted; seeded temperature sampling gives the tokens it gives without
+    running ahead; a stop token ends its request at the same place."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 20
+    prompts = model["prompts"]
+    want = [plain.greedy_generate(model["wide_raw"], model["wide_tensors"], p, new) for p in prompts]
+    longest = max(len(p) for p in prompts) + new
+    few = -(-longest // model["page"])  # the longest request just fits alone; together they do not
+    for blocks in (64, few):
+        with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=blocks, budget=64,
+                         run_ahead=True) as engine:
+            outputs = engine.generate(prompts, SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+            assert [o.new_token_ids for o in outputs] == want, f"{blocks} pages"
+            assert engine.runner.graphs.num_replays > 0
+            engine.scheduler.check_invariants()
+            assert all(pool.num_in_use == 0 for pool in engine.scheduler.cache.pools)
+            if blocks == few:
+                assert engine.stats()["num_preemptions"] > 0
+    stop = want[0][5]
+    expected = want[0][: want[0].index(stop) + 1]
+    with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=64, run_ahead=True) as engine:
+        outputs = engine.generate(prompts, [SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True,
+                                                           stop_token_ids=(stop,) if i == 0 else ())
+                                            for i in range(len(prompts))])
+        assert outputs[0].new_token_ids == expected and outputs[0].finish_reason == "stop"
+        assert [o.new_token_ids for o in outputs[1:]] == want[1:]
+    sampling = [SamplingParams(max_tokens=new, temperature=0.8, top_p=0.9, seed=7 + i, ignore_eos=True, logprobs=True)
+                for i in range(len(prompts))]
+    results = []
+    for ahead in (False, True):
+        with make_engine(model["folder"], "bfloat16", model["page"], num_blocks=64, run_ahead=ahead) as engine:
+            outputs = engine.generate(prompts, sampling)
+            results.append([(o.new_token_ids, o.logprobs) for o in outputs])
+    assert results[0] == results[1]
 
 
 def test_command_line_generates_the_plain_tokens(tmp_path):

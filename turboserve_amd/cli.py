@@ -38,6 +38,8 @@ def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> Non
     p.set_defaults(prefix_caching=False)
     p.add_argument("--tune-gemm", action="store_true",
                    help="time the BLAS library's kernels for a full step of prompt tokens at start-up and keep the fastest")
+    p.add_argument("--run-ahead", action="store_true",
+                   help="launch each decode step before the host has read the tokens of the step before it")
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -93,6 +95,7 @@ def _generate(args: argparse.Namespace) -> int:
     config = EngineConfig(
         model=args.model, device=args.device, dtype=args.dtype, seed=args.seed,
         tune_gemm_tokens=(args.max_num_batched_tokens,) if args.tune_gemm else (),
+        run_ahead=getattr(args, "run_ahead", False),
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
             block_size=args.block_size, num_blocks=args.num_blocks, enable_prefix_caching=args.prefix_caching,

@@ -68,6 +68,11 @@ class EngineConfig:
     tune_gemm_tokens: tuple[int, ...] = ()
     #: Where the timed choices are kept between runs; None is a per-user cache file.
     gemm_tuning_file: str | None = None
+    #: Launch a decode step before the host has read the tokens of the step before it (they
+    #: are copied on the device), so that the GPU does not wait while the host schedules and
+    #: builds outputs.  Results are the same tokens; a request that ends on a stop token costs
+    #: one token's worth of work that is thrown away.  No counterpart in the reference.
+    run_ahead: bool = False
 
     def __post_init__(self) -> None:
         if self.speculative is not None or self.lora is not None:
@@ -89,7 +94,7 @@ class EngineConfig:
         """An engine configuration from the process-wide ``TURBOSERVE_*`` variables the
         reference's settings read (src/turboserve/config.py:38-64, types.py:575-593): MODEL,
         DTYPE, DEVICE, GPU_MEMORY_UTILIZATION, MAX_NUM_SEQS, MAX_NUM_BATCHED_TOKENS, BLOCK_SIZE,
-        NUM_BLOCKS, ENABLE_CHUNKED_PREFILL.  Unset variables keep this class's defaults;
+        NUM_BLOCKS, ENABLE_CHUNKED_PREFILL, and this engine's own RUN_AHEAD.  Unset variables keep this class's defaults;
         ``overrides`` win over the environment."""
         env = os.environ if environ is None else environ
 
@@ -116,6 +121,7 @@ class EngineConfig:
             "dtype": get("DTYPE", str),
             "device": get("DEVICE", str),
             "gpu_memory_utilization": get("GPU_MEMORY_UTILIZATION", float),
+            "run_ahead": get("RUN_AHEAD", truth),
         }.items() if v is not None}
         fields["scheduler"] = SchedulerConfig(**scheduler)
         fields.update(overrides)

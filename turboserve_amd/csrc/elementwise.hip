@@ -564,3 +564,26 @@ extern "C" int ts_gather_rows(void* out, const void* x, const int* rows, int n, 
     return TS_ERR_DTYPE;
   return ts_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// patch_tokens: token_ids[i] = source[patch[i]] where patch[i] >= 0 (else left as it is).  A step
+// that is launched before the host has read the tokens the step before sampled takes them from
+// the sampler's device buffer this way.  patch[i] must be below `sources`; a value at or beyond
+// it is ignored (nothing is read out of bounds).
+// ---------------------------------------------------------------------------------------------
+__global__ void patch_tokens_kernel(int* __restrict__ token_ids, const int* __restrict__ patch,
+                                    const int* __restrict__ source, int n, int sources) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int from = patch[i];
+  if (from >= 0 && from < sources) token_ids[i] = source[from];
+}
+
+extern "C" int ts_patch_tokens(int* token_ids, const int* patch, const int* source, int n, int sources,
+                               hipStream_t stream) {
+  if (n == 0) return TS_OK;
+  if (!token_ids || !patch || !source || n < 0 || sources < 1) return TS_ERR_ARG;
+  hipLaunchKernelGGL(patch_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, token_ids, patch, source, n,
+                     sources);
+  return ts_launch_status();
+}

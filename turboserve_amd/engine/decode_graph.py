@@ -84,7 +84,7 @@ class DecodeGraphs:
             offsets[name] = (cursor, length)
             cursor += -(-length // 4) * 4  # keep every field 16-byte aligned
 
-        for name in ("token_ids", "positions", "token_seq", "context_lens", "state_slots", "logit_rows"):
+        for name in ("token_ids", "positions", "token_seq", "context_lens", "state_slots", "logit_rows", "patch"):
             take(name, batch)
         take("query_start_loc", batch + 1)
         take("max_context", 1)
@@ -151,8 +151,9 @@ class DecodeGraphs:
             self._pool = shape.graph.pool()
         return shape
 
-    def _fill(self, shape: _Graph, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Write a step into the next pinned buffer; rows beyond the entries are padding."""
+    def _fill(self, shape: _Graph, entries: Sequence[StepEntry], patch: dict[int, int] | None = None) -> torch.Tensor:
+        """Write a step into the next pinned buffer; rows beyond the entries are padding.
+        ``patch[i] = j``: entry ``i`` takes its token from element ``j`` of a device tensor."""
         shape.turn ^= 1
         host = shape.host_ints[shape.turn]
         data = host.numpy()
@@ -164,6 +165,9 @@ class DecodeGraphs:
 
         field("token_ids")[:live] = [e.tokens[0] for e in entries]
         field("token_ids")[live:] = 0
+        field("patch")[:] = -1
+        if patch:
+            field("patch")[list(patch)] = list(patch.values())
         field("positions")[:live] = [e.start for e in entries]
         field("positions")[live:] = 0
         field("token_seq")[:] = np.arange(batch, dtype=np.int32)
@@ -187,15 +191,21 @@ class DecodeGraphs:
 
     # -- the step --------------------------------------------------------------------------------
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], *, tokens_from: tuple[torch.Tensor, dict[int, int]] | None = None
+            ) -> torch.Tensor:
         """Replay the graph of the entries' shape; returns the graph's own 32-bit logits buffer
-        ``[len(entries), V]`` (overwritten by the next replay of that shape)."""
+        ``[len(entries), V]`` (overwritten by the next replay of that shape).  ``tokens_from =
+        (source, {entry index: element of source})``: those entries' token ids are not known on
+        the host yet and are copied on the device from ``source`` (int32) before the replay."""
         key = self._key(entries)
         shape = self._graphs.get(key)
         if shape is None:
             shape = self._graphs[key] = self._build(key)
-        host = self._fill(shape, entries)
+        host = self._fill(shape, entries, tokens_from[1] if tokens_from else None)
         shape.device_ints.copy_(host, non_blocking=True)
+        if tokens_from and tokens_from[1]:
+            start, length = shape.offsets["patch"]
+            self.model.runtime.ops.patch_tokens(shape.ctx.token_ids, shape.device_ints[start:start + length], tokens_from[0])
         shape.graph.replay()
         self.num_replays += 1
         return shape.logits[: len(entries)]

@@ -12,7 +12,7 @@ import dataclasses
 import logging
 import time
 from collections.abc import Sequence as SequenceABC
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any
 
 import torch
@@ -49,6 +49,25 @@ class EngineStats:
 
     def to_dict(self) -> dict[str, int | float]:
         return dataclasses.asdict(self)
+
+
+@dataclass
+class _InFlight:
+    """A step that has been launched and whose sampled tokens are still on the device."""
+
+    sampled: list  # the step's ScheduledSeq items that sample, in the order of the sampler's rows
+    pending: Any   # sampler.PendingSample (or a stand-in with read()); None if nothing samples
+    places: dict = field(default_factory=dict)  # seq_id -> place of this step's token in the request's output, if taken ahead
+
+
+@dataclass
+class _Sampled:
+    """A sampler result that is already on the host, in the shape of a pending one."""
+
+    result: Any
+
+    def read(self):
+        return self.result
 
 
 class LLMEngine:
@@ -121,6 +140,7 @@ class LLMEngine:
         self._num_generated_tokens = 0
         self._num_prompt_tokens = 0
         self._closed = False
+        self._in_flight: _InFlight | None = None  # a step launched ahead whose tokens have not been read
 
     # -- helpers --------------------------------------------------------------------------------
 
@@ -207,37 +227,96 @@ class LLMEngine:
     def step(self, *, now: float | None = None) -> list[RequestOutput]:
         """Advance every scheduled request.  An empty list is normal: nothing queued, only
         unfinished portions of prompts ran, or everything scheduled was preempted
-        (engine.py:340-356)."""
+        (engine.py:340-356).
+
+        With ``config.run_ahead`` a decode step is launched before the tokens of the step before
+        it have been read (``_run_ahead``); a call then returns the outputs of the step that was
+        launched by the call before it."""
         if self._closed:
             raise RuntimeError("engine is closed")
         timestamp = time.perf_counter() if now is None else now
-        scheduled = self.scheduler.schedule(now=timestamp)
-        outputs = [self._output_for_dropped(seq) for seq in scheduled.dropped]
-        if scheduled.is_empty:
-            return outputs
-        tokens, logprobs = self._execute(scheduled)
-        outputs.extend(self._process(scheduled, tokens, logprobs, now=timestamp))
+        outputs: list[RequestOutput] = []
+        flight, self._in_flight = self._in_flight, None
+        if flight is None:
+            scheduled = self.scheduler.schedule(now=timestamp)
+            outputs.extend(self._output_for_dropped(seq) for seq in scheduled.dropped)
+            if scheduled.is_empty:
+                return outputs
+            flight = self._launch(scheduled)
+        if self.config.run_ahead:
+            self._in_flight = self._run_ahead(flight, outputs, now=timestamp)
+        outputs.extend(self._collect(flight, now=timestamp))
         return outputs
 
-    def _execute(self, scheduled: SchedulerOutput) -> tuple[list[int], list[float] | None]:
-        logits = self.runner.step(scheduled.entries(), fresh_state_slots=scheduled.fresh_state_slots)
+    def _launch(self, scheduled: SchedulerOutput, tokens_from=None) -> "_InFlight":
+        """Start a step on the GPU: the model, then the sampler; nothing is waited for."""
+        logits = self.runner.step(scheduled.entries(), fresh_state_slots=scheduled.fresh_state_slots,
+                                  **({"tokens_from": tokens_from} if tokens_from is not None else {}))
         sampled = scheduled.sampled()
-        if not sampled:
-            return [], None
-        result = self.sampler.sample_sequences(logits, [item.seq for item in sampled])
-        return result.token_ids, result.logprobs
+        pending = self._launch_sampler(logits, [item.seq for item in sampled]) if sampled else None
+        return _InFlight(sampled, pending)
 
-    def _process(self, scheduled, tokens, logprobs, *, now: float) -> list[RequestOutput]:
-        """Feed sampled tokens back: stop checks, text, per-request deltas (engine.py:366-410)."""
+    def _launch_sampler(self, logits, sequences):
+        launch = getattr(self.sampler, "launch_sequences", None)
+        if launch is not None:
+            return launch(logits, sequences)
+        return _Sampled(self.sampler.sample_sequences(logits, sequences))  # a stand-in sampler without a launch/read split
+
+    def _run_ahead(self, flight: "_InFlight", outputs: list[RequestOutput], *, now: float) -> "_InFlight | None":
+        """Schedule and launch the step after ``flight`` while ``flight`` still runs.
+
+        Possible when that step is known without the tokens' values: every request of
+        ``flight`` samples, they are all the running requests, nothing waits to be admitted, none
+        of them reaches ``max_tokens`` with the token being sampled or needs its own history for
+        a penalty, and the step replays as a graph.  Each request gets a place for its unread
+        token; the step's token ids are copied on the device from the sampler's result.  A
+        request that then turns out to have ended (a stop token, a stop string, an abort) leaves
+        a row in the launched step whose result is dropped."""
+        live = [item.seq for item in flight.sampled if not item.seq.is_finished]
+        tokens = getattr(flight.pending, "tokens", None)
+        if not live or tokens is None or len(live) != len(flight.sampled):
+            return None
+        takes = getattr(self.runner, "takes_tokens_from", None)
+        if takes is None or not takes(len(live)) or not self.scheduler.only_running(live):
+            return None
+        for seq in live:
+            if seq.sampling.repetition_penalty != 1.0 or seq.num_output_tokens + 1 >= seq.sampling.max_tokens:
+                return None
+        source = {seq.seq_id: index for index, seq in enumerate(live)}
+        for seq in live:
+            flight.places[seq.seq_id] = seq.append_unread_token()
+        scheduled = self.scheduler.schedule(now=now)
+        outputs.extend(self._output_for_dropped(seq) for seq in scheduled.dropped)
+        if scheduled.is_empty:
+            return None
+        patch = {}
+        for index, item in enumerate(scheduled.scheduled):
+            if item.num_new_tokens != 1 or item.seq.seq_id not in source:
+                raise RuntimeError("the step scheduled ahead holds something other than the running requests' next tokens")
+            patch[index] = source[item.seq.seq_id]
+        return self._launch(scheduled, tokens_from=(tokens, patch))
+
+    def _collect(self, flight: "_InFlight", *, now: float) -> list[RequestOutput]:
+        """Wait for a launched step's tokens and feed them back: stop checks, text, per-request
+        deltas (engine.py:366-410)."""
+        if flight.pending is None:
+            return []
+        result = flight.pending.read()
+        tokens, logprobs = result.token_ids, result.logprobs
         outputs = []
-        for index, (item, token) in enumerate(zip(scheduled.sampled(), tokens)):
+        for index, (item, token) in enumerate(zip(flight.sampled, tokens)):
             seq = item.seq
             if seq.is_finished:
-                continue
+                continue  # aborted meanwhile, or ended by the step before this one was launched ahead of
             logprob = None
             if logprobs is not None and seq.sampling.logprobs:
                 logprob = logprobs[index]
-            reason = self.scheduler.append_token(seq, token, eos_token_ids=self._eos_token_ids, logprob=logprob, now=now)
+            place = flight.places.get(seq.seq_id)
+            if place is None:
+                reason = self.scheduler.append_token(seq, token, eos_token_ids=self._eos_token_ids, logprob=logprob, now=now)
+            else:
+                reason = self.scheduler.resolve_token(seq, place, token, eos_token_ids=self._eos_token_ids,
+                                                      logprob=logprob, now=now)
             outputs.append(self._emit(seq, token, reason, logprob, now=now))
         self._num_generated_tokens += len(outputs)
         return outputs
@@ -345,6 +424,7 @@ class LLMEngine:
         if self._closed:
             return
         self._closed = True
+        self._in_flight = None
         self.scheduler.reset()
         self._decoders.clear()
         self.storage = None

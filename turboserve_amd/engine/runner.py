@@ -48,9 +48,13 @@ class ModelRunner:
             self.graphs.release()
             self.graphs = None
 
-    def check_tokens(self, entries: Sequence[StepEntry]) -> None:
+    def check_tokens(self, entries: Sequence[StepEntry], unknown: Sequence[int] = ()) -> None:
+        """Every token id is inside the vocabulary; ``unknown``: indices of entries whose token
+        is still on the device (see ``step``)."""
         vocab = self.vocab_size
-        for entry in entries:
+        for index, entry in enumerate(entries):
+            if index in unknown:
+                continue
             for token in entry.tokens:
                 if not 0 <= token < vocab:
                     raise ValueError(f"request {entry.request!r}: token id {token} is outside the vocabulary of {vocab}")
@@ -67,16 +71,24 @@ class ModelRunner:
         )
 
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry], *, fresh_state_slots: Sequence[int] = ()) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], *, fresh_state_slots: Sequence[int] = (),
+             tokens_from: tuple[torch.Tensor, dict[int, int]] | None = None) -> torch.Tensor:
         """Run one step and return 32-bit logits ``[wanted, V]`` on the device, in the order of
         the entries and of each entry's ``want``.  A step that wants nothing still runs (it
-        fills the cache, worker.py:248-256) and returns ``[0, V]``."""
+        fills the cache, worker.py:248-256) and returns ``[0, V]``.
+
+        ``tokens_from = (source, {entry index: element})``: the single token of those entries
+        is element ``element`` of the int32 device tensor ``source`` (what the step before
+        sampled, not read back yet); only steps that replay as a graph take it
+        (``takes_tokens_from``)."""
         self.storage.zero_state_slots(fresh_state_slots)
         device = self.model.runtime.device
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=device)
         if self.graphs is not None and self.graphs.accepts(entries):
-            return self._graph_step(entries)
+            return self._graph_step(entries, tokens_from)
+        if tokens_from is not None:
+            raise ValueError("only a step of single tokens that replays as a graph can take tokens from the device")
         ctx = self.context_for(entries)
         stream = self.model.forward(ctx.token_ids, ctx, self.views)
         self.num_steps += 1
@@ -101,13 +113,17 @@ class ModelRunner:
         self.model.logits(stream, ctx.logit_rows)
         torch.cuda.synchronize(self.model.runtime.device)
 
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def takes_tokens_from(self, num_entries: int) -> bool:
+        """Whether a step of ``num_entries`` single tokens would replay as a graph."""
+        return self.graphs is not None and 0 < num_entries <= self.graphs.max_batch
+
+    def _graph_step(self, entries: Sequence[StepEntry], tokens_from=None) -> torch.Tensor:
         """A step of single tokens through its recorded graph.  The result is the graph's own
         buffer (or rows gathered from it): read it before the next step."""
         if self.check:
-            self.check_tokens(entries)
+            self.check_tokens(entries, tokens_from[1] if tokens_from else ())
             validate_entries(entries, len(self.layout.groups), self.storage.page_size)
-        logits = self.graphs.run(entries)
+        logits = self.graphs.run(entries, tokens_from=tokens_from)
         self.num_steps += 1
         wanted = [i for i, entry in enumerate(entries) if len(entry.want) > 0]
         if len(wanted) == len(entries):

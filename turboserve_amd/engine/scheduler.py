@@ -191,6 +191,27 @@ class Scheduler:
             self.finish(seq, reason, now=now, stop_token_id=stop)
         return reason
 
+    def resolve_token(
+        self, seq: Sequence, place: int, token_id: int, *, eos_token_ids=frozenset(), logprob: float | None = None,
+        now: float | None = None,
+    ) -> FinishReason | None:
+        """``append_token`` for a token whose place was taken ahead of its value
+        (``Sequence.append_unread_token``)."""
+        seq.set_unread_token(place, token_id, logprob=logprob, now=now)
+        reason = seq.check_stop(token_id, eos_token_ids=eos_token_ids)
+        if reason is not None:
+            stop = token_id if reason is FinishReason.STOP else None
+            self.finish(seq, reason, now=now, stop_token_id=stop)
+        return reason
+
+    def only_running(self, sequences: SequenceABC[Sequence]) -> bool:
+        """Whether ``sequences`` are exactly the requests that could be in the next step: nothing
+        waits, nothing is preempted, and the running requests are these."""
+        if self._waiting or self._preempted or len(self._running) != len(sequences):
+            return False
+        running = {seq.seq_id for seq in self._running}
+        return all(seq.seq_id in running and seq.status is SeqStatus.RUNNING for seq in sequences)
+
     def has_unfinished(self) -> bool:
         return bool(self._by_request)
 

@@ -136,6 +136,27 @@ class Sequence:
         if self.timing.t_first_token is None:
             self.timing.t_first_token = time.perf_counter() if now is None else now
 
+    #: Stands in the output for a token that is sampled but has not been read from the device.
+    UNREAD_TOKEN = -1
+
+    def append_unread_token(self) -> int:
+        """Make room for a token whose value is not known yet (the step after the one that
+        samples it is being prepared); returns its place in ``output_token_ids`` for
+        ``set_unread_token``."""
+        if self.is_finished:
+            raise ValueError(f"sequence {self.request_id!r} finished with {self.finish_reason}; no token can be appended")
+        self.output_token_ids.append(self.UNREAD_TOKEN)
+        return len(self.output_token_ids) - 1
+
+    def set_unread_token(self, place: int, token_id: int, *, logprob: float | None = None, now: float | None = None) -> None:
+        if self.output_token_ids[place] != self.UNREAD_TOKEN:
+            raise ValueError(f"sequence {self.request_id!r}: output token {place} is already known")
+        self.output_token_ids[place] = int(token_id)
+        if logprob is not None:
+            self.output_logprobs.append(float(logprob))
+        if self.timing.t_first_token is None:
+            self.timing.t_first_token = time.perf_counter() if now is None else now
+
     def check_stop(self, token_id: int, *, eos_token_ids=frozenset()) -> FinishReason | None:
         """Whether the token just appended ends the request: a stop id, an end-of-sequence id
         unless ``ignore_eos``, or ``max_tokens`` reached (sequence.py:282-296).  The stop token

@@ -47,6 +47,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_int, c_int, c_void_p],
@@ -247,6 +248,18 @@ class Ops:
         _check(self.core.ts_gather_rows(_ptr(out), _ptr(x), _ptr(rows), rows.numel(), x.shape[1],
                                         dtype_code(x.dtype), self.stream()), "ts_gather_rows")
         return out
+
+    def patch_tokens(self, token_ids: torch.Tensor, patch: torch.Tensor, source: torch.Tensor) -> None:
+        """``token_ids[i] = source[patch[i]]`` where ``patch[i] >= 0``, in place: a step's token
+        ids taken from what the step before sampled, without the host having seen them."""
+        _gpu(token_ids, patch, source)
+        _i32(token_ids, "token_ids")
+        _i32(patch, "patch")
+        _i32(source, "source")
+        _need(token_ids.dim() == 1 and patch.shape == token_ids.shape and source.dim() == 1 and source.numel() >= 1,
+              "token_ids and patch must be [n], source [m >= 1]")
+        _check(self.core.ts_patch_tokens(_ptr(token_ids), _ptr(patch), _ptr(source), token_ids.numel(), source.numel(),
+                                         self.stream()), "ts_patch_tokens")
 
     def rope_store(
         self,

@@ -27,6 +27,39 @@ class SamplerOutput:
     logprobs: list[float] | None = None  # nan for rows that did not ask (sampler.py:66-74)
 
 
+class PendingSample:
+    """What a sampling launch left on the device.  The copy to (pinned) host memory is queued
+    right behind the sampler, with an event after it, so that ``read()`` waits for exactly this
+    and not for whatever the stream was given afterwards (a step launched ahead)."""
+
+    def __init__(self, tokens: torch.Tensor | None, logprobs: torch.Tensor | None,
+                 params: SequenceABC[SamplingParams] = ()) -> None:
+        self.tokens = tokens        # int32 [n] where it was computed, or None for no rows
+        self.logprobs = logprobs    # float32 [n] or None
+        self.params = params
+        self._host_tokens = self._host_logprobs = self._event = None
+        if tokens is not None and tokens.is_cuda:
+            self._host_tokens = torch.empty(tokens.shape, dtype=tokens.dtype, pin_memory=True)
+            self._host_tokens.copy_(tokens, non_blocking=True)
+            if logprobs is not None:
+                self._host_logprobs = torch.empty(logprobs.shape, dtype=logprobs.dtype, pin_memory=True)
+                self._host_logprobs.copy_(logprobs, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(tokens.device))
+
+    def read(self) -> SamplerOutput:
+        if self.tokens is None:
+            return SamplerOutput(token_ids=[])
+        if self._event is not None:
+            self._event.synchronize()
+        tokens = self._host_tokens if self._host_tokens is not None else self.tokens
+        out = SamplerOutput(token_ids=tokens.tolist())
+        if self.logprobs is not None:
+            values = (self._host_logprobs if self._host_logprobs is not None else self.logprobs).tolist()
+            out.logprobs = [v if p.logprobs else float("nan") for v, p in zip(values, self.params)]
+        return out
+
+
 class Sampler:
     def __init__(self, ops) -> None:
         self.ops = ops
@@ -44,15 +77,27 @@ class Sampler:
         ``seeds[i]`` / ``draw_indices[i]``: key and counter of row ``i``'s draw.
         ``histories[i]``: prompt + output tokens, read only when the row has a repetition
         penalty other than 1."""
+        return self.launch(logits, params, seeds, draw_indices, histories).read()
+
+    def launch(
+        self,
+        logits: torch.Tensor,
+        params: SequenceABC[SamplingParams],
+        seeds: SequenceABC[int],
+        draw_indices: SequenceABC[int],
+        histories: SequenceABC[SequenceABC[int]] | None = None,
+    ) -> PendingSample:
+        """``sample`` without the wait: the kernels are launched and the tokens stay on the
+        device until ``PendingSample.read``."""
         rows = int(logits.shape[0])
         if len(params) != rows or len(seeds) != rows or len(draw_indices) != rows:
             raise ValueError(f"{len(params)} params / {len(seeds)} seeds / {len(draw_indices)} counters for {rows} rows")
         if histories is not None and len(histories) != rows:
             raise ValueError(f"{len(histories)} histories for {rows} rows of logits")
         if rows == 0:
-            return SamplerOutput(token_ids=[])
+            return PendingSample(None, None)
         if all(p.is_plain_greedy for p in params):
-            return SamplerOutput(token_ids=self.ops.argmax(logits).tolist())
+            return PendingSample(self.ops.argmax(logits), None, params)
 
         want_logprobs = any(p.logprobs for p in params)
         history_start = [0]
@@ -83,16 +128,16 @@ class Sampler:
         tokens, logprobs = self.ops.sample(
             logits, fdev[0], top_k, fdev[1], fdev[2], seed_lo, seed_hi, draw, hist, hstart, want_logprobs
         )
-        out = SamplerOutput(token_ids=tokens.tolist())
-        if logprobs is not None:
-            values = logprobs.tolist()
-            out.logprobs = [v if p.logprobs else float("nan") for v, p in zip(values, params)]
-        return out
+        return PendingSample(tokens, logprobs, list(params))
 
     def sample_sequences(self, logits: torch.Tensor, sequences: SequenceABC[Sequence]) -> SamplerOutput:
         """Sample for requests: options, seed, draw counter (= tokens produced so far) and,
         only if a penalty is set, the token history of each (sampler.py:240-256)."""
-        return self.sample(
+        return self.launch_sequences(logits, sequences).read()
+
+    def launch_sequences(self, logits: torch.Tensor, sequences: SequenceABC[Sequence]) -> PendingSample:
+        """``sample_sequences`` without the wait."""
+        return self.launch(
             logits,
             [seq.sampling for seq in sequences],
             [seq.sample_seed for seq in sequences],

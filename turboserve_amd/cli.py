@@ -38,8 +38,11 @@ def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> Non
     p.set_defaults(prefix_caching=False)
     p.add_argument("--tune-gemm", action="store_true",
                    help="time the BLAS library's kernels for a full step of prompt tokens at start-up and keep the fastest")
-    p.add_argument("--run-ahead", action="store_true",
-                   help="launch each decode step before the host has read the tokens of the step before it")
+    p.add_argument("--run-ahead", dest="run_ahead", action="store_true",
+                   help="launch each decode step before the host has read the tokens of the step before it (the default)")
+    p.add_argument("--no-run-ahead", dest="run_ahead", action="store_false",
+                   help="read every step's tokens before the next step is scheduled, as the reference does")
+    p.set_defaults(run_ahead=True)
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -95,7 +98,7 @@ def _generate(args: argparse.Namespace) -> int:
     config = EngineConfig(
         model=args.model, device=args.device, dtype=args.dtype, seed=args.seed,
         tune_gemm_tokens=(args.max_num_batched_tokens,) if args.tune_gemm else (),
-        run_ahead=getattr(args, "run_ahead", False),
+        run_ahead=getattr(args, "run_ahead", True),
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
             block_size=args.block_size, num_blocks=args.num_blocks, enable_prefix_caching=args.prefix_caching,

@@ -72,7 +72,7 @@ class EngineConfig:
     #: are copied on the device), so that the GPU does not wait while the host schedules and
     #: builds outputs.  Results are the same tokens; a request that ends on a stop token costs
     #: one token's worth of work that is thrown away.  No counterpart in the reference.
-    run_ahead: bool = False
+    run_ahead: bool = True
 
     def __post_init__(self) -> None:
         if self.speculative is not None or self.lora is not None:

@@ -192,3 +192,31 @@ def test_a_step_is_not_launched_ahead_of_a_request_that_ends_by_length_or_has_a_
     expected = continuation([5, 6, 7], SamplingParams(max_tokens=6, stop_token_ids=(stop,)))
     assert tokens == expected and tokens[-1] == stop and len(tokens) < 6 and runner.steps == len(tokens) + 1
     assert engine.step() == [] and engine.step() == []  # the dropped step is read and forgotten
+
+
+def test_requests_that_end_at_different_lengths_do_not_stop_the_running_ahead():
+    """A request whose token in flight is its last takes no part in the step launched ahead;
+    the others go on.  A request that ended on a stop token leaves a dropped row and the others
+    go on all the same."""
+    engine, runner = make_engine(True)
+    lengths = {"a": 3, "b": 9, "c": 6}
+    for name, length in lengths.items():
+        engine.add_request(name, [1, 2, ord(name) % VOCAB], SamplingParams(max_tokens=length, temperature=0.0, ignore_eos=True))
+    got = {name: [] for name in lengths}
+    while engine.has_unfinished():
+        for output in engine.step():
+            got[output.request_id].extend(output.new_token_ids)
+    for name, length in lengths.items():
+        assert got[name] == continuation([1, 2, ord(name) % VOCAB], SamplingParams(max_tokens=length))
+    assert runner.steps == 9 and runner.steps_ahead == 8  # every step but the first
+    stop = continuation([1, 2, 3], SamplingParams(max_tokens=9))[3]
+    engine, runner = make_engine(True)
+    engine.add_request("s", [1, 2, 3], SamplingParams(max_tokens=9, temperature=0.0, ignore_eos=True, stop_token_ids=(stop,)))
+    engine.add_request("t", [4, 5, 6], SamplingParams(max_tokens=9, temperature=0.0, ignore_eos=True))
+    got = {"s": [], "t": []}
+    while engine.has_unfinished():
+        for output in engine.step():
+            got[output.request_id].extend(output.new_token_ids)
+    assert got["s"] == continuation([1, 2, 3], SamplingParams(max_tokens=9, stop_token_ids=(stop,))) and len(got["s"]) < 9
+    assert got["t"] == continuation([4, 5, 6], SamplingParams(max_tokens=9))
+    assert runner.steps == 9 and runner.steps_ahead == 8

@@ -265,26 +265,28 @@ class LLMEngine:
     def _run_ahead(self, flight: "_InFlight", outputs: list[RequestOutput], *, now: float) -> "_InFlight | None":
         """Schedule and launch the step after ``flight`` while ``flight`` still runs.
 
-        Possible when that step is known without the tokens' values: every request of
-        ``flight`` samples, they are all the running requests, nothing waits to be admitted, none
-        of them reaches ``max_tokens`` with the token being sampled or needs its own history for
-        a penalty, and the step replays as a graph.  Each request gets a place for its unread
-        token; the step's token ids are copied on the device from the sampler's result.  A
-        request that then turns out to have ended (a stop token, a stop string, an abort) leaves
-        a row in the launched step whose result is dropped."""
+        Possible when that step is known without the tokens' values: the unfinished requests of
+        ``flight`` all sample and are all the running requests, nothing waits to be admitted,
+        none needs its own history for a penalty, and the step replays as a graph.  Each request
+        gets a place for its unread token (unless that token is its last by ``max_tokens``: then
+        it has no part in the next step); the step's token ids are copied on the device from the
+        sampler's result.  A request that then turns out to have ended (a stop token, a stop
+        string, an abort) leaves a row in the launched step whose result is dropped."""
+        source = {item.seq.seq_id: row for row, item in enumerate(flight.sampled) if not item.seq.is_finished}
         live = [item.seq for item in flight.sampled if not item.seq.is_finished]
         tokens = getattr(flight.pending, "tokens", None)
-        if not live or tokens is None or len(live) != len(flight.sampled):
+        if not live or tokens is None:
             return None
         takes = getattr(self.runner, "takes_tokens_from", None)
         if takes is None or not takes(len(live)) or not self.scheduler.only_running(live):
             return None
+        if any(seq.sampling.repetition_penalty != 1.0 for seq in live):
+            return None
         for seq in live:
-            if seq.sampling.repetition_penalty != 1.0 or seq.num_output_tokens + 1 >= seq.sampling.max_tokens:
-                return None
-        source = {seq.seq_id: index for index, seq in enumerate(live)}
-        for seq in live:
-            flight.places[seq.seq_id] = seq.append_unread_token()
+            # A request that reaches max_tokens with the token in flight takes no place: it has
+            # nothing to compute in the next step and ends when its token is read.
+            if seq.num_output_tokens + 1 < seq.sampling.max_tokens:
+                flight.places[seq.seq_id] = seq.append_unread_token()
         scheduled = self.scheduler.schedule(now=now)
         outputs.extend(self._output_for_dropped(seq) for seq in scheduled.dropped)
         if scheduled.is_empty:

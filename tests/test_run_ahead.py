@@ -97,7 +97,7 @@ def drive(engine, arrivals, *, abort_at=None):
         if abort_at is not None and step == abort_at[0]:
             engine.abort(abort_at[1])
         for output in engine.step():
-            got[output.request_id].extend(output.new_token_ids)
+            got.setdefault(output.request_id, []).extend(output.new_token_ids)
             if output.finished:
                 reasons[output.request_id] = output.finish_reason.value
         step += 1
@@ -151,12 +151,17 @@ def test_run_ahead_with_preemption_and_an_abort():
             expected[f"r{index}"] = continuation(prompt, params)
             arrivals[0].append((f"r{index}", prompt, params))
         engine, runner = make_engine(True, num_blocks=14, max_num_seqs=6)
+        for request_id, prompt, params in arrivals.pop(0):
+            sequence = engine.add_request(request_id, prompt, params)
+            if request_id == "r2":
+                aborted = sequence
         got, reasons = drive(engine, arrivals, abort_at=(6, "r2"))
         preemptions += engine.scheduler.stats()["num_preemptions"]
         assert runner.steps_ahead > 0
         for request_id, tokens in expected.items():
             if request_id == "r2":
                 assert "r2" not in reasons and got[request_id] == tokens[: len(got[request_id])]  # aborted on the way
+                assert aborted.output_token_ids == got[request_id]  # no place of an unread token is left behind
             else:
                 assert got[request_id] == tokens, (seed, request_id)
     assert preemptions > 0

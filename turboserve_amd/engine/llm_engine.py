@@ -309,7 +309,10 @@ class LLMEngine:
         for index, (item, token) in enumerate(zip(flight.sampled, tokens)):
             seq = item.seq
             if seq.is_finished:
-                continue  # aborted meanwhile, or ended by the step before this one was launched ahead of
+                # aborted meanwhile, or ended by the step before this one was launched ahead of
+                if seq.seq_id in flight.places:
+                    seq.drop_unread_token(flight.places[seq.seq_id])
+                continue
             logprob = None
             if logprobs is not None and seq.sampling.logprobs:
                 logprob = logprobs[index]

@@ -157,6 +157,11 @@ class Sequence:
         if self.timing.t_first_token is None:
             self.timing.t_first_token = time.perf_counter() if now is None else now
 
+    def drop_unread_token(self, place: int) -> None:
+        """Forget a place whose token will not be read (the request was aborted meanwhile)."""
+        if place < len(self.output_token_ids) and self.output_token_ids[place] == self.UNREAD_TOKEN:
+            del self.output_token_ids[place:]
+
     def check_stop(self, token_id: int, *, eos_token_ids=frozenset()) -> FinishReason | None:
         """Whether the token just appended ends the request: a stop id, an end-of-sequence id
         unless ``ignore_eos``, or ``max_tokens`` reached (sequence.py:282-296).  The stop token

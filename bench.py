@@ -4,7 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A "step" is one decode step of the whole engine path: the step function over a batch of
-single tokens against the paged cache, logits, greedy sampling, tokens back on the host.
+single tokens against the paged cache, logits, greedy sampling, tokens back on the host.  As
+in the engine's own loop a step is launched before the host has read the tokens of the step
+before it (its token ids are copied from the sampler's result on the device); every step's
+tokens are read, one step later, and the clock stops after the last are.
 The default run has the Qwen2.5-7B layer sizes (the benchmark's named configuration), random weights
 (N(0, 0.02), norm gains 1), a batch of 8 requests each holding a context of 8,192 tokens
 (cache filled with random keys and values; what is timed is real decode steps on top of it).
@@ -110,6 +113,7 @@ class DecodeBench:
         self.manager = CacheManager(self.storage.layout.windows(), num_pages, PAGE, batch + 1)
         self.runner = ModelRunner(model, self.storage, check=False)
         self.sampler = Sampler(model.runtime.ops)
+        self.pending = None  # the sampler's result of a step whose tokens have not been read yet
         generator = torch.Generator().manual_seed(1234)
         self.tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
         self.portion = torch.randint(0, config.vocab_size, (max(extra_tokens, 1),), generator=generator).tolist()
@@ -146,22 +150,48 @@ class DecodeBench:
             slots = self.manager.append(request, 1)
             entries.append(StepEntry(request=request, tokens=[self.tokens[request]], start=start,
                                      tables=held.tables, slots=slots, state_slot=held.state_slot, want=[0]))
-        logits = self.runner.step(entries)
         greedy = SamplingParams(temperature=0.0)
-        out = self.sampler.sample(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
-        self.tokens = out.token_ids
+        if portion_tokens or not self.runner.takes_tokens_from(self.batch):
+            # A step with a portion of a prompt does not replay as a graph: its tokens are read
+            # before the next step is built, as the engine does for such steps.
+            self.finish()
+            logits = self.runner.step(entries)
+            out = self.sampler.sample(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
+            self.tokens = out.token_ids
+        else:
+            # As the engine's loop does (LLMEngine._run_ahead): the step is launched with its token
+            # ids taken on the device from what the step before sampled, and that step's tokens
+            # are read only afterwards, so the GPU does not wait while the host builds a step.
+            before = self.pending
+            if before is not None:
+                for entry in entries:
+                    entry.tokens = [-1]
+                logits = self.runner.step(entries, tokens_from=(before.tokens, {i: i for i in range(self.batch)}))
+            else:
+                logits = self.runner.step(entries)
+            self.pending = self.sampler.launch(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
+            if before is not None:
+                self.tokens = before.read().token_ids
         if portion_tokens:
             self.manager.free("portion")
+
+    def finish(self) -> None:
+        """Read the tokens of the step that is still in flight, if one is."""
+        if self.pending is not None:
+            self.tokens = self.pending.read().token_ids
+            self.pending = None
 
     def run(self, steps: int, warmup: int, portion_tokens: int = 0) -> float:
         """Seconds for ``steps`` steps after ``warmup`` untimed ones."""
         torch = self.torch
         for _ in range(warmup):
             self.step(portion_tokens)
+        self.finish()
         torch.cuda.synchronize()
         started = time.perf_counter()
         for _ in range(steps):
             self.step(portion_tokens)
+        self.finish()
         torch.cuda.synchronize()
         return time.perf_counter() - started
 

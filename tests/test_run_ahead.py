@@ -225,3 +225,34 @@ def test_requests_that_end_at_different_lengths_do_not_stop_the_running_ahead():
     assert got["s"] == continuation([1, 2, 3], SamplingParams(max_tokens=9, stop_token_ids=(stop,))) and len(got["s"]) < 9
     assert got["t"] == continuation([4, 5, 6], SamplingParams(max_tokens=9))
     assert runner.steps == 9 and runner.steps_ahead == 8
+
+
+class LetterTokenizer:
+    """Token i decodes to the letter chr(ord('a') + i % 26)."""
+
+    def decode(self, ids, skip_special_tokens=True):
+        return "".join(chr(ord("a") + i % 26) for i in ids)
+
+    def encode(self, text, add_special_tokens=False):
+        return [ord(c) - ord("a") for c in text]
+
+
+def test_a_stop_string_ends_a_request_at_the_same_place_when_steps_run_ahead():
+    prompt = [3, 1, 4]
+    plain = continuation(prompt, SamplingParams(max_tokens=12))
+    text = LetterTokenizer().decode(plain)
+    stop = text[4:6]  # the request must end before these two letters
+    results = []
+    for ahead in (False, True):
+        cfg = SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=32, block_size=4, num_blocks=32)
+        runner = ToyRunner()
+        engine = LLMEngine(EngineConfig(model="/nonexistent", scheduler=cfg, run_ahead=ahead), model=object(),
+                           tokenizer=LetterTokenizer(), scheduler=Scheduler(cfg, CacheManager([None], 32, 4, 4)),
+                           runner=runner, sampler=ToySampler())
+        outputs = engine.generate([prompt, [2, 7, 1]], [SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True, stop=[stop]),
+                                                        SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)])
+        results.append([(o.new_token_ids, o.text_delta, o.finish_reason) for o in outputs])
+        assert outputs[0].finish_reason == "stop" and outputs[0].text_delta == text[: text.index(stop)]
+        assert outputs[1].new_token_ids == continuation([2, 7, 1], SamplingParams(max_tokens=12))
+        assert (runner.steps_ahead > 0) == ahead
+    assert results[0] == results[1]

@@ -250,8 +250,11 @@ class LLMEngine:
 
     def _launch(self, scheduled: SchedulerOutput, tokens_from=None) -> "_InFlight":
         """Start a step on the GPU: the model, then the sampler; nothing is waited for."""
-        logits = self.runner.step(scheduled.entries(), fresh_state_slots=scheduled.fresh_state_slots,
-                                  **({"tokens_from": tokens_from} if tokens_from is not None else {}))
+        entries = scheduled.entries()
+        if tokens_from is None:
+            logits = self.runner.step(entries, fresh_state_slots=scheduled.fresh_state_slots)
+        else:  # only a runner that said it takes them (`takes_tokens_from`) is asked to
+            logits = self.runner.step(entries, fresh_state_slots=scheduled.fresh_state_slots, tokens_from=tokens_from)
         sampled = scheduled.sampled()
         pending = self._launch_sampler(logits, [item.seq for item in sampled]) if sampled else None
         return _InFlight(sampled, pending)

@@ -100,6 +100,17 @@ def validate_entries(entries: Sequence[StepEntry], num_groups: int, page_size: i
                 raise ValueError(f"request {entry.request!r}: wanted place {place} is outside its {count} tokens")
 
 
+def _flat(lists: Sequence[Sequence[int]], count: int) -> np.ndarray:
+    """The lists one after the other as int32 (each converted in one call: a prompt portion is
+    thousands of values)."""
+    if not lists:
+        return np.zeros(0, dtype=np.int32)
+    out = np.concatenate([np.asarray(values, dtype=np.int32) for values in lists])
+    if out.size != count:
+        raise ValueError(f"{out.size} values for {count} tokens")
+    return out
+
+
 def build_context(
     entries: Sequence[StepEntry],
     *,
@@ -140,7 +151,7 @@ def build_context(
     block_array = np.asarray([[b[1], b[2]] for b in blocks], dtype=np.int32).reshape(-1)
 
     pieces: list[np.ndarray] = [
-        np.fromiter((t for e in entries for t in e.tokens), dtype=np.int32, count=num_tokens),
+        _flat([e.tokens for e in entries], num_tokens),
         np.concatenate([np.arange(e.start, e.start + n, dtype=np.int32) for e, n in zip(entries, query_lens)])
         if num_seqs else np.zeros(0, dtype=np.int32),
         np.repeat(np.arange(num_seqs, dtype=np.int32), query_lens),
@@ -151,7 +162,7 @@ def build_context(
         block_array,
     ]
     for g in range(num_groups):
-        pieces.append(np.fromiter((s for e in entries for s in e.slots[g]), dtype=np.int32, count=num_tokens))
+        pieces.append(_flat([e.slots[g] for e in entries], num_tokens))
         table = np.full((num_seqs, widths[g]), PAD_PAGE, dtype=np.int32)
         for i, e in enumerate(entries):
             row = table_array(e.tables[g])

@@ -179,6 +179,62 @@ def test_decode_graphs_replay_like_eager(model):
             assert torch.equal(eager, graph), f"{dtype}: a graph replay differs from the eager step"
 
 
+def test_recorded_steps_survive_the_growth_of_the_rotary_tables(tmp_path):
+    """A recorded step holds the addresses of the rotary tables it was recorded with.  The
+    tables of this model start at 48 positions: a short request decodes (its step is recorded
+    against tables of 96), a 1,500-token prompt makes the tables grow, memory of the old tables'
+    size is then filled with NaN (so a freed table would be overwritten), and a second short
+    request decodes through the step recorded first.  Its logits are the plain
+    implementation's, and bit for bit those of a run without recorded steps."""
+    from turboserve_amd.engine.replay import TraceReplayer
+
+    config = {**tiny.CONFIG_A, "max_position_embeddings": 48}
+    folder = tiny.make_model_dir(tmp_path / "m", config, 11, torch.float32, std=tiny.WIDE_STD)
+    raw, tensors = tiny.read_model_dir(folder)
+    requests = {"s1": tiny.random_tokens(256, 14, 1), "long": tiny.random_tokens(256, 1503, 2),
+                "s2": tiny.random_tokens(256, 17, 3)}
+
+    def decode_tail(rid, count, end):
+        tokens = requests[rid]
+        return [{"entries": [{"id": rid, "tokens": [tokens[len(tokens) - count + k]], "want": [0]}],
+                 "end": [rid] if end and k == count - 1 else []} for k in range(count)]
+
+    steps = [{"entries": [{"id": "s1", "tokens": requests["s1"][:-4], "want": list(range(10))}], "end": []},
+             *decode_tail("s1", 4, True),
+             {"entries": [{"id": "long", "tokens": requests["long"][:-3], "want": [1499]}], "end": []},
+             {"entries": [{"id": "s2", "tokens": requests["s2"][:-5], "want": list(range(12))}], "end": []},
+             *decode_tail("s2", 5, True),
+             *decode_tail("long", 3, True)]
+    for index, record in enumerate(steps):
+        record["step"] = index
+    expected = {rid: plain.forward_logits(raw, tensors, tokens) for rid, tokens in requests.items()}
+    results = {}
+    for use_graphs in (False, True):
+        replayer = TraceReplayer(folder, dtype="float32", max_tokens=64 + 1536 + 64, page_size=16)
+        rope = replayer.model.blocks[0].mixer.position
+        if not use_graphs:
+            replayer.runner.graphs = None
+        outs, junk = {}, []
+        for record in steps:
+            outs[record["step"]] = replayer.run_step(record).float().cpu()
+            if record["entries"][0]["id"] == "long" and len(record["entries"][0]["tokens"]) > 1:
+                assert rope.capacity >= 1500
+                junk = [torch.full((rows, 8), float("nan"), device="cuda") for rows in (48, 96) for _ in range(64)]
+                torch.cuda.synchronize()
+        if use_graphs:
+            assert replayer.runner.graphs.num_replays == 12
+            assert len(replayer.runner.graphs._graphs) == 2, "s1 and s2 replay one recorded step, `long` another"
+            assert len(rope.superseded) >= 1, "the tables grew after a step had been recorded"
+        del junk
+        results[use_graphs] = outs
+        for rid, first in (("s1", 0), ("s2", 0), ("long", 1499)):
+            got = torch.cat([outs[s["step"]] for s in steps if s["entries"][0]["id"] == rid])
+            worst = float((got - expected[rid][first:]).abs().max())
+            assert worst <= 1e-4, f"graphs={use_graphs} request {rid}: {worst:.3e}"
+    for step in results[False]:
+        assert torch.equal(results[False][step], results[True][step]), f"step {step}: recorded differs from eager"
+
+
 def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
     """An engine asked to time the BLAS library's kernels at start-up: the choices are written
     to the given file, nothing is timed once the engine serves, products below the size worth

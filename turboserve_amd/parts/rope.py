@@ -26,9 +26,16 @@ def rotary_tables(capacity: int, head_dim: int, theta: float, factor: float) -> 
 class RotaryEncoding(PositionEncoding):
     """Half-split rotary encoding: the pair ``(i, i + D/2)`` of every query and key head is
     turned by the angle of the token's position (layers.py:214-222, 298-302).  The rotation is
-    computed in 32-bit from 32-bit tables and rounded once.  Tables grow by doubling, driven
-    by the host-known largest position of a step (layers.py:272-288).  It has no weights, so
-    layers with the same constants share one instance and one pair of tables."""
+    computed in 32-bit from 32-bit tables and rounded once.  It has no weights, so layers with
+    the same constants share one instance and one pair of tables.
+
+    The tables are made once, at the first step, for ``max_positions`` (the model's
+    ``max_position_embeddings``) or ``initial_positions`` when given; a step that reaches
+    further makes them grow by doubling, driven by the host-known largest position
+    (layers.py:272-288).  A recorded step (a HIP graph) holds the addresses of the tables it was
+    recorded with, so tables that growth has superseded are kept, never freed: they cover every
+    position such a recording can bring, because the recording's widest context was inside them
+    when it was made."""
 
     shareable = True
 
@@ -41,6 +48,7 @@ class RotaryEncoding(PositionEncoding):
         theta: float,
         scaling_factor: float = 1.0,
         max_positions: int = 2048,
+        initial_positions: int | None = None,
     ) -> None:
         super().__init__(prefix, runtime)
         if head_dim % 2 != 0:
@@ -51,14 +59,21 @@ class RotaryEncoding(PositionEncoding):
         self.cos: torch.Tensor | None = None
         self.sin: torch.Tensor | None = None
         self.capacity = 0
-        #: First table size; the tables themselves are made at the first step (layers.py:265).
-        self.initial_capacity = min(int(max_positions), 1024)
+        #: First table size; the tables themselves are made at the first step.  The reference
+        #: starts at ``min(max_positions, 1024)`` (layers.py:265); here the whole of
+        #: ``max_positions`` is made at once (7B: 32,768 x 64 x 4 bytes x 2 = 16.8 MB), so that
+        #: growth is the exception.
+        self.initial_capacity = int(max_positions if initial_positions is None else initial_positions)
+        #: Tables that growth has replaced; recorded steps may still read them.
+        self.superseded: list[tuple[torch.Tensor, torch.Tensor]] = []
 
     def ensure_capacity(self, num_positions: int) -> None:
         if num_positions <= self.capacity:
             return
         target = max(num_positions, 2 * self.capacity, self.initial_capacity, 16)
         cos, sin = rotary_tables(target, self.head_dim, self.theta, self.scaling_factor)
+        if self.cos is not None:
+            self.superseded.append((self.cos, self.sin))
         self.cos = cos.to(self.runtime.device)
         self.sin = sin.to(self.runtime.device)
         self.capacity = target

@@ -25,6 +25,12 @@ class InvalidPageError(PageAllocatorError):
 
 
 class PageAllocator:
+    """Pages ``0 .. num_pages - 1``.  Only pages in use cost host memory: pages never handed out
+    yet are a range (``_fresh .. num_pages - 1``, which a list of free ids would begin with
+    anyway), pages given back wait behind them in a queue, and reference counts are kept for
+    pages in use only.  A pool that fills a large device with a small model's pages is millions
+    of pages long."""
+
     def __init__(self, num_pages: int, page_size: int) -> None:
         if num_pages < 0:
             raise ValueError(f"num_pages must be non-negative, got {num_pages}")
@@ -32,26 +38,31 @@ class PageAllocator:
             raise ValueError(f"page_size must be positive, got {page_size}")
         self.num_pages = num_pages
         self.page_size = page_size
-        self._refs = [0] * num_pages
-        self._free: deque[int] = deque(range(num_pages))
+        self._refs: dict[int, int] = {}  # page -> count, pages in use only
+        self._fresh = 0  # pages from here on have never been handed out
+        self._returned: deque[int] = deque()  # pages given back, oldest first
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return self.num_pages - len(self._refs)
 
     @property
     def num_in_use(self) -> int:
-        return self.num_pages - len(self._free)
+        return len(self._refs)
 
     def refcount(self, page: int) -> int:
         self._check_id(page)
-        return self._refs[page]
+        return self._refs.get(page, 0)
 
     def allocate(self) -> int:
-        """One page with a reference count of 1."""
-        if not self._free:
+        """One page with a reference count of 1: the page that has been free longest."""
+        if self._fresh < self.num_pages:
+            page = self._fresh
+            self._fresh += 1
+        elif self._returned:
+            page = self._returned.popleft()
+        else:
             raise OutOfPagesError(f"no free cache page: {self.num_in_use}/{self.num_pages} in use")
-        page = self._free.popleft()
         self._refs[page] = 1
         return page
 
@@ -59,15 +70,15 @@ class PageAllocator:
         """``count`` pages or none at all (kv_cache.py:211-228)."""
         if count < 0:
             raise ValueError(f"count must be non-negative, got {count}")
-        if count > len(self._free):
+        if count > self.num_free:
             raise OutOfPagesError(
-                f"cannot allocate {count} pages: {len(self._free)} free, {self.num_in_use}/{self.num_pages} in use"
+                f"cannot allocate {count} pages: {self.num_free} free, {self.num_in_use}/{self.num_pages} in use"
             )
         return [self.allocate() for _ in range(count)]
 
     def incref(self, page: int) -> int:
         self._check_id(page)
-        if self._refs[page] == 0:
+        if page not in self._refs:
             raise InvalidPageError(f"cannot share page {page}: it is free")
         self._refs[page] += 1
         return self._refs[page]
@@ -75,36 +86,48 @@ class PageAllocator:
     def decref(self, page: int) -> int:
         """Drop one reference; at zero the page goes to the back of the free list."""
         self._check_id(page)
-        if self._refs[page] == 0:
+        count = self._refs.get(page, 0)
+        if count == 0:
             raise InvalidPageError(f"double free of page {page}: it is already free")
-        self._refs[page] -= 1
-        if self._refs[page] == 0:
-            self._free.append(page)
-        return self._refs[page]
+        if count == 1:
+            del self._refs[page]
+            self._returned.append(page)
+            return 0
+        self._refs[page] = count - 1
+        return count - 1
 
     def decref_many(self, pages: Iterable[int]) -> None:
         for page in pages:
             self.decref(page)
 
     def reset(self) -> None:
-        self._refs = [0] * self.num_pages
-        self._free = deque(range(self.num_pages))
+        self._refs = {}
+        self._fresh = 0
+        self._returned = deque()
 
     def stats(self) -> dict[str, int]:
         return {"num_pages": self.num_pages, "num_free_pages": self.num_free, "num_pages_in_use": self.num_in_use}
 
     def check_invariants(self) -> None:
         """Every page is free xor referenced, and no page is on the free list twice (:316-334)."""
-        free = set(self._free)
-        if len(free) != len(self._free):
+        returned = set(self._returned)
+        if len(returned) != len(self._returned):
             raise PageAllocatorError("a page appears twice on the free list")
-        for page, count in enumerate(self._refs):
-            if count < 0:
-                raise PageAllocatorError(f"page {page} has a negative reference count")
-            if count == 0 and page not in free:
-                raise PageAllocatorError(f"page {page} is unreferenced but not free (lost)")
-            if count > 0 and page in free:
+        if not 0 <= self._fresh <= self.num_pages:
+            raise PageAllocatorError(f"{self._fresh} pages handed out of a pool of {self.num_pages}")
+        for page in returned:
+            if not 0 <= page < self._fresh:
+                raise PageAllocatorError(f"page {page} was given back but never handed out")
+            if page in self._refs:
                 raise PageAllocatorError(f"page {page} is referenced but also free")
+        for page, count in self._refs.items():
+            if not 0 <= page < self._fresh:
+                raise PageAllocatorError(f"page {page} is referenced but was never handed out")
+            if count < 1:
+                raise PageAllocatorError(f"page {page} has a reference count of {count}")
+        if len(returned) + len(self._refs) != self._fresh:
+            lost = set(range(self._fresh)) - returned - set(self._refs)
+            raise PageAllocatorError(f"pages {sorted(lost)[:8]} are unreferenced but not free (lost)")
 
     def _check_id(self, page: int) -> None:
         if not 0 <= page < self.num_pages:

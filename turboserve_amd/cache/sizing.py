@@ -19,6 +19,10 @@ from turboserve_amd.cache.manager import ceil_div
 from turboserve_amd.config.engine_config import SchedulerConfig
 
 
+#: Slots are int32 on the device: a pool holds fewer than this many token places.
+MAX_SLOTS = 2**31 - 1
+
+
 class MemoryProfileError(RuntimeError):
     """No room for a single cache page (memory.py:323-329)."""
 
@@ -40,15 +44,10 @@ class CacheSizing:
         return asdict(self)
 
 
-def activation_headroom_bytes(
-    scheduler: SchedulerConfig, *, hidden: int, intermediate: int, qkv_width: int, vocab: int, itemsize: int
-) -> int:
-    """A step's transient tensors at the token budget (memory.py:208-242): a few
-    ``[T, max(H, 2 I)]`` buffers, the fused projection output and 32-bit logits per request."""
-    tokens = scheduler.max_num_batched_tokens
-    wide = max(hidden, 2 * intermediate)
-    return tokens * 4 * wide * itemsize + tokens * hidden * 4 * 2 + tokens * qkv_width * itemsize \
-        + scheduler.max_num_seqs * vocab * 4 * 2
+def activation_headroom_bytes(model, scheduler: SchedulerConfig, itemsize: int) -> int:
+    """A step's transient tensors at the scheduler's budgets (memory.py:208-242), as the model's
+    own parts report them (``DecoderModel.activation_bytes``)."""
+    return model.activation_bytes(scheduler.max_num_batched_tokens, scheduler.max_num_seqs, itemsize)
 
 
 def window_pages_needed(window: int, scheduler: SchedulerConfig) -> int:
@@ -75,6 +74,7 @@ def size_cache(
     cap = None if max_model_len is None else ceil_div(max_model_len, page) * scheduler.max_num_seqs
 
     def clamp(group: int, count: int) -> int:
+        count = min(count, MAX_SLOTS // page)  # slots (page * page size + offset) travel as int32
         if windows[group] is not None:
             count = min(count, window_pages_needed(windows[group], scheduler))
         if cap is not None:

@@ -31,6 +31,8 @@ class CacheStorage:
     ) -> None:
         if len(num_pages) != len(layout.groups):
             raise ValueError(f"{len(num_pages)} pool sizes for {len(layout.groups)} groups")
+        if any(count * page_size > 2**31 - 1 for count in num_pages):
+            raise ValueError(f"pools of {list(num_pages)} pages of {page_size} tokens: slots would not fit 32-bit integers")
         self.layout = layout
         self.page_size = page_size
         self.num_pages = list(num_pages)

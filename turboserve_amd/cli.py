@@ -140,13 +140,9 @@ def _kv_size(args: argparse.Namespace) -> int:
             block_size=args.block_size, enable_prefix_caching=args.prefix_caching,
         ),
     )
-    model_config, model = describe_model(read_config_json(config.model))
+    _, model = describe_model(read_config_json(config.model))
     itemsize = 2 if config.resolved_dtype() == "bfloat16" else 4
-    activation = activation_headroom_bytes(
-        config.scheduler, hidden=model_config.hidden_size, intermediate=model_config.intermediate_size,
-        qkv_width=model_config.q_proj_size + 2 * model_config.kv_proj_size, vocab=model_config.vocab_size,
-        itemsize=itemsize,
-    )
+    activation = activation_headroom_bytes(model, config.scheduler, itemsize)
     if not torch.cuda.is_available():
         print("no GPU is visible: the sizing needs the device's memory", file=sys.stderr)
         return 1

@@ -3,8 +3,8 @@
 A step that brings one token for each of its requests launches a few hundred small kernels;
 at a batch of one the launches, not the GPU, set the pace.  Such a step is therefore recorded
 once per shape as a HIP graph (``torch.cuda.CUDAGraph``) over static buffers and replayed:
-per step the host fills one pinned int32 buffer (tokens, positions, slots, block tables,
-context lengths), copies it to the device and launches the graph.
+per step the host fills one pinned int32 buffer (the packed step of ``engine.batch``, in the
+shape's layout), copies it to the device and launches the graph.
 
 Shapes are bucketed so that few graphs serve every batch: the number of requests is rounded up
 to a power of two (the extra rows are padding: position 0, context 1, no cache write, results
@@ -20,11 +20,9 @@ from __future__ import annotations
 
 from collections.abc import Sequence
 
-import numpy as np
 import torch
 
-from turboserve_amd.cache.page_table import table_array
-from turboserve_amd.engine.batch import StepContext, StepEntry
+from turboserve_amd.engine.batch import StepContext, StepEntry, StepLayout, StepLimits, check_packed, context_views, pack_step
 
 
 def next_power_of_two(n: int) -> int:
@@ -37,24 +35,26 @@ class _Graph:
     def __init__(self, batch: int, widths: tuple[int, ...]) -> None:
         self.batch = batch
         self.widths = widths
+        self.layout = StepLayout.make(batch, batch, batch, widths)
         self.graph: torch.cuda.CUDAGraph | None = None
         self.device_ints: torch.Tensor | None = None
         self.host_ints: list[torch.Tensor] = []
         self.turn = 0
         self.ctx: StepContext | None = None
         self.logits: torch.Tensor | None = None
-        self.offsets: dict[str, tuple[int, int]] = {}
 
 
 class DecodeGraphs:
     def __init__(self, model, views, *, page_size: int, num_groups: int, pad_state_slot: int,
-                 max_batch: int = 128) -> None:
+                 max_batch: int = 128, limits: StepLimits | None = None) -> None:
         self.model = model
         self.views = views
         self.page_size = page_size
         self.num_groups = num_groups
         self.pad_state_slot = pad_state_slot
         self.max_batch = max_batch
+        #: What every replayed step's page ids, slots and token ids are checked against.
+        self.limits = limits
         self.device = model.runtime.device
         self._graphs: dict[tuple, _Graph] = {}
         self._pool = None
@@ -74,50 +74,17 @@ class DecodeGraphs:
 
     # -- buffers ---------------------------------------------------------------------------------
 
-    def _layout(self, batch: int, widths: tuple[int, ...]) -> tuple[dict[str, tuple[int, int]], int]:
-        """Offsets (start, length) of every field in the packed int32 buffer."""
-        offsets: dict[str, tuple[int, int]] = {}
-        cursor = 0
-
-        def take(name: str, length: int) -> None:
-            nonlocal cursor
-            offsets[name] = (cursor, length)
-            cursor += -(-length // 4) * 4  # keep every field 16-byte aligned
-
-        for name in ("token_ids", "positions", "token_seq", "context_lens", "state_slots", "logit_rows", "patch"):
-            take(name, batch)
-        take("query_start_loc", batch + 1)
-        take("max_context", 1)
-        for g, width in enumerate(widths):
-            take(f"slots{g}", batch)
-            take(f"table{g}", batch * width)
-        return offsets, cursor
-
     def _build(self, key: tuple) -> _Graph:
         batch, widths = key
         shape = _Graph(batch, widths)
-        shape.offsets, total = self._layout(batch, widths)
+        total = shape.layout.total
         shape.device_ints = torch.zeros(total, dtype=torch.int32, device=self.device)
         shape.host_ints = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]
-
-        def view(name: str) -> torch.Tensor:
-            start, length = shape.offsets[name]
-            return shape.device_ints[start:start + length]
-
         max_context = max(widths) * self.page_size
         shape.ctx = StepContext(
             num_tokens=batch,
             num_seqs=batch,
-            token_ids=view("token_ids"),
-            positions=view("positions"),
-            token_seq=view("token_seq"),
-            query_start_loc=view("query_start_loc"),
-            context_lens=view("context_lens"),
-            state_slots=view("state_slots"),
-            logit_rows=view("logit_rows"),
-            prefill_blocks=torch.zeros((0, 2), dtype=torch.int32, device=self.device),
-            slot_mapping=[view(f"slots{g}") for g in range(self.num_groups)],
-            block_tables=[view(f"table{g}").view(batch, widths[g]) for g in range(self.num_groups)],
+            **context_views(shape.layout, shape.device_ints),
             query_lens=[1] * batch,
             context_lens_host=[max_context] * batch,
             max_query_len=1,
@@ -128,7 +95,7 @@ class DecodeGraphs:
             num_prefill_tokens=0,
             max_prefill_context_len=0,
             max_decode_context_len=max_context,
-            max_decode_context_dev=view("max_context"),
+            recorded=True,
         )
         # Harmless contents for the eager warm-up and the recording: every row is padding.
         shape.device_ints.copy_(self._fill(shape, []))
@@ -151,61 +118,36 @@ class DecodeGraphs:
             self._pool = shape.graph.pool()
         return shape
 
-    def _fill(self, shape: _Graph, entries: Sequence[StepEntry], patch: dict[int, int] | None = None) -> torch.Tensor:
-        """Write a step into the next pinned buffer; rows beyond the entries are padding.
-        ``patch[i] = j``: entry ``i`` takes its token from element ``j`` of a device tensor."""
+    def _fill(self, shape: _Graph, entries: Sequence[StepEntry], patch: dict[int, int] | None = None,
+              check: bool = False) -> torch.Tensor:
+        """Write a step into the next pinned buffer (the packer of every step, ``pack_step``);
+        rows beyond the entries are padding.  ``patch[i] = j``: entry ``i`` takes its token from
+        element ``j`` of a device tensor."""
         shape.turn ^= 1
         host = shape.host_ints[shape.turn]
         data = host.numpy()
-        batch, live = shape.batch, len(entries)
-
-        def field(name: str) -> np.ndarray:
-            start, length = shape.offsets[name]
-            return data[start:start + length]
-
-        field("token_ids")[:live] = [e.tokens[0] for e in entries]
-        field("token_ids")[live:] = 0
-        field("patch")[:] = -1
-        if patch:
-            field("patch")[list(patch)] = list(patch.values())
-        field("positions")[:live] = [e.start for e in entries]
-        field("positions")[live:] = 0
-        field("token_seq")[:] = np.arange(batch, dtype=np.int32)
-        field("context_lens")[:live] = [e.start + 1 for e in entries]
-        field("context_lens")[live:] = 1
-        field("state_slots")[:live] = [e.state_slot for e in entries]
-        field("state_slots")[live:] = self.pad_state_slot
-        field("logit_rows")[:] = np.arange(batch, dtype=np.int32)
-        field("query_start_loc")[:] = np.arange(batch + 1, dtype=np.int32)
-        field("max_context")[0] = max((e.start + 1 for e in entries), default=1)
-        for g, width in enumerate(shape.widths):
-            slots = field(f"slots{g}")
-            slots[:live] = [e.slots[g][0] for e in entries]
-            slots[live:] = -1  # padding writes nothing
-            table = field(f"table{g}").reshape(batch, width)
-            table[:] = 0  # padding (and the unused tail of a row) points at page 0: never read past the context
-            for i, e in enumerate(entries):
-                row = table_array(e.tables[g])
-                table[i, : row.size] = row
+        pack_step(data, shape.layout, entries, range(shape.batch), pad_state_slot=self.pad_state_slot, token_sources=patch)
+        if check and self.limits is not None:
+            check_packed(data, shape.layout, entries, self.page_size, self.limits)
         return host
 
     # -- the step --------------------------------------------------------------------------------
 
-    def run(self, entries: Sequence[StepEntry], *, tokens_from: tuple[torch.Tensor, dict[int, int]] | None = None
-            ) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], *, tokens_from: tuple[torch.Tensor, dict[int, int]] | None = None,
+            check: bool = True) -> torch.Tensor:
         """Replay the graph of the entries' shape; returns the graph's own 32-bit logits buffer
         ``[len(entries), V]`` (overwritten by the next replay of that shape).  ``tokens_from =
         (source, {entry index: element of source})``: those entries' token ids are not known on
-        the host yet and are copied on the device from ``source`` (int32) before the replay."""
+        the host yet and are copied on the device from ``source`` (int32) before the replay.
+        With ``check`` the packed step is validated before it is copied to the device."""
         key = self._key(entries)
         shape = self._graphs.get(key)
         if shape is None:
             shape = self._graphs[key] = self._build(key)
-        host = self._fill(shape, entries, tokens_from[1] if tokens_from else None)
+        host = self._fill(shape, entries, tokens_from[1] if tokens_from else None, check=check)
         shape.device_ints.copy_(host, non_blocking=True)
         if tokens_from and tokens_from[1]:
-            start, length = shape.offsets["patch"]
-            self.model.runtime.ops.patch_tokens(shape.ctx.token_ids, shape.device_ints[start:start + length], tokens_from[0])
+            self.model.runtime.ops.patch_tokens(shape.ctx.token_ids, shape.ctx.token_source, tokens_from[0])
         shape.graph.replay()
         self.num_replays += 1
         return shape.logits[: len(entries)]

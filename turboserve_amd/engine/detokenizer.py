@@ -32,6 +32,18 @@ class TokenizerFile:
         from tokenizers import Tokenizer
 
         self._tok = Tokenizer.from_file(str(path))
+        #: The id of the end-of-sequence token that ``tokenizer_config.json`` beside the file
+        #: names (``"eos_token"``: a string, or a mapping with ``"content"``), or ``None``.
+        self.eos_token_id: int | None = None
+        config = Path(path).with_name("tokenizer_config.json")
+        if config.is_file():
+            import json
+
+            named = json.loads(config.read_text(encoding="utf-8")).get("eos_token")
+            if isinstance(named, dict):
+                named = named.get("content")
+            if isinstance(named, str):
+                self.eos_token_id = self._tok.token_to_id(named)
 
     def encode(self, text: str, add_special_tokens: bool = False) -> list[int]:
         return list(self._tok.encode(text, add_special_tokens=add_special_tokens).ids)

@@ -111,12 +111,8 @@ class LLMEngine:
             runtime = model.runtime
             itemsize = torch.empty((), dtype=runtime.dtype).element_size()
             activation = 0
-            if model_config is not None and sched_cfg.num_blocks is None:
-                activation = activation_headroom_bytes(
-                    sched_cfg, hidden=model_config.hidden_size, intermediate=model_config.intermediate_size,
-                    qkv_width=model_config.q_proj_size + 2 * model_config.kv_proj_size,
-                    vocab=model_config.vocab_size, itemsize=itemsize,
-                )
+            if sched_cfg.num_blocks is None:
+                activation = activation_headroom_bytes(model, sched_cfg, itemsize)
             self.sizing = size_cache(
                 layout, sched_cfg, itemsize=itemsize, activation_bytes=activation,
                 gpu_memory_utilization=config.gpu_memory_utilization, max_model_len=config.max_model_len,
@@ -167,9 +163,16 @@ class LLMEngine:
                     tuning.results_file)
 
     def _resolve_eos_token_ids(self) -> frozenset[int]:
-        """The checkpoint's end-of-sequence ids (engine.py:223-237)."""
-        ids = getattr(self.model_config, "eos_token_ids", ()) or ()
-        return frozenset(int(i) for i in ids)
+        """Every id that ends a generation: the checkpoint configuration's and the tokenizer's
+        (engine.py:223-237; the two differ for chat checkpoints, whose tokenizer ends a turn
+        with a token that ``config.json`` does not list)."""
+        ids = {int(i) for i in (getattr(self.model_config, "eos_token_ids", ()) or ())}
+        named = getattr(self.tokenizer, "eos_token_id", None)
+        if isinstance(named, int) and not isinstance(named, bool):
+            ids.add(named)
+        elif isinstance(named, (list, tuple)):
+            ids.update(int(i) for i in named)
+        return frozenset(ids)
 
     @property
     def eos_token_ids(self) -> frozenset[int]:
@@ -203,7 +206,8 @@ class LLMEngine:
         token_ids = self.encode(prompt) if isinstance(prompt, str) else [int(t) for t in prompt]
         if not token_ids:
             raise ValueError(f"request {request_id!r} has an empty prompt")
-        vocab = getattr(self.model_config, "vocab_size", None)
+        plan = getattr(self.model, "plan", None)
+        vocab = None if plan is None else plan.vocab_size
         if vocab is not None and any(not 0 <= t < vocab for t in token_ids):
             raise ValueError(f"request {request_id!r} has a token id outside the vocabulary of {vocab}")
         sampling = sampling or SamplingParams()

@@ -27,22 +27,28 @@ from turboserve_amd.engine.batch import StepEntry
 from turboserve_amd.engine.loading import build_storage, load_model
 from turboserve_amd.engine.runner import ModelRunner
 
-#: Requests' token counts are rounded up to this when the pool is sized; pages divide it.
+#: ``max_tokens`` counts every live request's tokens rounded up to this (or to the page size, if
+#: that is larger).
 TOKEN_ROUNDING = 64
-MAX_LIVE_REQUESTS = 4
+#: Requests that may be live at once unless the caller says otherwise.
+DEFAULT_MAX_LIVE = 4
 
 
 class TraceReplayer:
     def __init__(self, model_dir: str | Path, *, dtype: str, max_tokens: int, page_size: int = 16,
-                 device: str = "cuda:0") -> None:
-        if TOKEN_ROUNDING % page_size != 0:
-            raise ValueError(f"page_size {page_size} does not divide {TOKEN_ROUNDING}")
+                 max_live: int = DEFAULT_MAX_LIVE, device: str = "cuda:0") -> None:
+        if page_size < 1 or page_size & (page_size - 1):
+            raise ValueError(f"page_size must be a power of two, got {page_size}")
         if max_tokens < 1:
             raise ValueError("--max-tokens must be positive")
+        if max_live < 1:
+            raise ValueError("--max-live must be positive")
         self.config, self.model, self.report = load_model(model_dir, dtype=dtype, device=device)
-        num_pages = -(-max_tokens // TOKEN_ROUNDING) * (TOKEN_ROUNDING // page_size)
-        self.storage = build_storage(self.model, num_pages, page_size, MAX_LIVE_REQUESTS)
-        self.manager = CacheManager(self.storage.layout.windows(), num_pages, page_size, MAX_LIVE_REQUESTS)
+        rounding = max(TOKEN_ROUNDING, page_size)
+        num_pages = -(-max_tokens // rounding) * (rounding // page_size)
+        self.max_live = max_live
+        self.storage = build_storage(self.model, num_pages, page_size, max_live)
+        self.manager = CacheManager(self.storage.layout.windows(), num_pages, page_size, max_live)
         self.runner = ModelRunner(self.model, self.storage)
 
     def run_step(self, record: dict[str, Any]):
@@ -91,8 +97,11 @@ def main(argv: list[str] | None = None) -> int:
     parser.add_argument("--out", required=True, help="folder the <step>.f32 files are written to")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at once (each rounded up to 64); sizes the page pool")
-    parser.add_argument("--page-size", type=int, default=16, help="tokens per cache page (divides 64)")
+    parser.add_argument("--page-size", type=int, default=16,
+                        help="tokens per cache page, a power of two; above 64, --max-tokens counts in pages")
+    parser.add_argument("--max-live", type=int, default=DEFAULT_MAX_LIVE, help="most requests live at once")
     args = parser.parse_args(argv)
-    replayer = TraceReplayer(args.model, dtype=args.dtype, max_tokens=args.max_tokens, page_size=args.page_size)
+    replayer = TraceReplayer(args.model, dtype=args.dtype, max_tokens=args.max_tokens, page_size=args.page_size,
+                             max_live=args.max_live)
     replayer.replay(sys.stdin, args.out)
     return 0

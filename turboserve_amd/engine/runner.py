@@ -16,7 +16,7 @@ import torch
 
 from turboserve_amd.cache.layout import CacheLayout
 from turboserve_amd.cache.storage import CacheStorage
-from turboserve_amd.engine.batch import StepContext, StepEntry, build_context, validate_entries
+from turboserve_amd.engine.batch import StepContext, StepEntry, StepLimits, build_context, validate_entries
 from turboserve_amd.engine.decode_graph import DecodeGraphs
 from turboserve_amd.models.decoder import DecoderModel
 
@@ -31,13 +31,18 @@ class ModelRunner:
         self.views = storage.views()
         self.vocab_size = model.plan.vocab_size
         self.num_steps = 0
+        #: What a checked step's page ids, slots, token ids and state slots must lie inside.
+        self.limits = StepLimits(
+            num_pages=tuple(storage.num_pages), windows=tuple(self.layout.windows()),
+            vocab_size=self.vocab_size, num_state_slots=storage.num_state_slots,
+        )
         #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``), unless a part
         #: of the model says it cannot be recorded (``Part.capturable``).
         self.graphs: DecodeGraphs | None = None
         if use_graphs and model.is_capturable():
             self.graphs = DecodeGraphs(
                 model, self.views, page_size=storage.page_size, num_groups=len(self.layout.groups),
-                pad_state_slot=storage.pad_state_slot, max_batch=max_graph_batch,
+                pad_state_slot=storage.pad_state_slot, max_batch=max_graph_batch, limits=self.limits,
             )
 
     def release(self) -> None:
@@ -48,26 +53,17 @@ class ModelRunner:
             self.graphs.release()
             self.graphs = None
 
-    def check_tokens(self, entries: Sequence[StepEntry], unknown: Sequence[int] = ()) -> None:
-        """Every token id is inside the vocabulary; ``unknown``: indices of entries whose token
-        is still on the device (see ``step``)."""
-        vocab = self.vocab_size
-        for index, entry in enumerate(entries):
-            if index in unknown:
-                continue
-            for token in entry.tokens:
-                if not 0 <= token < vocab:
-                    raise ValueError(f"request {entry.request!r}: token id {token} is outside the vocabulary of {vocab}")
-
     def context_for(self, entries: Sequence[StepEntry]) -> StepContext:
-        if self.check:
-            self.check_tokens(entries)
+        """The packed step on the device.  With ``check`` (always, except in measurements)
+        nothing a kernel would dereference leaves the host unchecked: token ids, page ids,
+        slots and state slots are validated against the vocabulary and the pools first."""
         return build_context(
             entries,
             num_groups=len(self.layout.groups),
             page_size=self.storage.page_size,
             device=self.model.runtime.device,
             check=self.check,
+            limits=self.limits,
         )
 
     @torch.inference_mode()
@@ -121,9 +117,8 @@ class ModelRunner:
         """A step of single tokens through its recorded graph.  The result is the graph's own
         buffer (or rows gathered from it): read it before the next step."""
         if self.check:
-            self.check_tokens(entries, tokens_from[1] if tokens_from else ())
             validate_entries(entries, len(self.layout.groups), self.storage.page_size)
-        logits = self.graphs.run(entries, tokens_from=tokens_from)
+        logits = self.graphs.run(entries, tokens_from=tokens_from, check=self.check)
         self.num_steps += 1
         wanted = [i for i, entry in enumerate(entries) if len(entry.want) > 0]
         if len(wanted) == len(entries):

@@ -7,7 +7,6 @@ the library cannot be built or loaded, or a tensor is not on a GPU, the op raise
 from __future__ import annotations
 
 import ctypes
-import os
 from ctypes import c_float, c_int, c_long, c_void_p
 
 import torch
@@ -133,6 +132,19 @@ def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtyp
           "value pages must be [NB, Hkv, D, BS] for key pages [NB, Hkv, BS, D]")
 
 
+def prefill_block_list(query_lens, context_lens, rows: int) -> list[list[int]]:
+    """``[request index, first row]`` of every block of ``rows`` consecutive rows of requests that
+    bring ``query_lens`` tokens and hold ``context_lens`` afterwards, rows numbered through the
+    requests in order; blocks whose last row sees the most keys come first."""
+    blocks, first_row = [], 0
+    for index, (count, context) in enumerate(zip(query_lens, context_lens)):
+        for offset in range(0, count, rows):
+            blocks.append((context - count + min(offset + rows, count), index, first_row + offset))
+        first_row += count
+    blocks.sort(key=lambda b: -b[0])
+    return [[block[1], block[2]] for block in blocks]
+
+
 class Ops:
     """The kernel library bound to one device."""
 
@@ -146,6 +158,13 @@ class Ops:
         for module in modules:
             load_module(module)
         self._tiled_plans: dict[tuple, tuple[int, int, int]] = {}  # (m, n, k, max_splits) -> grid of the tiled product
+        #: Compute units of the device (256 on an MI355X): the launch plans below size their grids by it.
+        self.compute_units = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
+        #: Wavefronts a decode attention launch aims for: one per SIMD, four SIMDs a compute unit
+        #: (each keeps two windows of loads in flight).
+        self.decode_target_waves = 4 * self.compute_units
+        #: Wavefronts (16 weight rows x one range of K each) the resident product aims for: 16 per compute unit.
+        self.skinny_resident_waves = 16 * self.compute_units
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -415,6 +434,18 @@ class Ops:
                   requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
                   _ptr(max_context_dev), self.stream()), "ts_attention_decode")
 
+    #: Rows of one request that a wavefront of the prefill attention kernel handles.
+    prefill_block_rows = 16
+
+    def prefill_blocks(self, query_lens, context_lens) -> torch.Tensor:
+        """The work list of :meth:`attention_prefill` for the multi-token requests at the front
+        of a step (their numbers of new tokens and their contexts after the step): int32
+        ``[n, 2]`` on the device, (request index, first row) of every block of
+        ``prefill_block_rows`` rows, those that see the most keys first, so the long ones start
+        early and the short ones fill the tail of the launch."""
+        blocks = prefill_block_list(query_lens, context_lens, self.prefill_block_rows)
+        return torch.tensor(blocks, dtype=torch.int32).view(-1, 2).to(self.device)
+
     def attention_prefill(
         self,
         out: torch.Tensor,
@@ -455,8 +486,6 @@ class Ops:
                   heads, kv_heads, block_size, float(scale), int(window or 0), self.stream()),
                "ts_attention_prefill")
 
-    #: Wavefronts a decode attention launch aims for (one per SIMD of a 256-CU device; each keeps two windows of loads in flight).
-    decode_target_waves = 1024
     #: Fewest keys worth a wavefront of its own.
     decode_min_keys = 128
 
@@ -488,17 +517,15 @@ class Ops:
         return y
 
     #: Most ranges of K the resident product is split into (its consumer adds them up).
-    skinny_max_splits = int(os.environ.get("TS_SKINNY_MAXS", "8"))
+    skinny_max_splits = 8
     #: Largest batch the weight-streaming products serve; above it the BLAS library is used.
     skinny_max_rows = 128
     #: Most rows the resident product takes (a split's activations stay in LDS).
     skinny_resident_rows = 16
-    #: Wavefronts (16 weight rows x one range of K each) the resident variant aims for: 16 per compute unit.
-    skinny_resident_waves = int(os.environ.get("TS_SKINNY_RW", "4096"))
     #: Wavefronts per workgroup of the resident variant (4 or 8); 0 chooses by the grid's size.
-    skinny_resident_wg = int(os.environ.get("TS_SKINNY_RWG", "0"))
+    skinny_resident_wg = 0
     #: Chunks of 256 staged in LDS at a time for up to 8 rows and for up to 16 rows (even numbers).
-    skinny_stage_chunks = tuple(int(v) for v in os.environ.get("TS_SKINNY_STAGE", "10,4").split(","))
+    skinny_stage_chunks = (10, 4)
 
     @staticmethod
     def skinny_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -513,18 +540,16 @@ class Ops:
         want = max(1, min(limit, -(-self.skinny_resident_waves // -(-n // 16))))
         per_split = -(-chunks // want)
         splits = -(-chunks // per_split)
-        waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 1024) else 4)
+        waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 4 * self.compute_units) else 4)
         return per_split, splits, waves, self.skinny_stage_chunks[0 if m <= 8 else 1]
 
-    #: Compute units the tiled product sizes its grid for.
-    tiled_compute_units = int(os.environ.get("TS_TILED_CUS", "256"))
     #: Up to this many rows a product of a wide matrix (at least 200 tiles of 160 rows) stays with
     #: the resident-activation kernel, which is a little faster there; everything else up to 128
     #: rows runs the tiled kernel.
-    resident_wide_rows = int(os.environ.get("TS_RESIDENT_WIDE_ROWS", "4"))
+    resident_wide_rows = 4
     #: Matrices smaller than this many bytes stay with the resident kernel up to 16 rows: the product
     #: lasts a few microseconds and the resident kernel's many small workgroups start faster.
-    resident_small_bytes = int(os.environ.get("TS_RESIDENT_SMALL_BYTES", str(64 << 20)))
+    resident_small_bytes = 64 << 20
 
     def _tiled_plan(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int]:
         """(iterations of 128 per split, splits, tile) of the tiled product.  The cost of a
@@ -547,13 +572,13 @@ class Ops:
                 splits = -(-iters // per_split)
                 if splits != want:
                     continue  # the same grid as a smaller `want`
-                groups = -(-tiles * splits // self.tiled_compute_units)
+                groups = -(-tiles * splits // self.compute_units)
                 cost = groups * rows * (per_split + 1)
                 cost *= 1.0 + 2.0 * splits * m / k  # partial sums written here and read by the consumer
                 cost *= 1.0 + 0.12 * m / rows       # activations a workgroup stages, relative to its weights
                 if tile == 2:
                     cost *= 0.95                    # two workgroups share a compute unit and fill each other's waits
-                resident = self.tiled_compute_units * (2 if tile == 2 else 1)
+                resident = self.compute_units * (2 if tile == 2 else 1)
                 cost *= 1.0 + 0.1 * (-(-tiles * splits // resident) - 1)  # later rounds start on a busy device, unevenly
                 if best is None or cost < best[0] * 0.999:
                     best = (cost, per_split, splits, tile)

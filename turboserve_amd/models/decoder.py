@@ -118,6 +118,19 @@ class DecoderModel:
             total += count
         return total
 
+    def activation_bytes(self, tokens: int, requests: int, itemsize: int) -> int:
+        """Room a step of ``tokens`` rows that wants logits for ``requests`` of them takes beside
+        weights and cache: the 32-bit residual stream and the output waiting to be added to it,
+        the neediest layer (norm output plus its largest part), twice over because the caching
+        allocator keeps freed blocks of other sizes, and the 32-bit logits with the sampler's
+        working copy (the reference's estimate has the same terms from Qwen2's sizes,
+        src/turboserve/engine/runtime/memory.py:208-242)."""
+        plan = self.plan
+        stream = tokens * plan.hidden_size * (4 + 4)
+        layer = max((block.activation_bytes(tokens, itemsize) for block in self.blocks), default=0)
+        layer += self.final_norm.activation_bytes(tokens, itemsize)
+        return 2 * (stream + layer) + requests * plan.vocab_size * 4 * 2
+
     # -- caches -------------------------------------------------------------------------------
 
     def is_capturable(self) -> bool:

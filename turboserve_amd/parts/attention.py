@@ -61,6 +61,10 @@ class GroupedQueryAttention(Mixer):
     def is_capturable(self) -> bool:
         return self.capturable and self.position.is_capturable()
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """The fused projection, the attention output and the output projection of a step."""
+        return tokens * (self.q_size + 2 * self.kv_size + self.q_size + self.hidden_size) * itemsize
+
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs = {
             self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden_size)),
@@ -112,9 +116,12 @@ class GroupedQueryAttention(Mixer):
         if fast:
             out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
             if ctx.num_prefill_seqs > 0:
+                # The launch's list of row blocks is the same for every layer of the step.
+                blocks = ctx.derive("attention_prefill_blocks", lambda step: ops.prefill_blocks(
+                    step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs]))
                 ops.attention_prefill(
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
-                    ctx.prefill_blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len,
+                    blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len,
                 )
             if ctx.num_decode_seqs > 0:
                 ops.attention_decode(

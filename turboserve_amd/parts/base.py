@@ -158,6 +158,12 @@ class Part:
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:  # pragma: no cover - default
         return None
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """Bytes of the transient tensors this part holds at once in a step of ``tokens`` rows
+        (``itemsize``: bytes of a run-dtype element).  The engine sums these over the model to
+        leave room beside the cache pages; a part that makes nothing large may say 0."""
+        return 0
+
 
 class Norm(Part):
     """Normalisation over the last dimension."""
@@ -224,6 +230,10 @@ class Block(Part):
 
     def is_capturable(self) -> bool:
         return self.capturable and all(part.is_capturable() for part in self.parts())
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """The largest of its parts' needs: they run one after the other."""
+        return max((part.activation_bytes(tokens, itemsize) for part in self.parts()), default=0)
 
     def parts(self) -> list[Part]:
         raise NotImplementedError

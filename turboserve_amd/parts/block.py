@@ -42,6 +42,13 @@ class PreNormBlock(Block):
     def parts(self) -> list[Part]:
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """A norm's output stays alive while the part it feeds runs."""
+        return max(
+            self.mixer_norm.activation_bytes(tokens, itemsize) + self.mixer.activation_bytes(tokens, itemsize),
+            self.ff_norm.activation_bytes(tokens, itemsize) + self.feed_forward.activation_bytes(tokens, itemsize),
+        )
+
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs: dict[str, TensorSpec] = {}
         for part in self.parts():

@@ -31,6 +31,10 @@ class SwiGLU(FeedForward):
             self.name("down_proj.weight"): TensorSpec((self.hidden_size, self.intermediate_size)),
         }
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """The gate|up projection, the activated product and the down projection of a step."""
+        return tokens * (3 * self.intermediate_size + self.hidden_size) * itemsize
+
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         gate, up = tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]
         self.gate_up_weight = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()

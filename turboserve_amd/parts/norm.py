@@ -25,6 +25,9 @@ class RMSNorm(Norm):
     def tensor_specs(self) -> dict[str, TensorSpec]:
         return {self.name("weight"): TensorSpec((self.size,), init="ones")}
 
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        return tokens * self.size * itemsize
+
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name("weight")].contiguous()
 

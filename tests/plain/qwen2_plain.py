@@ -3,7 +3,7 @@
 This file is the oracle of the test suite. It shares no code with ``turboserve_amd``: it reads
 a raw ``config.json`` mapping and a ``{tensor name: tensor}`` mapping (Hugging Face names) and
 computes with ordinary torch tensor arithmetic on the CPU.  Every function cites the lines of
-the reference (``/root/reference``) whose formula it restates.
+the reference (paths under its ``src/turboserve/`` and ``tests/``) whose formula it restates.
 
 Conventions: ``T`` tokens of ONE sequence at positions ``0..T-1`` unless ``positions`` says
 otherwise; ``H`` hidden size; ``Hq``/``Hkv`` query/KV heads; ``D`` head size.

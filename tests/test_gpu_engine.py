@@ -35,8 +35,27 @@ def model(request, tmp_path_factory):
     wide = tiny.make_model_dir(tmp_path_factory.mktemp(f"engine{request.param}_wide"), config, seed + 1, torch.float32,
                                std=tiny.WIDE_STD)
     wide_raw, wide_tensors = tiny.read_model_dir(wide)
+    # And one stored in bfloat16 (a spread that keeps the rounding error inside the bounds), so
+    # that the plain implementation computes with the very numbers the bfloat16 engine holds.
+    half = tiny.make_model_dir(tmp_path_factory.mktemp(f"engine{request.param}_bf16"), config, seed + 2, torch.bfloat16,
+                               std=tiny.std_for(torch.bfloat16, config["hidden_size"]))
+    half_raw, half_tensors = tiny.read_model_dir(half)
     return {"name": request.param, "folder": folder, "page": page, "raw": raw, "tensors": tensors, "prompts": prompts,
-            "vocab": config["vocab_size"], "wide_folder": wide, "wide_raw": wide_raw, "wide_tensors": wide_tensors}
+            "vocab": config["vocab_size"], "wide_folder": wide, "wide_raw": wide_raw, "wide_tensors": wide_tensors,
+            "bf16_folder": half, "bf16_raw": half_raw, "bf16_tensors": half_tensors}
+
+
+def check_logprobs(logits: torch.Tensor, output) -> None:
+    """A bfloat16 engine's greedy tokens and their log-probabilities against the plain
+    implementation's 32-bit logits for the same sequence (``logits[i]``: the row that chose token
+    ``i``): each token is the argmax up to the rounding bound of the logits (2% of the row's
+    largest, see ``test_gpu_replay``), and its log-probability, a difference of two such
+    numbers, is off by at most twice that."""
+    assert len(output.new_token_ids) == len(output.logprobs) > 0
+    for row, token, got in zip(logits, output.new_token_ids, output.logprobs):
+        bound = 2e-2 * float(row.abs().max())
+        assert float(row.max() - row[token]) <= bound, f"token {token} is not a near-argmax"
+        assert abs(got - plain.log_softmax_at(row, token)) <= 2 * bound, (token, got, plain.log_softmax_at(row, token))
 
 
 def test_greedy_generation_equals_plain(model):
@@ -251,7 +270,7 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
 
     def engine_with_tuning(results):
         return LLMEngine(EngineConfig(
-            model=str(model["folder"]), dtype="bfloat16", tune_gemm_tokens=(200,), gemm_tuning_file=str(results),
+            model=str(model["bf16_folder"]), dtype="bfloat16", tune_gemm_tokens=(200,), gemm_tuning_file=str(results),
             scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=256, block_size=model["page"], num_blocks=64),
         ))
 
@@ -269,10 +288,8 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
         engine.close()
         torch.cuda.tunable.enable(False)
     sequence = prompt + out.new_token_ids
-    logits = plain.forward_logits(model["raw"], plain.as_float32(model["tensors"]), sequence)
-    for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
-        want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
-        assert abs(got - want) <= 0.05, (i, got, want)
+    logits = plain.forward_logits(model["bf16_raw"], model["bf16_tensors"], sequence)
+    check_logprobs(logits[len(prompt) - 1:], out)
     # With the size limit lifted the same start-up times them and keeps its choices.
     monkeypatch.setattr(Ops, "library_tuning_min_work", 0)
     results = tmp_path / "choices.csv"
@@ -295,9 +312,8 @@ def test_many_requests_decode_together(model, count):
 
     prompts = [tiny.random_tokens(model["vocab"], 3 + i % 9, 300 + i) for i in range(count)]
     sampling = SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True, logprobs=True)
-    weights = plain.as_float32(model["tensors"])
     engine = LLMEngine(EngineConfig(
-        model=str(model["folder"]), dtype="bfloat16",
+        model=str(model["bf16_folder"]), dtype="bfloat16",
         scheduler=SchedulerConfig(max_num_seqs=128, max_num_batched_tokens=2048, block_size=model["page"], num_blocks=512),
     ))
     try:
@@ -307,10 +323,7 @@ def test_many_requests_decode_together(model, count):
         engine.close()
     for prompt, out in zip(prompts, outs):
         sequence = prompt + out.new_token_ids
-        logits = plain.forward_logits(model["raw"], weights, sequence)
-        for i, (token, got) in enumerate(zip(out.new_token_ids, out.logprobs)):
-            want = plain.log_softmax_at(logits[len(prompt) - 1 + i], token)
-            assert abs(got - want) <= 0.05, (i, got, want)
+        check_logprobs(plain.forward_logits(model["bf16_raw"], model["bf16_tensors"], sequence)[len(prompt) - 1:], out)
 
 
 def test_steps_launched_ahead_give_the_same_tokens(model):
@@ -352,6 +365,138 @@ def test_steps_launched_ahead_give_the_same_tokens(model):
             outputs = engine.generate(prompts, sampling)
             results.append([(o.new_token_ids, o.logprobs) for o in outputs])
     assert results[0] == results[1]
+
+
+def test_truncated_and_penalised_sampling_through_the_engine(model):
+    """top-k, top-p and the repetition penalty through ``LLMEngine`` (not only the kernel): every
+    token a request draws is the one the plain sampler draws from the plain logits of the
+    sequence so far, with the request's seed, draw number and history."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 10
+    settings = [dict(temperature=0.9, top_k=5), dict(temperature=1.1, top_p=0.6), dict(temperature=0.7, top_k=12, top_p=0.8),
+                dict(temperature=1.0, repetition_penalty=1.7), dict(temperature=0.0, repetition_penalty=2.5)]
+    prompts = [model["prompts"][i % len(model["prompts"])] for i in range(len(settings))]
+    params = [SamplingParams(max_tokens=new, seed=31 + i, ignore_eos=True, **kw) for i, kw in enumerate(settings)]
+    with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=64, run_ahead=True) as engine:
+        outputs = engine.generate(prompts, params)
+    for i, (prompt, output, kw) in enumerate(zip(prompts, outputs, settings)):
+        tokens = list(prompt)
+        assert len(output.new_token_ids) == new
+        for draw, token in enumerate(output.new_token_ids):
+            logits = plain.forward_logits(model["wide_raw"], model["wide_tensors"], tokens)[-1]
+            want, cdf = plain.sample_token(
+                logits, temperature=kw["temperature"], seed=31 + i, draw_index=draw, top_k=kw.get("top_k", 0),
+                top_p=kw.get("top_p", 1.0), penalty=kw.get("repetition_penalty", 1.0), history=tokens)
+            if token != want:  # only a uniform that falls on the edge of two tokens' intervals may differ
+                u = plain.philox_uniform(31 + i, draw)
+                low = float(cdf[token - 1]) if token > 0 else 0.0
+                assert cdf.numel() and low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"request {i} draw {draw}: {token} != {want}"
+            tokens.append(token)
+
+
+def test_prompts_are_not_cut_when_chunking_is_off(model):
+    """``enable_chunked_prefill=False``: a prompt runs whole or waits; one longer than the token
+    budget is refused at arrival (src/turboserve/engine/core/scheduler.py:530-548, 663-667)."""
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 6
+    want = [plain.greedy_generate(model["wide_raw"], model["wide_tensors"], p, new) for p in model["prompts"]]
+    budget = max(len(p) for p in model["prompts"]) + 2  # room for the longest prompt, not for two of them
+    engine = LLMEngine(EngineConfig(model=str(model["wide_folder"]), dtype="float32", scheduler=SchedulerConfig(
+        max_num_seqs=8, max_num_batched_tokens=budget, block_size=model["page"], num_blocks=64, enable_chunked_prefill=False)))
+    with engine:
+        seen = []
+        original = engine.runner.step
+
+        def watched(entries, **kw):
+            seen.extend((entry.start, len(entry.tokens)) for entry in entries)
+            return original(entries, **kw)
+
+        engine.runner.step = watched
+        outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+        assert [o.new_token_ids for o in outputs] == want
+        lengths = {len(p) for p in model["prompts"]}
+        assert all(count in lengths for start, count in seen if start == 0), "a prompt was cut into portions"
+        assert all(count == 1 for start, count in seen if start > 0)
+        with pytest.raises(ValueError):
+            engine.add_request("too-long", tiny.random_tokens(model["vocab"], budget + 1, 3))
+
+
+def test_more_requests_decode_than_a_recorded_step_takes(model):
+    """150 requests decoding at once: more than the 128 rows a recorded step takes, so the step
+    runs eagerly (the decode attention without a device-side longest context)."""
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    count = 150
+    prompts = [tiny.random_tokens(model["vocab"], 2 + i % 11, 700 + i) for i in range(count)]
+    sampling = SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True, logprobs=True)
+    results = {}
+    for dtype in ("float32", "bfloat16"):
+        folder = model["wide_folder"] if dtype == "float32" else model["bf16_folder"]
+        engine = LLMEngine(EngineConfig(model=str(folder), dtype=dtype, scheduler=SchedulerConfig(
+            max_num_seqs=256, max_num_batched_tokens=4096, block_size=model["page"], num_blocks=600)))
+        with engine:
+            results[dtype] = engine.generate(prompts, sampling)
+            assert engine.runner.graphs.num_replays == 0
+    for prompt, exact, fast in zip(prompts, results["float32"], results["bfloat16"]):
+        assert exact.new_token_ids == plain.greedy_generate(model["wide_raw"], model["wide_tensors"], prompt, 3)
+        sequence = prompt + fast.new_token_ids
+        logits = plain.forward_logits(model["bf16_raw"], model["bf16_tensors"], sequence)
+        for i, token in enumerate(fast.new_token_ids):
+            row = logits[len(prompt) - 1 + i]
+            assert float(row.max() - row[token]) <= 2e-2 * float(row.abs().max()), "not a near-argmax in bfloat16"
+
+
+def test_text_prompts_stop_strings_and_the_tokenizers_end_token(model, tmp_path):
+    """Text in, text out through a ``tokenizer.json`` (made here with the ``tokenizers`` library:
+    one word per token id): the prompt is encoded without special tokens, a stop string ends a
+    request and is cut from its text, and the end token that ``tokenizer_config.json`` names ends
+    a request although the model's ``config.json`` does not list it (the reference joins both,
+    src/turboserve/engine/runtime/engine.py:223-237)."""
+    import json
+    import shutil
+
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import WhitespaceSplit
+
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(model["wide_folder"], folder)
+    word = lambda token: f"w{token:04d}"  # one length for all, so no word is the start of another
+    vocab = {word(i): i for i in range(model["vocab"])}
+    tokenizer = Tokenizer(WordLevel(vocab, unk_token=word(0)))
+    tokenizer.pre_tokenizer = WhitespaceSplit()
+    tokenizer.save(str(folder / "tokenizer.json"))
+    prompt_ids = model["prompts"][-1]
+    text = " ".join(word(t) for t in prompt_ids)
+    free = plain.greedy_generate(model["wide_raw"], model["wide_tensors"], prompt_ids, 10)
+    assert len(set(free[:6])) == 6, "the continuation should not repeat a token early"
+    scheduler = SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=64, block_size=model["page"], num_blocks=64)
+    with LLMEngine(EngineConfig(model=str(folder), dtype="float32", scheduler=scheduler)) as engine:
+        assert engine.tokenizer is not None and engine.encode(text) == prompt_ids
+        plain_run = engine.generate([text], SamplingParams(max_tokens=10, temperature=0.0))[0]
+        assert plain_run.new_token_ids == free and plain_run.finish_reason == "length"
+        words = plain_run.text_delta.split()
+        assert words == [word(t) for t in free]
+        stopped = engine.generate([text], SamplingParams(max_tokens=10, temperature=0.0, stop=[word(free[3])]))[0]
+        assert stopped.finish_reason == "stop" and stopped.new_token_ids == free[:4]
+        assert stopped.text_delta.split() == [word(t) for t in free[:3]], "the stop string is cut from the text"
+    (folder / "tokenizer_config.json").write_text(json.dumps({"eos_token": {"content": word(free[4])}}))
+    with LLMEngine(EngineConfig(model=str(folder), dtype="float32", scheduler=scheduler)) as engine:
+        assert free[4] in engine.eos_token_ids
+        ended = engine.generate([text], SamplingParams(max_tokens=10, temperature=0.0))[0]
+        assert ended.finish_reason == "stop" and ended.new_token_ids == free[:5]
+        ignored = engine.generate([text], SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True))[0]
+        assert ignored.new_token_ids == free
 
 
 def test_command_line_generates_the_plain_tokens(tmp_path):

@@ -362,6 +362,64 @@ def test_toy_architecture_steps_like_its_plain_form(toy_folder, cut):
         assert float((got[rid] - want).abs().max()) <= 1e-4, f"{cut} {rid}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_generates_through_the_engine_and_the_command_line(toy_folder, tmp_path, dtype, capsys):
+    """The toy architecture (its configuration is a plain mapping with names of its own)
+    through ``LLMEngine`` with the cache sized from the device's memory, and through the command
+    line's ``generate`` and ``kv-size``: nothing in the engine, the sizing or the command line
+    reads an architecture's configuration fields."""
+    import json
+    import re
+
+    from turboserve_amd import cli
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+    from turboserve_amd.weights.random_init import write_random_model
+
+    register_toy_architecture()
+    folder = toy_folder
+    if dtype == "bfloat16":
+        # Without the routed feed-forward: a router's near-tie may fall to another expert in
+        # bfloat16, which is a different function, not a rounding error.
+        dense = {**TOY_CONFIG, "feed_forwards": ["swiglu"] * 4}
+        folder = write_random_model(dense, tmp_path / "toy_bf16", seed=5, dtype=torch.bfloat16, std=0.1)
+    raw, tensors = tiny.read_model_dir(folder)
+    prompts = [tiny.random_tokens(97, n, 40 + n) for n in (3, 12, 29)]
+    new = 6
+
+    def check_tokens(prompt, got):
+        tokens = list(prompt)
+        assert len(got) == new
+        for token in got:
+            logits = toy_plain_logits(raw, tensors, tokens)[-1]
+            slack = 0.0 if dtype == "float32" else 3e-2 * float(logits.abs().max())
+            assert float(logits.max() - logits[token]) <= slack, f"{dtype}: token {token} is not the plain argmax"
+            tokens.append(token)
+
+    config = EngineConfig(model=str(folder), dtype=dtype, max_model_len=64, scheduler=SchedulerConfig(
+        max_num_seqs=4, max_num_batched_tokens=16, block_size=8))
+    with LLMEngine(config) as engine:
+        assert engine.sizing is not None and engine.sizing.reason == "max_model_len cap"
+        assert engine.sizing.num_blocks == [32] and engine.sizing.activation_bytes > 0
+        outputs = engine.generate(prompts, SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+        for prompt, output in zip(prompts, outputs):
+            check_tokens(prompt, output.new_token_ids)
+        engine.scheduler.check_invariants()
+    capsys.readouterr()
+    args = ["engine", "generate", "--model", str(folder), "--dtype", dtype, "--max-tokens", str(new), "--ignore-eos",
+            "--num-blocks", "32", "--block-size", "8"]
+    assert cli.main(args + [a for p in prompts for a in ("--prompt-ids", ",".join(map(str, p)))]) == 0
+    shown = [json.loads(m) for m in re.findall(r"^output \d+: (\[.*\])$", capsys.readouterr().out, flags=re.M)]
+    assert len(shown) == len(prompts)
+    for prompt, got in zip(prompts, shown):
+        check_tokens(prompt, got)
+    assert cli.main(["engine", "kv-size", "--model", str(folder), "--dtype", dtype, "--max-model-len", "64", "--block-size", "8"]) == 0
+    sizing = capsys.readouterr().out
+    sizing = json.loads(sizing[sizing.index("{"):])
+    assert sizing["reason"] == "max_model_len cap" and sizing["num_blocks"] == [8 * 64] and sizing["activation_bytes"] > 0
+
+
 def test_a_part_can_keep_the_model_out_of_graphs(toy_folder):
     """A part that reads device data back on the host says `capturable = False`; the runner
     then records no HIP graph and steps the model eagerly, with the same logits."""

@@ -3,10 +3,11 @@ strings, the command line's options, the model plan as data."""
 
 from __future__ import annotations
 
+import numpy as np
 import pytest
 
 from turboserve_amd.cli import build_parser
-from turboserve_amd.engine.batch import StepEntry, build_context, validate_entries
+from turboserve_amd.engine.batch import StepEntry, StepLayout, StepLimits, build_context, check_packed, pack_step, validate_entries
 from turboserve_amd.engine.detokenizer import IncrementalDetokenizer, StopStringMatcher, StreamingDecoder
 from turboserve_amd.engine.sequence import Sequence
 from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
@@ -31,10 +32,16 @@ def test_batch_is_packed_with_multi_token_entries_first():
     assert ctx.slot_mapping[0].tolist() == [8, 9, 10, 11, 0, 6, 30]
     assert (ctx.num_prefill_seqs, ctx.num_decode_seqs, ctx.num_prefill_tokens) == (1, 2, 5)
     assert (ctx.max_query_len, ctx.max_context_len, ctx.max_decode_context_len) == (5, 7, 7)
-    assert ctx.prefill_blocks.tolist() == [[0, 0]]
-    long = build_context([entry("a", list(range(40)), 8, list(range(12))), entry("b", list(range(20)), 0, list(range(12, 17)))],
-                         num_groups=1, page_size=4, device="cpu")
-    assert long.prefill_blocks.tolist() == [[0, 32], [0, 16], [0, 0], [1, 56], [1, 40]]  # those that see most keys first
+    assert int(ctx.max_decode_context_dev[0]) == 7 and ctx.token_source.tolist() == [-1] * 7
+    # what a part derives from a step is made once and shared by its layers
+    made = []
+    assert ctx.derive("k", lambda step: made.append(step.num_tokens) or "x") == "x" and ctx.derive("k", None) == "x"
+    assert made == [7]
+    # the prefill attention's work list: blocks of 16 rows, those that see most keys first
+    from turboserve_amd.kernels.ops import prefill_block_list
+
+    assert prefill_block_list([5], [5], 16) == [[0, 0]]
+    assert prefill_block_list([40, 20], [48, 20], 16) == [[0, 32], [0, 16], [0, 0], [1, 56], [1, 40]]
 
 
 def test_batch_validation():
@@ -51,6 +58,78 @@ def test_batch_validation():
     bad.slots = [[0]]
     with pytest.raises(ValueError, match="slots for 2 tokens"):
         validate_entries([bad], 1, 4)
+
+
+def test_packed_step_is_checked_against_the_pools():
+    """What a kernel would turn into an address is refused on the host
+    (src/turboserve/engine/core/types.py:388-397, src/turboserve/engine/model/attention.py:105-112)."""
+    limits = StepLimits(num_pages=[8], windows=[None], vocab_size=50, num_state_slots=4)
+    build = lambda entries, lim=limits: build_context(entries, num_groups=1, page_size=4, device="cpu", limits=lim)
+    build([entry("ok", [1, 2, 3, 4, 5], 3, [7, 0])])
+    with pytest.raises(ValueError, match="page id 8 at index 1 .* outside the pool of 8 pages"):
+        build([entry("a", [1, 2, 3, 4, 5], 0, [2, 8])])
+    with pytest.raises(ValueError, match="page id -2"):
+        build([entry("a", [1], 0, [-2])])
+    with pytest.raises(ValueError, match="'a': no page at index 0 .* inside the keys 0..5"):
+        build([entry("a", [1, 2], 4, [-1, 3])])
+    with pytest.raises(ValueError, match="token id 50 is outside the vocabulary of 50"):
+        build([entry("a", [1, 50], 0, [2])])
+    with pytest.raises(ValueError, match="token id -1"):
+        build([entry("b", [7], 0, [2]), entry("a", [-1], 0, [3])])
+    wrong = entry("a", [1, 2, 3], 2, [5, 6])
+    wrong.slots = [[22, 23, 25]]  # position 4 lies in page 6: slot 24
+    with pytest.raises(ValueError, match="'a': slot 25 of group 0 is not where its block table puts position 4"):
+        build([wrong])
+    wrong.slots = [[22, -1, 24]]  # the skip mark is always allowed
+    build([wrong])
+    wrong.slots = [[22, 23, 32]]
+    with pytest.raises(ValueError, match="slot 32"):
+        build([wrong])
+    bad_state = entry("a", [1], 0, [1])
+    bad_state.state_slot = 5
+    with pytest.raises(ValueError, match="state slot 5 is outside the 4 slots"):
+        build([bad_state])
+    # A windowed group: pages wholly below the lowest key of the step's first query may be gone.
+    windowed = StepLimits(num_pages=[8], windows=[6], vocab_size=50)
+    build([entry("w", [1, 2], 13, [-1, -1, 3, 4])], windowed)       # first query at 13 reads keys 8..13: pages 2, 3
+    with pytest.raises(ValueError, match="no page at index 2 .* inside the keys 8..14"):
+        build([entry("w", [1, 2], 13, [-1, -1, -1, 4])], windowed)
+    with pytest.raises(ValueError, match="no page at index 1"):
+        build([entry("w", [1, 2], 13, [0, -1, 3, 4])], StepLimits(num_pages=[8], windows=[None]))
+    # unchecked steps (measurements) pack whatever they are given
+    build_context([entry("a", [1, 2, 3, 4, 5], 0, [2, 8])], num_groups=1, page_size=4, device="cpu", check=False, limits=limits)
+
+
+def test_one_packer_fills_exact_and_padded_shapes():
+    """A recorded step's buffer is the same packed layout with more rows: what lies beyond the
+    entries is padding that reads page 0, writes nothing and uses the padding state slot."""
+    entries = [entry("x", [9], 6, [5, 1]), entry("y", [8], 2, [7]), entry("z", [3], 0, [4])]
+    entries[1].state_slot = 2
+    layout = StepLayout.make(4, 4, 4, (4,))
+    data = np.full(layout.total, 77, dtype=np.int32)
+    pack_step(data, layout, entries, range(4), pad_state_slot=9, token_sources={1: 0})
+    field = lambda name: layout.view(data, name).tolist()
+    assert field("token_ids") == [9, 8, 3, 0] and field("positions") == [6, 2, 0, 0]
+    assert field("token_seq") == [0, 1, 2, 3] and field("query_start_loc") == [0, 1, 2, 3, 4]
+    assert field("context_lens") == [7, 3, 1, 1] and field("state_slots") == [0, 2, 0, 9]
+    assert field("token_source") == [-1, 0, -1, -1] and field("logit_rows") == [0, 1, 2, 3]
+    assert field("max_decode_context") == [7]
+    assert field("slot_mapping0") == [6, 30, 16, -1]
+    assert layout.view(data, "block_table0").reshape(4, 4).tolist() == [[5, 1, 0, 0], [7, 0, 0, 0], [4, 0, 0, 0], [0, 0, 0, 0]]
+    check_packed(data, layout, entries, 4, StepLimits(num_pages=[8], windows=[None], vocab_size=10, num_state_slots=9))
+    with pytest.raises(ValueError, match="'y': token id 8"):  # a token taken from the device is not known: only 'y' is checked here
+        pack_step(data, layout, entries, range(4), pad_state_slot=9, token_sources={0: 0})
+        check_packed(data, layout, entries, 4, StepLimits(num_pages=[8], windows=[None], vocab_size=8))
+    with pytest.raises(ValueError, match="do not fit"):
+        pack_step(data, layout, [*entries, entry("p", [1, 2], 0, [1])], range(4))
+    # every field starts on 16 bytes and the same layout serves a portion beside single tokens
+    assert all(start % 4 == 0 for start, _ in layout.offsets.values())
+    mixed = [entry("p", [1, 2, 3], 4, [2, 6]), entry("x", [9], 6, [5, 1])]
+    layout = StepLayout.make(4, 2, 2, (2,))
+    data = np.zeros(layout.total, dtype=np.int32)
+    pack_step(data, layout, mixed, [2, 3])
+    assert layout.view(data, "positions").tolist() == [4, 5, 6, 6] and layout.view(data, "token_seq").tolist() == [0, 0, 0, 1]
+    assert layout.view(data, "query_start_loc").tolist() == [0, 3, 4] and layout.view(data, "max_decode_context").tolist() == [7]
 
 
 def test_sequence_accounting():
@@ -186,3 +265,34 @@ def test_bench_contract_on_the_host():
     assert bench.prefill_flops(config, layers, 2048) == 2.0 * 2048 * linear + layers * 4 * h * 2048 * 2048 / 2 + 2.0 * v * h
     assert bench.SHAPES["14b"][1]["num_hidden_layers"] == 48 and bench.SHAPES["32b"][1]["intermediate_size"] == 27648
     assert bench.PEAK_FLOPS["bf16"] == 2.5e15 and bench.PEAK_FLOPS["fp32"] == 157.3e12 and bench.HBM_PEAK_GBS == 8000.0
+
+
+def test_end_tokens_are_the_configs_and_the_tokenizers(tmp_path):
+    """The set of ids that end a generation joins ``config.json``'s and the tokenizer's
+    (src/turboserve/engine/runtime/engine.py:223-237); a ``tokenizer.json`` gets its end token
+    from the ``tokenizer_config.json`` beside it."""
+    import json
+    from types import SimpleNamespace
+
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import WhitespaceSplit
+
+    from turboserve_amd.engine.detokenizer import get_tokenizer
+    from turboserve_amd.engine.llm_engine import LLMEngine
+
+    tokenizer = Tokenizer(WordLevel({"a": 0, "b": 1, "<end>": 2, "<turn>": 3}, unk_token="a"))
+    tokenizer.pre_tokenizer = WhitespaceSplit()
+    tokenizer.save(str(tmp_path / "tokenizer.json"))
+    assert get_tokenizer(tmp_path).eos_token_id is None and get_tokenizer(tmp_path / "nothing") is None
+    (tmp_path / "tokenizer_config.json").write_text(json.dumps({"eos_token": "<turn>"}))
+    loaded = get_tokenizer(tmp_path)
+    assert loaded.eos_token_id == 3 and loaded.encode("b a <end>") == [1, 0, 2]
+    (tmp_path / "tokenizer_config.json").write_text(json.dumps({"eos_token": {"content": "<end>", "lstrip": False}}))
+    assert get_tokenizer(tmp_path).eos_token_id == 2
+    resolve = lambda config_ids, tok: LLMEngine._resolve_eos_token_ids(
+        SimpleNamespace(model_config=SimpleNamespace(eos_token_ids=config_ids), tokenizer=tok))
+    assert resolve((2,), loaded) == frozenset({2, 3})
+    assert resolve((), None) == frozenset() and resolve((7, 9), None) == frozenset({7, 9})
+    assert resolve((1,), SimpleNamespace(eos_token_id=[4, 5])) == frozenset({1, 4, 5})
+    assert LLMEngine._resolve_eos_token_ids(SimpleNamespace(model_config={"no": "attribute"}, tokenizer=loaded)) == frozenset({3})

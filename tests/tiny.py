@@ -79,8 +79,21 @@ TINY = {"A": (CONFIG_A, 0, PAGE_A), "B": (CONFIG_B, 1, PAGE_B), "C": (CONFIG_C, 
 #: A wider spread of the weights for 32-bit comparisons.  With the usual 0.02 a model this small
 #: hardly mixes its inputs (greedy generation repeats one token, attention weights are near
 #: uniform); with 0.15 every layer matters to the next token, so a fault in any of them shows.
-#: bfloat16 runs keep 0.02: their rounding error grows with the spread, the bounds do not.
 WIDE_STD = 0.15
+#: The spread for bfloat16 comparisons.  Rounding error grows faster than the spread (peaked
+#: attention turns a rounded score into a moved weight): against the 32-bit plain
+#: implementation the engine is off by up to 0.7% of a position's largest logit at 0.05, 1.6% at
+#: 0.1 and 3.9% at 0.15 (hidden size 64 to 96), and the reference's own formulas evaluated in
+#: bfloat16 (the plain implementation on bfloat16 tensors) by 1.6-2.8% at 0.1.  At 0.1 a lost
+#: page of one layer's cache still moves the logits by 24-100%.  What matters is the gain of a
+#: projection, spread x sqrt(hidden size): a model 200 wide at 0.1 is off by 3.4% in the
+#: reference's own bfloat16 arithmetic.  So the spread is 0.1 at 64 wide and falls with the width.
+BF16_STD = 0.1
+BF16_GAIN = BF16_STD * 64 ** 0.5
+
+
+def std_for(dtype: torch.dtype, hidden_size: int = 64) -> float:
+    return WIDE_STD if dtype == torch.float32 else BF16_GAIN / hidden_size ** 0.5
 
 
 def make_model_dir(folder: Path, config: dict, seed: int, dtype: torch.dtype = torch.float32, std: float = 0.02) -> Path:

@@ -9,6 +9,9 @@
 // top-k and top-p are applied as value thresholds found by bisection over the ordered bit
 // patterns of the logits, so equal logits are kept or dropped together.
 #include "common.hpp"
+#include "ts_no_alloc.h"
+
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 
@@ -150,6 +153,39 @@ extern "C" int ts_argmax(int* tokens, const float* logits, void* scratch, int ro
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
   hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(ARGMAX_SLICES), 0, stream, tokens, values, indices);
   return ts_launch_status();
+}
+
+// The same two stages with the partial results in an array of the library's own, for callers
+// that cannot allocate (see ts_no_alloc.h).  Host code never passes the array's name to a
+// kernel: its device address is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[(size_t)TS_ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * 8];
+
+#define TS_MAX_DEVICES 64
+static void* scratch_address[TS_MAX_DEVICES];  // per device; null until looked up
+static std::mutex scratch_mutex;
+
+// The address of `scratch` on the current device, or null if it cannot be found.
+static void* scratch_on_current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= TS_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (scratch_address[device] == nullptr) {
+    void* address = nullptr;
+    if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    scratch_address[device] = address;
+  }
+  return scratch_address[device];
+}
+
+extern "C" int ts_argmax_static(int* tokens, const float* logits, int rows, int vocab, hipStream_t stream) {
+  if (rows == 0) return TS_OK;
+  if (!tokens || !logits || vocab < 1 || rows < 0) return TS_ERR_ARG;
+  if (rows > TS_ARGMAX_STATIC_MAX_ROWS) return TS_ERR_SHAPE;
+  void* address = scratch_on_current_device();
+  if (address == nullptr) return TS_ERR_LAUNCH;
+  // Every element the second kernel reads (rows x 64 values, rows x 64 indices) is written by the
+  // first in this call: what an earlier call left in the array does not matter.
+  return ts_argmax(tokens, logits, address, rows, vocab, stream);
 }
 
 // Per-row parameters, all device arrays of `rows` entries:

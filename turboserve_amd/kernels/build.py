@@ -96,7 +96,7 @@ def source_hash(module: str) -> str:
     sources, extra = module_spec(module)
     digest = hashlib.sha256()
     digest.update(" ".join((*HIPCC_FLAGS, *extra)).encode())
-    headers = sorted(CSRC.glob("*.hpp"))
+    headers = sorted([*CSRC.glob("*.hpp"), *CSRC.glob("*.h")])
     for path in [*headers, *(CSRC / name for name in sources)]:
         digest.update(path.name.encode())
         digest.update(path.read_bytes())

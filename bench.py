@@ -3,20 +3,29 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A "step" is one decode step of the whole engine path: the step function over a batch of
-single tokens against the paged cache, logits, greedy sampling, tokens back on the host.  As
-in the engine's own loop a step is launched before the host has read the tokens of the step
-before it (its token ids are copied from the sampler's result on the device); every step's
-tokens are read, one step later, and the clock stops after the last are.
-The default run has the Qwen2.5-7B layer sizes (the benchmark's named configuration), random weights
-(N(0, 0.02), norm gains 1), a batch of 8 requests each holding a context of 8,192 tokens
-(cache filled with random keys and values; what is timed is real decode steps on top of it).
-One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times one
-2,048-token prompt; ``roofline`` prices the decode step against HBM bandwidth; ``points``
-holds decode at batch 1 and 64.  The prefill's projections are BLAS-library products; which
-of the library's kernels runs each is timed once before the measurement
-(``--no-gemm-tuning`` leaves it to the library's heuristic).  Peaks are the published MI355X
-figures: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+Everything is measured through the engine's own entry point: requests are given to
+``LLMEngine`` (scheduler, cache manager, step function, sampler) and the clock runs around
+calls of ``LLMEngine.step()``, the loop ``generate()`` runs.  A "step" is one decode step: every
+live request gets one token.  As always in the engine, a decode step is launched before the
+host has read the tokens of the step before it.
+
+The default run has the Qwen2.5-7B layer sizes (the benchmark's named configuration), random
+weights (N(0, 0.02), norm gains 1) and 8 requests whose prompts of uniform-random token ids
+are prefilled (chunked, by the engine) to a context of 8,192 tokens; then W untimed and K timed
+decode steps.  One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times
+one 2,048-token prompt from arrival to its first token; ``roofline`` prices the decode step
+against HBM bandwidth; ``points`` holds decode at batch 1 and 64 at the same context and the
+benchmark's literal workload (prompts of 512 tokens, 256 generated, end-of-sequence ignored,
+greedy) at 1, 8 and 64 requests, with the details of those runs under ``workload``.  The
+prefill's projections are BLAS-library products; which of the library's kernels runs each is
+timed once at the engine's start (``--no-gemm-tuning`` leaves it to the library's heuristic).
+Peaks are the published MI355X figures: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3
+TFLOP/s.
+
+Other runs: ``--shape 14b --batch 32 --mixed-prefill 2048`` (every step holds the decode tokens
+and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool of all the
+free memory), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a ``rocprofv3
+--kernel-trace`` of any of these runs).
 """
 
 from __future__ import annotations
@@ -56,6 +65,8 @@ SHAPES = {"7b": ("Qwen2.5-7B", SHAPE_7B), "14b": ("Qwen2.5-14B", SHAPE_14B), "32
 CONTEXT = 8192
 PREFILL_TOKENS = 2048
 PAGE = 16
+#: The benchmark's literal decode workload: prompt length and generated tokens.
+WORKLOAD_PROMPT, WORKLOAD_NEW = 512, 256
 
 
 def parse_args() -> argparse.Namespace:
@@ -68,137 +79,179 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=CONTEXT)
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    p.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    p.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the literal workload")
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--no-gemm-tuning", action="store_true",
                    help="leave the choice of the BLAS library's prefill kernels to its heuristic")
     p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
     p.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (the default run is 7b)")
-    p.add_argument("--fill-hbm", action="store_true",
-                   help="size the cache pool to the free device memory and interleave the requests' pages in it")
+    p.add_argument("--fill-hbm", action="store_true", help="size the cache pool to the free device memory")
     p.add_argument("--mixed-prefill", type=int, default=0, metavar="N",
-                   help="time steps that hold the batch's decode tokens and one N-token portion of a prompt")
+                   help="time steps that hold the batch's decode tokens and one whole N-token prompt")
+    p.add_argument("--no-run-ahead", action="store_true",
+                   help="read every step's tokens before the next is scheduled, as the reference's loop does")
+    p.add_argument("--kernel-shares", metavar="TRACE.csv", default=None,
+                   help="print the per-kernel table of a rocprofv3 kernel trace of a run of this program and exit")
+    p.add_argument("--shares-steps", type=int, default=4, help="steps at the end of the trace that the table covers")
     return p.parse_args()
 
 
-class DecodeBench:
-    """Requests with a given context already in the cache, decoded one token per step through
-    the engine's own cache manager, step function and sampler."""
+def tuning_file() -> str:
+    return os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")
 
-    def __init__(self, model, config, batch: int, context: int, steps_total: int, *, fill_hbm: bool = False,
-                 extra_tokens: int = 0) -> None:
-        import torch
 
-        from turboserve_amd.cache.manager import CacheManager
-        from turboserve_amd.engine.loading import build_storage
-        from turboserve_amd.engine.runner import ModelRunner
-        from turboserve_amd.sampling.sampler import Sampler
+def make_engine(model, config, *, max_num_seqs: int, budget: int, tokens_per_request: int, fill_hbm: bool = False,
+                tune_tokens: tuple[int, ...] = (), run_ahead: bool = True):
+    """An ``LLMEngine`` around the already loaded model, with a cache pool for ``max_num_seqs``
+    requests of ``tokens_per_request`` tokens (or, with ``fill_hbm``, 90% of the free memory)."""
+    import torch
 
-        self.torch = torch
-        self.batch = batch
-        self.context = context
-        self.vocab_size = config.vocab_size
-        pages_per_request = -(-(context + steps_total + 1) // PAGE)
-        num_pages = batch * pages_per_request + -(-extra_tokens // PAGE)
-        if fill_hbm:
-            # As many pages as 90% of what is free holds (at least what the requests need).
-            free, _ = torch.cuda.mem_get_info()
-            page_bytes = config.kv_bytes_per_token(model.runtime.dtype) * PAGE
-            num_pages = max(num_pages, int(free * 0.9) // page_bytes)
-        self.num_pages = num_pages
-        self.storage = build_storage(model, num_pages, PAGE, batch + 1)
-        for pages in self.storage.pages:
-            for member in pages:  # piecewise: a 200 GB pool is not filled in one launch's temporaries
-                member.normal_(0.0, 0.5)
-        self.manager = CacheManager(self.storage.layout.windows(), num_pages, PAGE, batch + 1)
-        self.runner = ModelRunner(model, self.storage, check=False)
-        self.sampler = Sampler(model.runtime.ops)
-        self.pending = None  # the sampler's result of a step whose tokens have not been read yet
-        generator = torch.Generator().manual_seed(1234)
-        self.tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
-        self.portion = torch.randint(0, config.vocab_size, (max(extra_tokens, 1),), generator=generator).tolist()
-        for request in range(batch):
-            self.manager.admit(request)
-        if fill_hbm:
-            # Page by page in turn, as requests that grow together get them: interleaved tables.
-            remaining = [context - 1] * batch
-            while any(remaining):
-                for request in range(batch):
-                    take = min(PAGE, remaining[request])
-                    if take:
-                        self.manager.append(request, take)
-                        remaining[request] -= take
-        else:
-            for request in range(batch):
-                self.manager.append(request, context - 1)  # the context's last token is decoded below
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
 
-    def step(self, portion_tokens: int = 0) -> None:
-        """One decode step of the batch; with ``portion_tokens`` the step also holds the first
-        portion, that long, of a new request's prompt (its pages are given back afterwards)."""
-        from turboserve_amd.engine.batch import StepEntry
-        from turboserve_amd.sampling.params import SamplingParams
+    num_blocks = max_num_seqs * -(-tokens_per_request // PAGE)
+    if fill_hbm:
+        free, _ = torch.cuda.mem_get_info()
+        page_bytes = config.kv_bytes_per_token(model.runtime.dtype) * PAGE
+        num_blocks = max(num_blocks, int(free * 0.9) // page_bytes)
+    engine_config = EngineConfig(
+        model="(random weights)", dtype="bfloat16" if model.runtime.dtype == torch.bfloat16 else "float32", seed=0,
+        tune_gemm_tokens=tune_tokens, gemm_tuning_file=tuning_file(), run_ahead=run_ahead,
+        scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget, block_size=PAGE,
+                                  num_blocks=num_blocks),
+    )
+    return LLMEngine(engine_config, model=model, model_config=config)
 
-        entries = []
-        if portion_tokens:
-            held = self.manager.admit("portion")
-            slots = self.manager.append("portion", portion_tokens)
-            entries.append(StepEntry(request="portion", tokens=self.portion[:portion_tokens], start=0,
-                                     tables=held.tables, slots=slots, state_slot=held.state_slot, want=[]))
-        for request in range(self.batch):
-            held = self.manager.get(request)
-            start = held.num_tokens
-            slots = self.manager.append(request, 1)
-            entries.append(StepEntry(request=request, tokens=[self.tokens[request]], start=start,
-                                     tables=held.tables, slots=slots, state_slot=held.state_slot, want=[0]))
-        greedy = SamplingParams(temperature=0.0)
-        if portion_tokens or not self.runner.takes_tokens_from(self.batch):
-            # A step with a portion of a prompt does not replay as a graph: its tokens are read
-            # before the next step is built, as the engine does for such steps.
-            self.finish()
-            logits = self.runner.step(entries)
-            out = self.sampler.sample(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
-            self.tokens = out.token_ids
-        else:
-            # As the engine's loop does (LLMEngine._run_ahead): the step is launched with its token
-            # ids taken on the device from what the step before sampled, and that step's tokens
-            # are read only afterwards, so the GPU does not wait while the host builds a step.
-            before = self.pending
-            if before is not None:
-                for entry in entries:
-                    entry.tokens = [-1]
-                logits = self.runner.step(entries, tokens_from=(before.tokens, {i: i for i in range(self.batch)}))
-            else:
-                logits = self.runner.step(entries)
-            self.pending = self.sampler.launch(logits, [greedy] * self.batch, [0] * self.batch, [0] * self.batch)
-            if before is not None:
-                self.tokens = before.read().token_ids
-        if portion_tokens:
-            self.manager.free("portion")
 
-    def finish(self) -> None:
-        """Read the tokens of the step that is still in flight, if one is."""
-        if self.pending is not None:
-            self.tokens = self.pending.read().token_ids
-            self.pending = None
+def random_prompts(config, count: int, length: int, seed: int) -> list[list[int]]:
+    import torch
 
-    def run(self, steps: int, warmup: int, portion_tokens: int = 0) -> float:
-        """Seconds for ``steps`` steps after ``warmup`` untimed ones."""
-        torch = self.torch
-        for _ in range(warmup):
-            self.step(portion_tokens)
-        self.finish()
+    generator = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, config.vocab_size, (length,), generator=generator).tolist() for _ in range(count)]
+
+
+def run_decode(model, config, batch: int, prompt_len: int, *, steps: int, warmup: int, fill_hbm: bool = False,
+               mixed_prefill: int = 0, tune: bool = False, run_ahead: bool = True) -> dict:
+    """``batch`` requests with prompts of ``prompt_len`` uniform-random ids through
+    ``LLMEngine``: prefill (chunked by the engine; requests whose prompt is done decode
+    meanwhile), ``warmup`` untimed decode steps of the whole batch, ``steps`` timed ones.  With
+    ``mixed_prefill`` every step also holds one new request's whole prompt of that many tokens
+    (which ends after its first token)."""
+    import torch
+
+    from turboserve_amd.sampling.params import SamplingParams
+
+    budget = max(PREFILL_TOKENS, mixed_prefill + batch, batch)
+    # Tokens a request may have to produce: the steps of this run and those it decodes while the
+    # others' prompts are still being prefilled, with a few to spare (no request may end inside the clock).
+    max_new = warmup + steps + batch * -(-prompt_len // budget) + 8
+    engine = make_engine(
+        model, config, max_num_seqs=batch + (1 if mixed_prefill else 0), budget=budget,
+        tokens_per_request=prompt_len + max_new + (-(-mixed_prefill // batch) if mixed_prefill else 0),
+        fill_hbm=fill_hbm, tune_tokens=(mixed_prefill + batch,) if (mixed_prefill and tune) else (), run_ahead=run_ahead,
+    )
+    pool_tokens = min(engine.storage.num_pages) * PAGE
+    decode = SamplingParams(max_tokens=max_new, temperature=0.0, ignore_eos=True)
+    one = SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True)
+    extra = random_prompts(config, 1, max(mixed_prefill, 1), 99)[0]
+    sequences = [engine.add_request(f"r{index}", prompt, decode)
+                 for index, prompt in enumerate(random_prompts(config, batch, prompt_len, 1234))]
+    started = time.perf_counter()
+    first_tokens = 0
+    while first_tokens < batch:  # the prompts' portions, until every request has its first token
+        first_tokens += sum(1 for out in engine.step() if out.output_tokens == 1)
+    torch.cuda.synchronize()
+    prefill_seconds = time.perf_counter() - started
+    arrivals = 0
+
+    def step() -> None:
+        nonlocal arrivals
+        if mixed_prefill:
+            engine.add_request(f"p{arrivals}", extra, one)
+            arrivals += 1
+        engine.step()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    context_before = sum(seq.num_tokens for seq in sequences) / batch
+    started = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - started
+    stats = engine.stats()
+    assert not any(seq.is_finished for seq in sequences), "a request ended inside the timed steps"
+    for index in range(batch):
+        engine.abort(f"r{index}")
+    engine.close()
+    return {"tokens_per_s": batch * steps / seconds, "step_seconds": seconds / steps, "prefill_seconds": prefill_seconds,
+            "mean_context": context_before + steps / 2, "pool_tokens": pool_tokens,
+            "preemptions": int(stats["num_preemptions"])}
+
+
+def run_workload(model, config, batch: int, prompt_len: int, new_tokens: int, run_ahead: bool = True) -> dict:
+    """The benchmark's literal decode workload through ``LLMEngine``'s loop (the loop the
+    reference times, src/turboserve/engine/runtime/engine.py:414-448): ``batch`` prompts of
+    ``prompt_len`` uniform-random ids, ``new_tokens`` generated each, greedy, end-of-sequence
+    ignored.  Decoding is priced over the steps in which the whole batch decodes: from the
+    moment the last request has its first token to the moment the first request ends."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    engine = make_engine(model, config, max_num_seqs=batch, budget=PREFILL_TOKENS,
+                         tokens_per_request=prompt_len + new_tokens + 1, run_ahead=run_ahead)
+    sampling = SamplingParams(max_tokens=new_tokens, temperature=0.0, ignore_eos=True)
+    sequences = [engine.add_request(f"w{index}", prompt, sampling)
+                 for index, prompt in enumerate(random_prompts(config, batch, prompt_len, 777))]
+    started = time.perf_counter()
+    first_tokens = finished = tokens = calls = 0
+    window_start = window_end = None
+    context_at_start = 0.0
+    while engine.has_unfinished():
+        outputs = engine.step()
+        now = time.perf_counter()
+        if window_start is not None and window_end is None:
+            calls += 1
+            tokens += sum(len(out.new_token_ids) for out in outputs)
+        first_tokens += sum(1 for out in outputs if out.output_tokens == 1)
+        finished += sum(1 for out in outputs if out.finished)
+        if window_start is None and first_tokens == batch:
+            window_start = now
+            context_at_start = sum(seq.num_tokens for seq in sequences) / batch
+        if window_end is None and finished > 0:
+            window_end = now
+    total = time.perf_counter() - started
+    engine.close()
+    assert all(seq.num_output_tokens == new_tokens for seq in sequences)
+    window = window_end - window_start
+    return {"tokens_per_s": tokens / window, "step_seconds": window / calls, "steps": calls,
+            "mean_context": context_at_start + calls / 2, "first_tokens_seconds": window_start - started,
+            "total_seconds": total, "total_tokens_per_s": batch * new_tokens / total}
+
+
+def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True) -> float:
+    """Seconds (best of ``repeats``) from the arrival of a ``tokens``-long prompt to its first
+    token on the host, through ``LLMEngine`` with a step budget that takes the prompt whole."""
+    import torch
+
+    from turboserve_amd.sampling.params import SamplingParams
+
+    engine = make_engine(model, config, max_num_seqs=1, budget=tokens, tokens_per_request=tokens + 1,
+                         tune_tokens=(tokens,) if tune else ())
+    prompt = random_prompts(config, 1, tokens, 4321)[0]
+    best = float("inf")
+    for attempt in range(repeats + 1):
         torch.cuda.synchronize()
         started = time.perf_counter()
-        for _ in range(steps):
-            self.step(portion_tokens)
-        self.finish()
+        engine.add_request(f"p{attempt}", prompt, SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True))
+        outputs = []
+        while not outputs:
+            outputs = engine.step()
         torch.cuda.synchronize()
-        return time.perf_counter() - started
-
-    def close(self) -> None:
-        self.runner.release()
-        self.storage = None
-        self.torch.cuda.empty_cache()
+        best = min(best, time.perf_counter() - started)
+        assert outputs[0].finished and len(outputs[0].new_token_ids) == 1
+    engine.close()
+    return best
 
 
 def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
@@ -222,50 +275,13 @@ def prefill_flops(config, layers: int, tokens: int) -> float:
     return 2.0 * tokens * linear + attention + 2.0 * config.vocab_size * h
 
 
-def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True) -> float:
-    """Seconds (best of ``repeats``) for one step over a ``tokens``-long prompt, to its last
-    position's logits on the host.  With ``tune`` the BLAS library's kernels for the step's
-    products are timed first in a dry step and the fastest kept, as an engine started with
-    ``tune_gemm_tokens`` does."""
-    import torch
-
-    from turboserve_amd.cache.manager import CacheManager
-    from turboserve_amd.engine.batch import StepEntry
-    from turboserve_amd.engine.loading import build_storage
-    from turboserve_amd.engine.runner import ModelRunner
-
-    num_pages = -(-tokens // PAGE)
-    storage = build_storage(model, num_pages, PAGE, 1)
-    manager = CacheManager(storage.layout.windows(), num_pages, PAGE, 1)
-    runner = ModelRunner(model, storage, check=False)
-    if tune and model.runtime.dtype == torch.bfloat16:
-        from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
-
-        with LibraryGemmTuning(os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")):
-            runner.dry_run(tokens)
-    generator = torch.Generator().manual_seed(4321)
-    prompt = torch.randint(0, config.vocab_size, (tokens,), generator=generator).tolist()
-    best = float("inf")
-    for _ in range(repeats + 1):
-        held = manager.admit("p")
-        slots = manager.append("p", tokens)
-        entry = StepEntry(request="p", tokens=prompt, start=0, tables=held.tables, slots=slots,
-                          state_slot=held.state_slot, want=[tokens - 1])
-        torch.cuda.synchronize()
-        started = time.perf_counter()
-        logits = runner.step([entry])
-        logits.argmax(dim=-1).tolist()
-        torch.cuda.synchronize()
-        best = min(best, time.perf_counter() - started)
-        manager.free("p")
-    runner.release()
-    del storage
-    torch.cuda.empty_cache()
-    return best
-
-
 def main() -> int:
     args = parse_args()
+    if args.kernel_shares:
+        from turboserve_amd.profiling import format_shares, step_shares
+
+        print(format_shares(step_shares(args.kernel_shares, steps=args.shares_steps)))
+        return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU by design)")
         return 2
@@ -287,50 +303,37 @@ def main() -> int:
     layers = config.num_hidden_layers
     itemsize = 2 if dtype == torch.bfloat16 else 4
     dtype_key = "bf16" if dtype == torch.bfloat16 else "fp32"
-
-    pool_tokens = 0
-
-    def decode_rate(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        nonlocal pool_tokens
-        bench = DecodeBench(model, config, batch, args.context, steps + warmup, fill_hbm=args.fill_hbm,
-                            extra_tokens=args.mixed_prefill)
-        pool_tokens = bench.num_pages * PAGE
-        if args.mixed_prefill and not args.no_gemm_tuning and dtype == torch.bfloat16:
-            from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
-
-            with LibraryGemmTuning(os.path.join(tempfile.gettempdir(), f"turboserve_amd_bench_gemm_{os.getuid()}.csv")):
-                bench.runner.dry_run(args.mixed_prefill + batch)
-        seconds = bench.run(steps, warmup, args.mixed_prefill)
-        bench.close()
-        return batch * steps / seconds, seconds / steps
+    tune = not args.no_gemm_tuning and dtype == torch.bfloat16
+    run_ahead = not args.no_run_ahead
 
     if args.only_prefill:
-        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=not args.no_gemm_tuning)
+        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=tune)
         print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}))
         return 0
 
-    value, step_seconds = decode_rate(args.batch, args.steps, args.warmup)
+    main_run = run_decode(model, config, args.batch, args.context - 1, steps=args.steps, warmup=args.warmup,
+                          fill_hbm=args.fill_hbm, mixed_prefill=args.mixed_prefill, tune=tune, run_ahead=run_ahead)
+    step_seconds = main_run["step_seconds"]
     if args.mixed_prefill:
         # A mixed step is priced by its products' flops, not by bytes: say what ran and stop there.
         flops = (prefill_flops(config, layers, args.mixed_prefill)
                  + 2.0 * args.batch * decode_bytes(config, layers, 0, 0, 1)  # every weight once per decode token
                  + 4.0 * args.batch * layers * config.q_proj_size * args.context)  # and its attention
         print(json.dumps({
-            "metric": f"mixed step: {args.batch} decode tokens + one {args.mixed_prefill}-token prompt portion "
-                      f"({shape_name} shape, one MI355X)",
+            "metric": f"mixed step: {args.batch} decode tokens + one {args.mixed_prefill}-token prompt "
+                      f"({shape_name} shape, one MI355X, through LLMEngine)",
             "value": round((args.batch + args.mixed_prefill) / step_seconds, 1), "unit": "tokens/s",
-            "decode_tokens_per_s": round(value, 2), "ms_per_step": round(step_seconds * 1e3, 3),
+            "decode_tokens_per_s": round(main_run["tokens_per_s"], 2), "ms_per_step": round(step_seconds * 1e3, 3),
             "steps": args.steps, "warmup": args.warmup, "dtype": dtype_key, "decode_context": args.context,
-            "layers": layers, "kv_pool_tokens": pool_tokens,
+            "layers": layers, "kv_pool_tokens": main_run["pool_tokens"],
             "flops_frac": round(flops / step_seconds / PEAK_FLOPS[dtype_key], 4),
         }))
         return 0
-    mean_context = args.context + args.warmup + args.steps / 2
-    read = decode_bytes(config, layers, args.batch, mean_context, itemsize)
+    read = decode_bytes(config, layers, args.batch, main_run["mean_context"], itemsize)
     achieved = read / step_seconds / 1e9
     result = {
         "metric": f"decode tok/s ({shape_name} shape, paged cache, one MI355X)",
-        "value": round(value, 2),
+        "value": round(main_run["tokens_per_s"], 2),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -340,7 +343,7 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": dtype_key,
-        "data": "synthetic: random weights N(0,0.02), uniform-random token ids, cache pre-filled with random keys/values",
+        "data": "synthetic: random weights N(0,0.02), uniform-random token ids; prompts prefilled by the engine",
         "config": {
             "model": f"{shape_name} shape (Qwen2ForCausalLM)",
             "global_batch": args.batch,
@@ -358,9 +361,9 @@ def main() -> int:
             "rms_norm_eps": config.rms_norm_eps,
             "tie_word_embeddings": config.tie_word_embeddings,
             "page_size": PAGE,
-            "kv_pool_tokens": pool_tokens,
+            "kv_pool_tokens": main_run["pool_tokens"],
             "prefill_tokens": PREFILL_TOKENS,
-            "prefill_gemm_choice": "library heuristic" if args.no_gemm_tuning else "library candidates timed at start-up",
+            "path": "LLMEngine.step (scheduler, cache manager, step function, sampler)" + ("" if run_ahead else ", no run-ahead"),
             "sampling": "greedy",
         },
         "roofline": {
@@ -372,7 +375,7 @@ def main() -> int:
         },
     }
     if not args.no_prefill:
-        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=not args.no_gemm_tuning)
+        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=tune)
         flops = prefill_flops(config, layers, PREFILL_TOKENS)
         result["prefill"] = {
             "value": round(PREFILL_TOKENS / seconds, 1),
@@ -381,11 +384,25 @@ def main() -> int:
             "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4),
         }
     if not args.no_points:
-        points = {}
+        points, workload = {}, {}
         for batch in (1, 64):
-            rate, _ = decode_rate(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
-            points[f"decode_b{batch}"] = round(rate, 2)
+            run = run_decode(model, config, batch, args.context - 1, steps=max(8, args.steps // 2),
+                             warmup=max(2, args.warmup // 2), run_ahead=run_ahead)
+            points[f"decode_b{batch}"] = round(run["tokens_per_s"], 2)
+        # The benchmark's literal workload: prompts of 512 ids, 256 generated, 1 / 8 / 64 requests.
+        for batch in (1, 8, 64):
+            run = run_workload(model, config, batch, WORKLOAD_PROMPT, WORKLOAD_NEW, run_ahead=run_ahead)
+            read = decode_bytes(config, layers, batch, run["mean_context"], itemsize)
+            points[f"decode_b{batch}_prompt{WORKLOAD_PROMPT}_new{WORKLOAD_NEW}"] = round(run["tokens_per_s"], 2)
+            workload[f"b{batch}"] = {
+                "ms_per_step": round(run["step_seconds"] * 1e3, 4), "steps": run["steps"],
+                "mean_context": round(run["mean_context"], 1),
+                "hbm_frac": round(read / run["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4),
+                "first_tokens_ms": round(run["first_tokens_seconds"] * 1e3, 2),
+                "whole_run_tokens_per_s": round(run["total_tokens_per_s"], 2),
+            }
         result["points"] = points
+        result["workload"] = workload
     info = collect()
     result["hw"] = {"gpu": info["gpu_name"], "torch": info["torch"]["version"], "hip": info["torch"]["hip_version"],
                     "git": (info["git"]["sha"] or "")[:12]}

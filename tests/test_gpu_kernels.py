@@ -435,6 +435,9 @@ ATTENTION_GEOMETRIES = [
     (2, 1, 256, 64),
     (6, 2, 256, 16),    # G = 3 at the largest head size: staged windows above 64 KiB of LDS
     (10, 2, 48, 8),     # G = 5, a head size that is no multiple of 32
+    (9, 3, 32, 16),     # G = 3 at the smallest head size of the 32-tokens-per-wavefront prefill kernel
+    (10, 2, 96, 32),    # G = 5 (two chunks of four heads, the second with one live wavefront), head size 96
+    (40, 8, 128, 16),   # G = 5 on 8 KV heads, as the 14B and 32B shapes
 ]
 
 
@@ -461,6 +464,15 @@ def test_attention_decode_mfma(ops, heads, kv_heads, dim, page, window):
         case.ints(case.qsl), case.ints(contexts), 0, len(contexts), heads, dim ** -0.5, window, max(contexts),
     )
     torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+
+
+def prefill_blocks_of(ops, case, heads, kv_heads, dim, seqs, shuffle=None):
+    """(rows per block the kernel for this geometry takes, its work list for ``seqs``)."""
+    rows = ops.prefill_block_rows(dim, heads, kv_heads)
+    blocks = [(s, case.qsl[s] + off) for s, (_, qlen) in enumerate(seqs) for off in range(0, qlen, rows)]
+    if shuffle is not None:
+        random.Random(shuffle).shuffle(blocks)
+    return rows, blocks
 
 
 def test_attention_decode_mfma_far_key_and_subrange(ops):
@@ -496,12 +508,12 @@ def test_attention_decode_mfma_at_tens_of_thousands_of_keys(ops):
     # the same cache, its last 40 positions as a prompt portion
     seqs = [(40000, 40)]
     portion = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, None, seed=9, spike=23456)
-    blocks = [(0, off) for off in range(0, 40, 16)]
+    rows, blocks = prefill_blocks_of(ops, portion, heads, kv_heads, dim, seqs)
     out = torch.zeros(40, heads * dim, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(
         out, portion.dev(portion.q), heads * dim, portion.dev(portion.kp), portion.dev(portion.vp),
         portion.dev(portion.table), portion.ints(portion.qsl), portion.ints([40000]), portion.ints(blocks), heads,
-        dim ** -0.5, None, 40000,
+        dim ** -0.5, None, 40000, rows,
     )
     torch.testing.assert_close(out.float().cpu(), portion.expected, **tol(torch.bfloat16))
 
@@ -513,26 +525,41 @@ def test_attention_prefill_mfma(ops, heads, kv_heads, dim, page, window):
     every alignment against pages and 32-key windows."""
     seqs = [(70, 70), (33, 2), (600, 77), (129, 16), (257, 17), (48, 48), (2, 2), (515, 33)]
     case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, window, seed=dim + 2)
-    blocks = [(s, case.qsl[s] + off) for s, (_, qlen) in enumerate(seqs) for off in range(0, qlen, 16)]
-    random.Random(3).shuffle(blocks)
+    rows, blocks = prefill_blocks_of(ops, case, heads, kv_heads, dim, seqs, shuffle=3)
     out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(
         out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
         case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, window,
-        max(c for c, _ in seqs),
+        max(c for c, _ in seqs), rows,
     )
     torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+
+
+def test_prefill_block_rows_follow_the_geometry(ops):
+    """32 rows per wavefront where the wide kernel runs (three or more query heads per KV head,
+    head sizes 32 to 128 in steps of 32), 16 elsewhere; a work list of the other length is refused."""
+    from turboserve_amd.kernels.ops import KernelError
+
+    assert ops.prefill_block_rows(128, 28, 4) == 32 and ops.prefill_block_rows(64, 8, 1) == 32
+    assert ops.prefill_block_rows(128, 8, 4) == 16 and ops.prefill_block_rows(48, 10, 2) == 16
+    assert ops.prefill_block_rows(256, 6, 2) == 16 and ops.prefill_block_rows(80, 40, 2) == 16
+    case = PagedCase(torch.bfloat16, 14, 2, 128, 16, [(40, 40)], None, seed=1)
+    out = torch.zeros(40, 14 * 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="rows"):
+        ops.attention_prefill(out, case.dev(case.q), 14 * 128, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+                              case.ints(case.qsl), case.ints([40]), case.ints([(0, 0), (0, 16), (0, 32)]), 14, 128 ** -0.5,
+                              None, 40, 16)
 
 
 def test_attention_prefill_mfma_far_key(ops):
     heads, kv_heads, dim, page = 28, 4, 128, 16
     seqs = [(3000, 40), (2100, 2100)]
     case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, None, seed=11, spike=77)
-    blocks = [(s, case.qsl[s] + off) for s, (_, qlen) in enumerate(seqs) for off in range(0, qlen, 16)]
+    rows, blocks = prefill_blocks_of(ops, case, heads, kv_heads, dim, seqs)
     out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(
         out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
-        case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, None, 3000,
+        case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, None, 3000, rows,
     )
     got = out.float().cpu()
     torch.testing.assert_close(got, case.expected, **tol(torch.bfloat16))
@@ -570,11 +597,11 @@ def test_attention_at_the_windows_edge(ops, heads, kv_heads, dim, page, window):
     rows = case.expected.view(qlen, -1).abs().mean(1) > 4.0
     positions = torch.arange(ctx - qlen, ctx)
     assert torch.equal(rows, (positions >= spike) & (positions <= spike + window - 1))
-    blocks = [(0, off) for off in range(0, qlen, 16)]
+    rows, blocks = prefill_blocks_of(ops, case, heads, kv_heads, dim, [(ctx, qlen)])
     out = torch.zeros(qlen, heads * dim, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(
         out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
-        case.ints(case.qsl), case.ints([ctx]), case.ints(blocks), heads, dim ** -0.5, window, ctx,
+        case.ints(case.qsl), case.ints([ctx]), case.ints(blocks), heads, dim ** -0.5, window, ctx, rows,
     )
     torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
     got = ops.paged_attention_generic(

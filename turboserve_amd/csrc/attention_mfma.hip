@@ -27,6 +27,8 @@
 // with fewer, one wavefront serves two heads from registers alone (prefill_kernel).
 #include "common.hpp"
 
+#include <type_traits>
+
 #ifndef TS_HEAD_DIM
 #error "compile with -DTS_HEAD_DIM=<head size>"
 #endif
@@ -658,6 +660,16 @@ __device__ __forceinline__ void fetch_window(StagedWindow& r, const PageGeometry
 // Write the fetched window `w` to LDS.  Values of keys outside lo..last are whatever an earlier
 // owner of the page left: they are cleared here, so that a stale non-finite value cannot meet a
 // zero probability (only a window that is not wholly inside lo..last needs it).
+// Row of the 32-row score tile (v_mfma_f32_32x32x16_bf16) that holds key offset ko of a window.
+// The accumulator gives lane half h (lanes 32 h .. 32 h + 31) the rows 8 a + 4 h + b in register
+// 4 a + b; as B operand of the second product the same lane must hold, for the 16-key step s,
+// the keys 16 s + 8 h .. + 7.  So registers 0..7 are the keys of step 0 and 8..15 those of step
+// 1: key offset 16 (a / 2) + 8 h + 4 (a % 2) + b sits in row 8 a + 4 h + b.
+__device__ __forceinline__ int wide_key_row(int ko) {
+  return 8 * (2 * (ko >> 4) + ((ko >> 2) & 1)) + 4 * ((ko >> 3) & 1) + (ko & 3);
+}
+
+template <bool WIDE = false>
 __device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const StagedWindow& r, int w, int lo, int last,
                                              int wave, int lane) {
 #pragma unroll
@@ -668,7 +680,7 @@ __device__ __forceinline__ void stage_window(uint16_t* ks, uint16_t* vs, const S
       // t = (ko / 4) % 2, row m = 4 (ko / 8) + ko % 4, stored at 16 t + m, so that the 16 lanes
       // of an LDS pass read 16 consecutive rows (distinct banks with the padded stride).
       const int ko = KEYS_PER_WAVE * wave + piece / (D / 8);
-      const int slot = 16 * ((ko >> 2) & 1) + ((ko >> 3) << 2) + (ko & 3);
+      const int slot = WIDE ? wide_key_row(ko) : 16 * ((ko >> 2) & 1) + ((ko >> 3) << 2) + (ko & 3);
       *reinterpret_cast<u32x4*>(ks + slot * K_ROW + 8 * (piece % (D / 8))) = r.k[i];
     }
   }
@@ -878,6 +890,386 @@ static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16
   return ts_launch_status();
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// prefill, 32 tokens per wavefront (head sizes 32, 64, 96, 128; three or more query heads per
+// KV head): one workgroup of four wavefronts per (block of 32 rows, KV head, four of its query
+// heads), one head per wavefront.  S^T = K Q^T is a 32 x 32 tile of v_mfma_f32_32x32x16_bf16
+// (rows: the window's 32 keys, columns: the 32 tokens), O^T = V^T P^T four such tiles.  A column's
+// 32 scores lie in two lanes (l and l ^ 32), 16 registers each, so the softmax's maximum and sum
+// are taken inside a lane and crossed once; per score it costs under half the vector
+// instructions of the 16-column kernels, and a key row read from LDS serves 32 tokens.  Windows
+// are fetched and staged exactly as in prefill_shared_kernel (same LDS image but for the order
+// of the key rows, see wide_key_row).
+// ---------------------------------------------------------------------------------------------
+#if TS_HEAD_DIM % 32 == 0 && TS_HEAD_DIM <= 128
+#define TS_WIDE_PREFILL 1
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int WIDE_ROWS = 32;
+constexpr int KJ16 = D / 16;  // 16-deep steps of the first product
+constexpr int NT32 = D / 32;  // 32-wide tiles of the head dimension (second product)
+
+// Keys and values of a window travel separately in this kernel (the keys of a window are needed
+// one round before its values), so the fetched pieces are kept apart.
+struct StagedKeys {
+  u32x4 k[K_EACH];
+};
+struct StagedValues {
+  u32x4 v[V_EACH];
+};
+
+// The two halves of fetch_window: this wavefront's eight key rows, or the eight keys' values, of
+// window `w` (keys outside lo..last are replaced, see live_key).
+// `page` is the page of the wavefront's eight keys of window `w` (page_of_chunk), looked up a round
+// earlier so that nothing waits for it here; a window at the edge of lo..last looks its pages up
+// per lane instead.
+__device__ __forceinline__ int page_of_chunk(const PageGeometry& g, int w, int wave) {
+  return g.table[__builtin_amdgcn_readfirstlane(w + KEYS_PER_WAVE * wave) >> g.block_shift];
+}
+
+__device__ __forceinline__ void fetch_keys(StagedKeys& r, const PageGeometry& g, int w, int lo, int last, int wave,
+                                           int lane, int page_id) {
+  const int first_key = w + KEYS_PER_WAVE * wave;  // the same in every lane of the wavefront
+  if (w >= lo && w + WINDOW_KEYS - 1 <= last) {
+    const long long page = page_id;
+    const uint16_t* kbase = g.k_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D +
+                            (long long)(first_key & g.block_mask) * D;
+#pragma unroll
+    for (int i = 0; i < K_EACH; ++i)
+      r.k[i] = load8(kbase + 8 * min(lane + i * TS_WAVE, K_WAVE_PIECES - 1));  // spare lanes repeat the last piece
+  } else {
+#pragma unroll
+    for (int i = 0; i < K_EACH; ++i) {
+      const int piece = min(lane + i * TS_WAVE, K_WAVE_PIECES - 1);
+      const int key = live_key(first_key + piece / (D / 8), w, lo, last);
+      const long long page = g.table[key >> g.block_shift];
+      r.k[i] = load8(g.k_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D +
+                     (long long)(key & g.block_mask) * D + 8 * (piece % (D / 8)));
+    }
+  }
+}
+
+__device__ __forceinline__ void fetch_values(StagedValues& r, const PageGeometry& g, int w, int lo, int last, int wave,
+                                             int lane, int page_id) {
+  const int first_key = w + KEYS_PER_WAVE * wave;
+  int chunk = first_key;
+  long long page = page_id;
+  if (!(w >= lo && w + WINDOW_KEYS - 1 <= last)) {
+    const bool live = first_key + 7 >= lo && first_key <= last;
+    chunk = live ? first_key : (live_key(first_key, w, lo, last) & ~7);
+    page = g.table[__builtin_amdgcn_readfirstlane(chunk) >> g.block_shift];
+  }
+  const uint16_t* vbase = g.v_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D + (chunk & g.block_mask);
+#pragma unroll
+  for (int i = 0; i < V_EACH; ++i)
+    r.v[i] = load8(vbase + ((long long)min(lane + i * TS_WAVE, D - 1) << g.block_shift));
+}
+
+// The halves of stage_window, keys in the row order of the 32-row score tile (wide_key_row).
+__device__ __forceinline__ void stage_keys(uint16_t* ks, const StagedKeys& r, int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < K_EACH; ++i) {
+    const int piece = lane + i * TS_WAVE;
+    if (piece < K_WAVE_PIECES) {
+      const int ko = KEYS_PER_WAVE * wave + piece / (D / 8);
+      *reinterpret_cast<u32x4*>(ks + wide_key_row(ko) * K_ROW + 8 * (piece % (D / 8))) = r.k[i];
+    }
+  }
+}
+
+__device__ __forceinline__ void stage_values(uint16_t* vs, const StagedValues& r, int w, int lo, int last, int wave,
+                                             int lane) {
+  const int chunk = w + KEYS_PER_WAVE * wave;
+  const bool edge = w < lo || w + WINDOW_KEYS - 1 > last;
+#pragma unroll
+  for (int i = 0; i < V_EACH; ++i) {
+    const int d = lane + i * TS_WAVE;
+    if (d >= D) continue;
+    u32x4 value = r.v[i];
+    if (edge) {  // stale values of keys outside lo..last are cleared (see stage_window)
+      asm volatile("" ::: "memory");  // keeps this a branch, taken by a block's first and last windows only
+      const bool live = chunk + 7 >= lo && chunk <= last;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t low = (live && chunk + 2 * e <= last) ? 0x0000ffffu : 0u;
+        const uint32_t high = (live && chunk + 2 * e + 1 <= last) ? 0xffff0000u : 0u;
+        value[e] &= low | high;
+      }
+    }
+    *reinterpret_cast<u32x4*>(vs + d * V_ROW + KEYS_PER_WAVE * wave) = value;
+  }
+}
+
+// How far (in powers of two) a column's scores may rise above the reference its probabilities
+// are taken against before the reference is moved and the accumulators rescaled.  Probabilities
+// then reach 2^8 at most, which 32-bit sums and bfloat16 operands hold as well as values up to 1;
+// after a column's first windows its reference hardly ever moves again, and the rescaling of the
+// D / 2 accumulator registers is skipped.
+constexpr float WIDE_RESCALE_SLACK = 8.f;
+
+// Scores of keys the lane's column must not see become -inf (in place).  Register i of lane
+// half h holds the key at offset 16 (i / 8) + 8 h + 4 ((i / 4) % 2) + i % 4 of the window.
+__device__ __forceinline__ void wide_mask(f32x16& s, int w, int half, int first_valid, int last_valid) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int key = w + 16 * (i >> 3) + 8 * half + 4 * ((i >> 2) & 1) + (i & 3);
+    s[i] = (key >= first_valid && key <= last_valid) ? s[i] : -INFINITY;
+  }
+}
+
+// S^T of the window staged at `ks` for the wavefront's 32 tokens and its head, as one
+// accumulation chain on the matrix cores.
+__device__ __forceinline__ void wide_scores(f32x16& s, const uint16_t* ks, const Frag8 (&qf)[KJ16], int col, int half) {
+  const uint16_t* krow = ks + col * K_ROW + 8 * half;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < KJ16; ++j)
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(krow + 16 * j)), as_bf16x8(qf[j]), s, 0, 0, 0);
+}
+
+__global__ void __launch_bounds__(STAGE_WAVES * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
+                    const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
+                    const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
+                    const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
+                    int pair_blocks, int heads, int kv_heads, int block_shift, float scale_log2, int window) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
+  uint16_t* ks = staged;
+  uint16_t* vs = staged + 2 * K_TILE;
+  const int lane = threadIdx.x & (TS_WAVE - 1);
+  const int wave = threadIdx.x / TS_WAVE;
+  const int col = lane & 31;
+  const int half = lane >> 5;
+  const int gsize = heads / kv_heads;
+  constexpr int HW = STAGE_WAVES;
+  const int head_chunks = (gsize + HW - 1) / HW;
+  // Workgroup id -> (block, KV head, chunk of its query heads) and the pairing of heavy and
+  // light blocks: as in prefill_shared_kernel.
+  const int lanes_y = kv_heads * head_chunks;
+  const int y = blockIdx.x % lanes_y;
+  int block = blockIdx.x / lanes_y;
+  if (pair_blocks && block >= (num_blocks + 1) / 2) block = num_blocks - 1 - (block - (num_blocks + 1) / 2);
+  const int kvh = y / head_chunks;
+  const int hg = (y % head_chunks) * HW + wave;  // this wavefront's head within the KV head's group
+  const bool wave_live = hg < gsize;
+  const int seq = blocks[2 * block];
+  const int row0 = blocks[2 * block + 1];
+  const int row_end = query_start_loc[seq + 1];
+  const int ctx = context_lens[seq];
+  const int pos0 = ctx - (row_end - query_start_loc[seq]) + (row0 - query_start_loc[seq]);  // position of row0
+  const int cols = min(WIDE_ROWS, row_end - row0);
+  const bool col_valid = col < cols;
+  const int p_col = col_valid ? pos0 + col : -1;  // an invalid column sees nothing and is never stored
+  const int lo_col = (window > 0 && p_col - window + 1 > 0) ? p_col - window + 1 : 0;
+  const int p_last = pos0 + cols - 1;
+  const int lo_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int begin = lo_first & ~(WINDOW_KEYS - 1);
+  const int end = p_last + 1;
+  const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+  auto interior = [&](int w) { return cols == WIDE_ROWS && w >= lo_last && w + WINDOW_KEYS - 1 <= pos0; };
+
+  PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, table_width, kv_heads, kvh, block_shift,
+                   (1 << block_shift) - 1};
+  // The queries as B operands: lane holds, for token `col`, head dimensions 16 j + 8 half .. + 7.
+  Frag8 qf[KJ16];
+  {
+    const uint16_t* row = (col_valid && wave_live)
+                              ? q + (size_t)(row0 + col) * q_stride + (size_t)(kvh * gsize + hg) * D + 8 * half
+                              : nullptr;
+#pragma unroll
+    for (int j = 0; j < KJ16; ++j) qf[j] = row ? load8(row + 16 * j) : Frag8{0u, 0u, 0u, 0u};
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x16 acc[NT32];
+#pragma unroll
+  for (int t = 0; t < NT32; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+
+  // A software pipeline over the windows W(i) = begin + 32 i.  Round i issues, as one stretch of
+  // straight-line code, the products of two other windows beside the softmax of W(i): the
+  // scores of W(i + 1) and the accumulation of W(i - 1)'s values with the probabilities of the
+  // round before.  The matrix instructions and the vector instructions between them do not
+  // depend on each other, so a wavefront keeps both units busy on its own (instructions issue in
+  // order: a vector instruction behind a chain of dependent matrix instructions would wait for
+  // the whole chain).  Meanwhile the keys of W(i + 2) and the values of W(i), fetched a round
+  // ago, go to LDS, and the keys of W(i + 3) and the values of W(i + 1) are asked for.  LDS
+  // holds two windows of keys and two of values.  Windows past the last are the last again
+  // (loads stay unconditional, see prefill_shared_kernel); their scores are computed and dropped.
+  const int last_window = (end - 1) & ~(WINDOW_KEYS - 1);
+  auto window_at = [&](int i) { return min(begin + i * WINDOW_KEYS, last_window); };
+  StagedKeys kr[2];
+  StagedValues vr[2];
+  // The pages of this wavefront's keys in the windows W(i + 1) .. W(i + 4) of round i.
+  int page1 = page_of_chunk(geo, window_at(1), wave), page2 = page_of_chunk(geo, window_at(2), wave);
+  int page3 = page_of_chunk(geo, window_at(3), wave), page4 = page_of_chunk(geo, window_at(4), wave);
+  {
+    const int page0 = page_of_chunk(geo, window_at(0), wave);
+    fetch_keys(kr[0], geo, window_at(0), lo_first, p_last, wave, lane, page0);
+    fetch_keys(kr[1], geo, window_at(1), lo_first, p_last, wave, lane, page1);
+    fetch_values(vr[0], geo, window_at(0), lo_first, p_last, wave, lane, page0);
+  }
+  // The value windows start as zeros: the first round multiplies one of them by probabilities
+  // that are all zero, and what LDS held before could be anything.
+  for (int e = threadIdx.x * 8; e < 2 * V_TILE; e += STAGE_WAVES * TS_WAVE * 8)
+    *reinterpret_cast<u32x4*>(vs + e) = u32x4{0u, 0u, 0u, 0u};
+  stage_keys(ks, kr[0], wave, lane);
+  stage_keys(ks + K_TILE, kr[1], wave, lane);
+  fetch_keys(kr[0], geo, window_at(2), lo_first, p_last, wave, lane, page2);
+  __syncthreads();
+  f32x16 s[2];  // the scores of the round's window and of the next, by parity of the round
+  wide_scores(s[0], ks, qf, col, half);
+  __syncthreads();  // round 0 writes the window after next where these scores' keys were
+  Frag8 pp0 = {0u, 0u, 0u, 0u}, pp1 = {0u, 0u, 0u, 0u};  // the probabilities of the round before
+
+  // acc += V^T P^T for the value window staged at `vtile`.
+  auto accumulate_values = [&](const uint16_t* vtile, const Frag8 p0, const Frag8 p1) {
+    const uint16_t* vrow = vtile + col * V_ROW + 8 * half;
+#pragma unroll
+    for (int t = 0; t < NT32; ++t) {
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(vrow + 32 * t * V_ROW)), as_bf16x8(p0),
+                                                        acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(vrow + 32 * t * V_ROW + 16)), as_bf16x8(p1),
+                                                        acc[t], 0, 0, 0);
+    }
+  };
+
+  auto round = [&](auto parity, int i) {
+    constexpr int A = decltype(parity)::value;  // i % 2
+    constexpr int B = A ^ 1;
+    const int w = begin + i * WINDOW_KEYS;
+    fetch_keys(kr[B], geo, window_at(i + 3), lo_first, p_last, wave, lane, page3);
+    fetch_values(vr[B], geo, window_at(i + 1), lo_first, p_last, wave, lane, page1);
+    page1 = page2;
+    page2 = page3;
+    page3 = page4;
+    page4 = page_of_chunk(geo, window_at(i + 5), wave);  // asked for now, used a round from now
+    if (wave_live) {
+      if (!interior(w)) {
+        asm volatile("" ::: "memory");  // keeps this a branch: as selects it would cost every window 64 instructions
+        wide_mask(s[A], w, half, lo_col, p_col);
+      }
+      // The column's largest score here, over the lane's 16 and those of lane ^ 32.
+      float mx = fmaxf(fmaxf(s[A][0], s[A][1]), s[A][2]);
+#pragma unroll
+      for (int e = 3; e < 15; e += 2) mx = fmaxf(fmaxf(mx, s[A][e]), s[A][e + 1]);
+      mx = fmaxf(mx, s[A][15]);
+      float xa, xb;
+      swap_rows(mx, true, xa, xb);
+      mx = max_of_numbers(xa, xb) * scale_log2;  // the scale is positive: the maximum commutes with it
+      const bool moves = mx > m + WIDE_RESCALE_SLACK;
+      if (__any(moves)) {
+        // Some column's reference moves: the values of the window before are accumulated at
+        // once, with the probabilities that belong to the old reference, then everything so far
+        // is rescaled.  Lanes whose scores stayed below the slack keep their reference (a factor
+        // of exactly 1; a column that has seen nothing yet and sees nothing here must not form
+        // -inf - -inf).
+        accumulate_values(vs + B * V_TILE, pp0, pp1);
+        pp0 = pp1 = Frag8{0u, 0u, 0u, 0u};
+        const float alpha = moves ? fast_exp2(m - mx) : 1.f;  // 0 for a column that had seen nothing
+        m = moves ? mx : m;
+        l *= alpha;
+#pragma unroll
+        for (int t = 0; t < NT32; ++t) acc[t] *= alpha;
+      }
+      // From here to the end of the round's products: no branch, so that the compiler may
+      // interleave the three independent strands as asked below.  The two products alternate in
+      // program order: the scores are one chain of dependent matrix instructions, the values'
+      // are D / 32 short ones.
+      {
+        const uint16_t* krow = ks + B * K_TILE + col * K_ROW + 8 * half;
+        const uint16_t* vrow = vs + B * V_TILE + col * V_ROW + 8 * half;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[B][e] = 0.f;
+        static_assert(KJ16 == 2 * NT32, "one step of each product per turn");
+#pragma unroll
+        for (int j = 0; j < KJ16; ++j) {
+          s[B] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(krow + 16 * j)), as_bf16x8(qf[j]), s[B], 0, 0, 0);
+          acc[j / 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(vrow + 32 * (j / 2) * V_ROW + 16 * (j & 1))),
+                                                              as_bf16x8((j & 1) ? pp1 : pp0), acc[j / 2], 0, 0, 0);
+        }
+      }
+      const float m_use = (m == -INFINITY) ? 0.f : m;  // nothing visible so far: contribute zeros
+      float sum0 = 0.f, sum1 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        s[A][e] = fast_exp2(fmaf(s[A][e], scale_log2, -m_use));
+        s[A][e + 1] = fast_exp2(fmaf(s[A][e + 1], scale_log2, -m_use));
+        sum0 += s[A][e];
+        sum1 += s[A][e + 1];
+      }
+      l += sum0 + sum1;
+      pp0 = Frag8{pack2(s[A][0], s[A][1]), pack2(s[A][2], s[A][3]), pack2(s[A][4], s[A][5]), pack2(s[A][6], s[A][7])};
+      pp1 = Frag8{pack2(s[A][8], s[A][9]), pack2(s[A][10], s[A][11]), pack2(s[A][12], s[A][13]),
+                  pack2(s[A][14], s[A][15])};
+      // Order asked of the scheduler: a few LDS reads ahead, then per matrix instruction (which
+      // occupies its unit for 32 cycles) one more LDS read and three vector instructions (4 to 8
+      // cycles each).
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // DS read
+#pragma unroll
+      for (int k = 0; k < 2 * KJ16; ++k) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        if (k < 2 * KJ16 - 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // VALU
+      }
+    }
+    stage_keys(ks + A * K_TILE, kr[A], wave, lane);
+    stage_values(vs + A * V_TILE, vr[A], window_at(i), lo_first, p_last, wave, lane);
+    __syncthreads();
+  };
+  const int rounds = (end - begin + WINDOW_KEYS - 1) / WINDOW_KEYS;
+  for (int i = 0; i < rounds; i += 2) {
+    round(std::integral_constant<int, 0>{}, i);
+    if (i + 1 < rounds) round(std::integral_constant<int, 1>{}, i + 1);
+  }
+  // The last window's values are still to be accumulated.
+  if (wave_live) accumulate_values(vs + ((rounds - 1) & 1) * V_TILE, pp0, pp1);
+
+  float la, lb;
+  swap_rows(l, true, la, lb);
+  if (col_valid && wave_live) {
+    const float inv = 1.f / (la + lb);
+    uint16_t* orow = out + ((size_t)(row0 + col) * heads + kvh * gsize + hg) * D + 4 * half;
+#pragma unroll
+    for (int t = 0; t < NT32; ++t) {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        // registers 4 a .. 4 a + 3 of tile t: head dimensions 32 t + 8 a + 4 half + 0..3
+        *reinterpret_cast<u32x2*>(orow + 32 * t + 8 * a) =
+            Frag4{pack2(acc[t][4 * a] * inv, acc[t][4 * a + 1] * inv), pack2(acc[t][4 * a + 2] * inv, acc[t][4 * a + 3] * inv)};
+      }
+    }
+  }
+}
+
+static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t* q, long q_stride,
+                               const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
+                               int table_width, const int* query_start_loc, const int* context_lens,
+                               const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
+                               float scale_log2, int window) {
+  constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
+  static_assert(lds <= 64 * 1024, "two workgroups' staged windows must fit in LDS");
+  constexpr int HW = STAGE_WAVES;
+  const int gsize = heads / kv_heads;
+  const int chunks = (gsize + HW - 1) / HW;
+  const long long total = (long long)num_blocks * kv_heads * chunks;
+  if (total > 0x7fffffffLL) return TS_ERR_SHAPE;
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int device = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return TS_ERR_LAUNCH;
+    compute_units = prop.multiProcessorCount;
+  }
+  const int pair_blocks = total <= 2LL * compute_units ? 1 : 0;
+  hipLaunchKernelGGL(prefill_wide_kernel, dim3((unsigned)total), dim3(HW * TS_WAVE), lds, stream, out, q, q_stride,
+                     k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks, num_blocks,
+                     pair_blocks, heads, kv_heads, shift, scale_log2, window);
+  return ts_launch_status();
+}
+#endif  // wide prefill
+
 }  // namespace
 
 // Decode attention for the requests seq_begin .. seq_begin + requests - 1 of the step, each of
@@ -915,13 +1307,24 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
   return ts_launch_status();
 }
 
-// Prefill attention for `num_blocks` blocks of 16 consecutive rows; blocks [num_blocks, 2] holds
-// (request index, first row) of each, rows being token rows of the step.  Writes the rows of
+// Prefill attention for `num_blocks` blocks of `block_rows` consecutive rows (16 or 32: what
+// ts_attention_prefill_rows_d says for the geometry); blocks [num_blocks, 2] holds (request
+// index, first row) of each, rows being token rows of the step.  Writes the rows of
 // `out [T, heads * D]` the blocks cover.
+// Rows per block that ts_attention_prefill_d<D> wants in `blocks` for this geometry.
+extern "C" int TS_SYM(ts_attention_prefill_rows_d)(int heads, int kv_heads) {
+#ifdef TS_WIDE_PREFILL
+  if (kv_heads >= 1 && heads % kv_heads == 0 && heads / kv_heads >= 3) return WIDE_ROWS;
+#endif
+  (void)heads;
+  (void)kv_heads;
+  return 16;
+}
+
 extern "C" int TS_SYM(ts_attention_prefill_d)(
     void* out, const void* q, long q_stride, const void* k_pages, const void* v_pages, const int* block_table,
     int table_width, const int* query_start_loc, const int* context_lens, const int* blocks, int num_blocks,
-    int heads, int kv_heads, int block_size, float scale, int window, hipStream_t stream) {
+    int block_rows, int heads, int kv_heads, int block_size, float scale, int window, hipStream_t stream) {
   if (num_blocks == 0) return TS_OK;
   if (!out || !q || !k_pages || !v_pages || !block_table || !query_start_loc || !context_lens || !blocks)
     return TS_ERR_ARG;
@@ -930,6 +1333,13 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   int shift = 0;
   while ((1 << shift) < block_size) ++shift;
   const int gsize = heads / kv_heads;
+  if (block_rows != TS_SYM(ts_attention_prefill_rows_d)(heads, kv_heads)) return TS_ERR_ARG;
+#ifdef TS_WIDE_PREFILL
+  if (gsize >= 3)
+    return launch_prefill_wide(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
+                               (const uint16_t*)v_pages, block_table, table_width, query_start_loc, context_lens,
+                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+#endif
   // Three or more query heads per KV head: workgroups of four wavefronts, one or two heads each,
   // share every window of keys and values through LDS.
   if (gsize >= 3) {

@@ -68,8 +68,9 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
                                              c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                              c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
         f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
-                                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float,
+                                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                               c_int, c_void_p],
+        f"ts_attention_prefill_rows_d{head_dim}": [c_int, c_int],
     }
 
 
@@ -434,16 +435,19 @@ class Ops:
                   requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
                   _ptr(max_context_dev), self.stream()), "ts_attention_decode")
 
-    #: Rows of one request that a wavefront of the prefill attention kernel handles.
-    prefill_block_rows = 16
+    def prefill_block_rows(self, head_dim: int, heads: int, kv_heads: int) -> int:
+        """Consecutive rows of one request that a wavefront of the prefill attention kernel
+        handles for this geometry (16 or 32): the length of the blocks its work list is made of."""
+        lib = load_module(build.attention_module(head_dim))
+        return int(getattr(lib, f"ts_attention_prefill_rows_d{head_dim}")(heads, kv_heads))
 
-    def prefill_blocks(self, query_lens, context_lens) -> torch.Tensor:
+    def prefill_blocks(self, query_lens, context_lens, rows: int) -> torch.Tensor:
         """The work list of :meth:`attention_prefill` for the multi-token requests at the front
         of a step (their numbers of new tokens and their contexts after the step): int32
-        ``[n, 2]`` on the device, (request index, first row) of every block of
-        ``prefill_block_rows`` rows, those that see the most keys first, so the long ones start
+        ``[n, 2]`` on the device, (request index, first row) of every block of ``rows`` rows
+        (:meth:`prefill_block_rows`), those that see the most keys first, so the long ones start
         early and the short ones fill the tail of the launch."""
-        blocks = prefill_block_list(query_lens, context_lens, self.prefill_block_rows)
+        blocks = prefill_block_list(query_lens, context_lens, rows)
         return torch.tensor(blocks, dtype=torch.int32).view(-1, 2).to(self.device)
 
     def attention_prefill(
@@ -461,10 +465,11 @@ class Ops:
         scale: float,
         window: int | None,
         max_context: int,
+        block_rows: int = 16,
     ) -> None:
-        """Matrix-core attention for blocks of 16 consecutive rows of multi-token requests:
-        ``blocks [n, 2]`` holds (request index, first row) of each; writes those rows of
-        ``out [T, heads * D]``."""
+        """Matrix-core attention for blocks of ``block_rows`` consecutive rows of multi-token
+        requests (what :meth:`prefill_block_rows` says for the geometry): ``blocks [n, 2]`` holds
+        (request index, first row) of each; writes those rows of ``out [T, heads * D]``."""
         _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens, blocks)
         _i32(block_table, "block_table")
         _i32(query_start_loc, "query_start_loc")
@@ -479,11 +484,13 @@ class Ops:
         _need(heads % kv_heads == 0 and block_table.dim() == 2, "heads / block table do not fit")
         _need(blocks.dim() == 2 and blocks.shape[1] == 2, "blocks must be [n, 2]")
         _need(max_context <= block_table.shape[1] * block_size, "block table does not cover the context")
+        _need(block_rows == self.prefill_block_rows(head_dim, heads, kv_heads),
+              f"blocks of {block_rows} rows are not what the kernel for this geometry takes")
         lib = load_module(build.attention_module(head_dim))
         fn = getattr(lib, f"ts_attention_prefill_d{head_dim}")
         _check(fn(_ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                   block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), _ptr(blocks), blocks.shape[0],
-                  heads, kv_heads, block_size, float(scale), int(window or 0), self.stream()),
+                  block_rows, heads, kv_heads, block_size, float(scale), int(window or 0), self.stream()),
                "ts_attention_prefill")
 
     #: Fewest keys worth a wavefront of its own.

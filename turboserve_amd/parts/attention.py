@@ -116,12 +116,13 @@ class GroupedQueryAttention(Mixer):
         if fast:
             out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
             if ctx.num_prefill_seqs > 0:
-                # The launch's list of row blocks is the same for every layer of the step.
-                blocks = ctx.derive("attention_prefill_blocks", lambda step: ops.prefill_blocks(
-                    step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs]))
+                # The launch's list of row blocks is the same for every layer with this geometry.
+                rows = ops.prefill_block_rows(self.head_dim, self.num_heads, self.num_kv_heads)
+                blocks = ctx.derive(("attention_prefill_blocks", rows), lambda step: ops.prefill_blocks(
+                    step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs], rows))
                 ops.attention_prefill(
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
-                    blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len,
+                    blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len, rows,
                 )
             if ctx.num_decode_seqs > 0:
                 ops.attention_decode(

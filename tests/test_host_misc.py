@@ -296,3 +296,43 @@ def test_end_tokens_are_the_configs_and_the_tokenizers(tmp_path):
     assert resolve((), None) == frozenset() and resolve((7, 9), None) == frozenset({7, 9})
     assert resolve((1,), SimpleNamespace(eos_token_id=[4, 5])) == frozenset({1, 4, 5})
     assert LLMEngine._resolve_eos_token_ids(SimpleNamespace(model_config={"no": "attribute"}, tokenizer=loaded)) == frozenset({3})
+
+
+def test_kernel_shares_of_a_trace(tmp_path):
+    """The per-kernel table of a ``rocprofv3 --kernel-trace`` CSV: the last steps of the trace,
+    a step ending with the marker kernel; kernels grouped by short name and grid."""
+    from turboserve_amd.profiling import format_shares, short_name, step_shares
+
+    assert short_name("void (anonymous namespace)::gemm_tiled_kernel<5, 2>(float*, unsigned short*)") == "gemm_tiled_kernel<5, 2>"
+    assert short_name("(anonymous namespace)::decode_kernel(float*, int)") == "decode_kernel"
+    assert short_name("void at::native::vectorized_elementwise_kernel<8, at::native::FillFunctor<c10::BFloat16>, std::array<char*, 1ul> >(int)"
+                      ).startswith("at::native::vectorized_elementwise_kernel<8, at::native::FillFunctor")
+    header = ("Kind,Agent_Id,Queue_Id,Stream_Id,Thread_Id,Dispatch_Id,Kernel_Id,Kernel_Name,Correlation_Id,Start_Timestamp,"
+              "End_Timestamp,LDS_Block_Size,Scratch_Size,VGPR_Count,Accum_VGPR_Count,SGPR_Count,Workgroup_Size_X,"
+              "Workgroup_Size_Y,Workgroup_Size_Z,Grid_Size_X,Grid_Size_Y,Grid_Size_Z")
+    rows, clock = [], 1000
+
+    def kernel(name, grid, duration):
+        nonlocal clock
+        rows.append(f'"KERNEL_DISPATCH","Agent 1",1,0,1,{len(rows)},1,"{name}",0,{clock},{clock + duration},0,0,8,0,16,64,1,1,{grid},1,1')
+        clock += duration + 100
+
+    kernel("void setup_kernel(int)", 64, 50_000)  # before the steps: not counted
+    for step in range(3):
+        for _ in range(2):
+            kernel("void (anonymous namespace)::gemm_tiled_kernel<5, 2>(float*)", 60672, 50_000)
+            kernel("void (anonymous namespace)::gemm_tiled_kernel<5, 2>(float*)", 243456, 10_000)  # same kernel, another product
+        kernel("void argmax_rows_kernel(int*, float const*, int const*)", 512, 5_000)
+    trace = tmp_path / "1_kernel_trace.csv"
+    trace.write_text(header + "\n" + "\n".join(rows) + "\n")
+    result = step_shares(trace, steps=2)
+    assert result.steps == 2 and result.kernels_per_step == 5 and abs(result.busy_us - 125.0) < 1e-9
+    first, second, third = result.rows
+    assert (first.name, first.grid, first.calls_per_step, first.average_us, first.per_step_us) == (
+        "gemm_tiled_kernel<5, 2>", (60672, 1, 1), 2, 50.0, 100.0)
+    assert second.grid == (243456, 1, 1) and second.per_step_us == 20.0 and third.name == "argmax_rows_kernel"
+    assert abs(first.share - 0.8) < 1e-9
+    text = format_shares(result, top=2)
+    assert "| `gemm_tiled_kernel<5, 2>` | 60672, 1, 1 | 2 | 50.0 | 100.0 | 80.0% |" in text and "1 other kernels" in text
+    with pytest.raises(ValueError, match="not enough"):
+        step_shares(trace, steps=3)

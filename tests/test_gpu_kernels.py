@@ -84,11 +84,12 @@ def test_embed_swiglu_gather(ops, dtype):
     zero_up = gu.clone()
     zero_up[:, 200:] = 0
     assert float(ops.swiglu(zero_up.to(DEV)).abs().max()) == 0.0
-    # the same values with gate and up alternating, for a width that takes the 4-wide kernel and one that does not
-    for inter in (200, 201):
-        gu = torch.randn(7, 2 * inter, generator=g).to(dtype)
+    # the same values with gate and up alternating, for widths that take the 8-wide kernel (bfloat16), the
+    # 4-wide one and neither, over more rows than a workgroup has threads
+    for rows, inter in ((7, 200), (7, 201), (7, 204), (300, 72)):
+        gu = torch.randn(rows, 2 * inter, generator=g).to(dtype)
         want = torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]
-        pairs = torch.stack([gu[:, :inter], gu[:, inter:]], dim=2).reshape(7, 2 * inter).contiguous()
+        pairs = torch.stack([gu[:, :inter], gu[:, inter:]], dim=2).reshape(rows, 2 * inter).contiguous()
         halves = ops.swiglu(gu.to(DEV)).cpu()
         torch.testing.assert_close(halves.float(), want, **tol(dtype))
         assert torch.equal(ops.swiglu(pairs.to(DEV), paired=True).cpu(), halves)
@@ -438,6 +439,9 @@ ATTENTION_GEOMETRIES = [
     (9, 3, 32, 16),     # G = 3 at the smallest head size of the 32-tokens-per-wavefront prefill kernel
     (10, 2, 96, 32),    # G = 5 (two chunks of four heads, the second with one live wavefront), head size 96
     (40, 8, 128, 16),   # G = 5 on 8 KV heads, as the 14B and 32B shapes
+    (14, 2, 64, 8),     # G = 7 on pages of 8 keys: the prefill kernel's wavefronts fetch for themselves
+    (28, 2, 64, 32),    # G = 14: two workgroups of seven heads and a feeding wavefront per KV head
+    (16, 1, 32, 16),    # G = 16: three workgroups of six heads, the last with four live ones
 ]
 
 
@@ -549,6 +553,24 @@ def test_prefill_block_rows_follow_the_geometry(ops):
         ops.attention_prefill(out, case.dev(case.q), 14 * 128, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
                               case.ints(case.qsl), case.ints([40]), case.ints([(0, 0), (0, 16), (0, 32)]), 14, 128 ** -0.5,
                               None, 40, 16)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,tokens", [(14, 2, 128, 1200), (14, 2, 128, 3100), (14, 2, 64, 4200)])
+def test_attention_prefill_mfma_every_launch_plan(ops, heads, kv_heads, dim, tokens):
+    """The 32-tokens-per-wavefront kernel picks its form by the size of the grid (on 256 compute
+    units: 1,200 tokens, fed workgroups on part of the device; 3,100 tokens, self-fed workgroups
+    with heavy and light blocks paired; 4,200 tokens, more fed workgroups than compute units).
+    One prompt each, beside a short portion at the end of another request."""
+    seqs = [(tokens, tokens), (900, 70)]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, 16, seqs, None, seed=tokens)
+    rows, blocks = prefill_blocks_of(ops, case, heads, kv_heads, dim, seqs)
+    assert rows == 32
+    out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints([c for c, _ in seqs]), case.ints(blocks), heads, dim ** -0.5, None, tokens, rows,
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
 
 
 def test_attention_prefill_mfma_far_key(ops):

@@ -927,16 +927,36 @@ __device__ __forceinline__ int page_of_chunk(const PageGeometry& g, int w, int w
   return g.table[__builtin_amdgcn_readfirstlane(w + KEYS_PER_WAVE * wave) >> g.block_shift];
 }
 
+// A lane's 32-bit offset as the compiler must see it for a load to take a scalar base and this
+// offset as they are: widened next to the load.  Widened once before the loop (where the
+// compiler would move it, the offset being the same every round) it becomes a 64-bit register
+// pair, and every load needs a 64-bit addition first.
+__device__ __forceinline__ size_t lane_offset(uint32_t offset) {
+  asm volatile("" : "+v"(offset));
+  return offset;
+}
+
+// Byte address of the first key row (or, for values, of head dimension 0's first value) of the
+// chunk of eight keys that begins at `first_key` on page `page`: all of it the same in every lane,
+// so it is worked out by the scalar unit, and a lane adds a 32-bit offset of its own.
+__device__ __forceinline__ const char* chunk_base(const uint16_t* pages, const PageGeometry& g, long long page,
+                                                  int first_key, int key_stride) {
+  const long long row = ((page * g.kv_heads + g.kvh) << g.block_shift) * D;
+  return reinterpret_cast<const char*>(pages) + 2 * (row + (long long)(first_key & g.block_mask) * key_stride);
+}
+
+// INSIDE: the caller knows that the window lies within lo..last, and nothing is tested.
+template <bool INSIDE>
 __device__ __forceinline__ void fetch_keys(StagedKeys& r, const PageGeometry& g, int w, int lo, int last, int wave,
                                            int lane, int page_id) {
   const int first_key = w + KEYS_PER_WAVE * wave;  // the same in every lane of the wavefront
-  if (w >= lo && w + WINDOW_KEYS - 1 <= last) {
-    const long long page = page_id;
-    const uint16_t* kbase = g.k_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D +
-                            (long long)(first_key & g.block_mask) * D;
+  if (INSIDE || (w >= lo && w + WINDOW_KEYS - 1 <= last)) {
+    const char* kbase = chunk_base(g.k_pages, g, page_id, first_key, D);
 #pragma unroll
-    for (int i = 0; i < K_EACH; ++i)
-      r.k[i] = load8(kbase + 8 * min(lane + i * TS_WAVE, K_WAVE_PIECES - 1));  // spare lanes repeat the last piece
+    for (int i = 0; i < K_EACH; ++i) {
+      uint32_t offset = 16u * (uint32_t)min(lane + i * TS_WAVE, K_WAVE_PIECES - 1);  // spare lanes repeat the last piece
+      r.k[i] = *reinterpret_cast<const u32x4*>(kbase + lane_offset(offset));
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < K_EACH; ++i) {
@@ -949,20 +969,23 @@ __device__ __forceinline__ void fetch_keys(StagedKeys& r, const PageGeometry& g,
   }
 }
 
+template <bool INSIDE>
 __device__ __forceinline__ void fetch_values(StagedValues& r, const PageGeometry& g, int w, int lo, int last, int wave,
                                              int lane, int page_id) {
   const int first_key = w + KEYS_PER_WAVE * wave;
   int chunk = first_key;
   long long page = page_id;
-  if (!(w >= lo && w + WINDOW_KEYS - 1 <= last)) {
+  if (!INSIDE && !(w >= lo && w + WINDOW_KEYS - 1 <= last)) {
     const bool live = first_key + 7 >= lo && first_key <= last;
-    chunk = live ? first_key : (live_key(first_key, w, lo, last) & ~7);
-    page = g.table[__builtin_amdgcn_readfirstlane(chunk) >> g.block_shift];
+    chunk = __builtin_amdgcn_readfirstlane(live ? first_key : (live_key(first_key, w, lo, last) & ~7));
+    page = g.table[chunk >> g.block_shift];
   }
-  const uint16_t* vbase = g.v_pages + ((page * g.kv_heads + g.kvh) << g.block_shift) * D + (chunk & g.block_mask);
+  const char* vbase = chunk_base(g.v_pages, g, page, chunk, 1);
 #pragma unroll
-  for (int i = 0; i < V_EACH; ++i)
-    r.v[i] = load8(vbase + ((long long)min(lane + i * TS_WAVE, D - 1) << g.block_shift));
+  for (int i = 0; i < V_EACH; ++i) {
+    const uint32_t offset = 2u * ((uint32_t)min(lane + i * TS_WAVE, D - 1) << g.block_shift);
+    r.v[i] = *reinterpret_cast<const u32x4*>(vbase + lane_offset(offset));
+  }
 }
 
 // The halves of stage_window, keys in the row order of the 32-row score tile (wide_key_row).
@@ -977,10 +1000,11 @@ __device__ __forceinline__ void stage_keys(uint16_t* ks, const StagedKeys& r, in
   }
 }
 
+template <bool INSIDE>
 __device__ __forceinline__ void stage_values(uint16_t* vs, const StagedValues& r, int w, int lo, int last, int wave,
                                              int lane) {
   const int chunk = w + KEYS_PER_WAVE * wave;
-  const bool edge = w < lo || w + WINDOW_KEYS - 1 > last;
+  const bool edge = !INSIDE && (w < lo || w + WINDOW_KEYS - 1 > last);
 #pragma unroll
   for (int i = 0; i < V_EACH; ++i) {
     const int d = lane + i * TS_WAVE;
@@ -1028,22 +1052,71 @@ __device__ __forceinline__ void wide_scores(f32x16& s, const uint16_t* ks, const
     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(load8(krow + 16 * j)), as_bf16x8(qf[j]), s, 0, 0, 0);
 }
 
-__global__ void __launch_bounds__(STAGE_WAVES * TS_WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// All four pieces of a window that lies inside lo..last, for the wavefront that feeds a
+// workgroup.  Pages hold 16 keys or more there, so two neighbouring pieces lie on one page, next
+// to each other: `page[h]` is the page of the window's keys 16 h .. 16 h + 15, and a half costs
+// one address worked out by the scalar unit; its loads differ in their constant offsets.
+__device__ __forceinline__ void fetch_keys_halves(StagedKeys (&r)[4], const PageGeometry& g, int w, int lane,
+                                                  const int (&page)[2]) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const char* base = chunk_base(g.k_pages, g, page[h], w + 16 * h, D);
+#pragma unroll
+    for (int i = 0; i < K_EACH; ++i) {
+      const uint32_t offset = 16u * (uint32_t)min(lane + i * TS_WAVE, K_WAVE_PIECES - 1);
+      const char* at = base + lane_offset(offset);
+      r[2 * h].k[i] = *reinterpret_cast<const u32x4*>(at);
+      r[2 * h + 1].k[i] = *reinterpret_cast<const u32x4*>(at + KEYS_PER_WAVE * D * 2);
+    }
+  }
+}
+
+__device__ __forceinline__ void fetch_values_halves(StagedValues (&r)[4], const PageGeometry& g, int w, int lane,
+                                                    const int (&page)[2]) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const char* base = chunk_base(g.v_pages, g, page[h], w + 16 * h, 1);
+#pragma unroll
+    for (int i = 0; i < V_EACH; ++i) {
+      const uint32_t offset = 2u * ((uint32_t)min(lane + i * TS_WAVE, D - 1) << g.block_shift);
+      const char* at = base + lane_offset(offset);
+      r[2 * h].v[i] = *reinterpret_cast<const u32x4*>(at);
+      r[2 * h + 1].v[i] = *reinterpret_cast<const u32x4*>(at + KEYS_PER_WAVE * 2);
+    }
+  }
+}
+
+// A window is fetched and staged in WINDOW_KEYS / KEYS_PER_WAVE pieces of eight keys.  In the
+// self-fed form of the kernel below each of a workgroup's four wavefronts moves one piece beside
+// its head's arithmetic.  In the fed form one more wavefront moves all four pieces and does
+// nothing else, and up to seven wavefronts of heads do nothing but arithmetic: a wavefront issues
+// at most one instruction every four cycles whatever its kind, and the address arithmetic, loads
+// and LDS writes of a round cost a self-fed wavefront as much time as its matrix instructions.
+// Eight wavefronts of this register size fill a compute unit (two per SIMD).  The fed form
+// wants pages of 16 keys or more (see fetch_keys_halves).
+constexpr int WIDE_PIECES = WINDOW_KEYS / KEYS_PER_WAVE;
+constexpr int FED_MAX_HEADS = 7;
+constexpr int FED_MIN_HEADS = 5;  // fewer heads beside the feeder leave SIMDs with one wavefront
+
+template <bool FED>
+__global__ void __launch_bounds__((FED ? FED_MAX_HEADS + 1 : STAGE_WAVES) * TS_WAVE)
+    __attribute__((amdgpu_waves_per_eu(2, 2)))
 prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long q_stride,
                     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                     const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
                     const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
-                    int pair_blocks, int heads, int kv_heads, int block_shift, float scale_log2, int window) {
+                    int pair_blocks, int group_heads, int heads, int kv_heads, int block_shift, float scale_log2,
+                    int window) {
   extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
   uint16_t* ks = staged;
   uint16_t* vs = staged + 2 * K_TILE;
   const int lane = threadIdx.x & (TS_WAVE - 1);
-  const int wave = threadIdx.x / TS_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TS_WAVE);  // known to be the same in every lane
   const int col = lane & 31;
   const int half = lane >> 5;
   const int gsize = heads / kv_heads;
-  constexpr int HW = STAGE_WAVES;
-  const int head_chunks = (gsize + HW - 1) / HW;
+  // group_heads: the heads a workgroup serves, one per wavefront (self-fed: four).
+  const int head_chunks = (gsize + group_heads - 1) / group_heads;
   // Workgroup id -> (block, KV head, chunk of its query heads) and the pairing of heavy and
   // light blocks: as in prefill_shared_kernel.
   const int lanes_y = kv_heads * head_chunks;
@@ -1051,8 +1124,10 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   int block = blockIdx.x / lanes_y;
   if (pair_blocks && block >= (num_blocks + 1) / 2) block = num_blocks - 1 - (block - (num_blocks + 1) / 2);
   const int kvh = y / head_chunks;
-  const int hg = (y % head_chunks) * HW + wave;  // this wavefront's head within the KV head's group
-  const bool wave_live = hg < gsize;
+  const bool feeder = FED && wave == group_heads;  // the wavefront that only moves windows
+  const bool feeds = !FED || feeder;
+  const int hg = (y % head_chunks) * group_heads + wave;  // this wavefront's head within the KV head's group
+  const bool wave_live = !feeder && hg < gsize;
   const int seq = blocks[2 * block];
   const int row0 = blocks[2 * block + 1];
   const int row_end = query_start_loc[seq + 1];
@@ -1097,34 +1172,58 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   // ago, go to LDS, and the keys of W(i + 3) and the values of W(i + 1) are asked for.  LDS
   // holds two windows of keys and two of values.  Windows past the last are the last again
   // (loads stay unconditional, see prefill_shared_kernel); their scores are computed and dropped.
+  const int rounds = (end - begin + WINDOW_KEYS - 1) / WINDOW_KEYS;
   const int last_window = (end - 1) & ~(WINDOW_KEYS - 1);
   auto window_at = [&](int i) { return min(begin + i * WINDOW_KEYS, last_window); };
-  StagedKeys kr[2];
-  StagedValues vr[2];
-  // The pages of this wavefront's keys in the windows W(i + 1) .. W(i + 4) of round i.
-  int page1 = page_of_chunk(geo, window_at(1), wave), page2 = page_of_chunk(geo, window_at(2), wave);
-  int page3 = page_of_chunk(geo, window_at(3), wave), page4 = page_of_chunk(geo, window_at(4), wave);
-  {
-    const int page0 = page_of_chunk(geo, window_at(0), wave);
-    fetch_keys(kr[0], geo, window_at(0), lo_first, p_last, wave, lane, page0);
-    fetch_keys(kr[1], geo, window_at(1), lo_first, p_last, wave, lane, page1);
-    fetch_values(vr[0], geo, window_at(0), lo_first, p_last, wave, lane, page0);
+  // The pieces this wavefront moves: its own one, or all of them.
+  constexpr int MOVED = FED ? WIDE_PIECES : 1;
+  auto piece_of = [&](int k) { return FED ? k : wave; };
+  StagedKeys kr[2][MOVED];
+  StagedValues vr[2][MOVED];
+  // The pages of the moved pieces in the windows W(i + 1) .. W(i + 4) of round i: the feeder
+  // keeps one per half window (the page of pieces 2 h and 2 h + 1), a self-fed wavefront its piece's.
+  constexpr int PAGES = FED ? 2 : 1;
+  auto page_piece = [&](int g) { return FED ? 2 * g : wave; };  // a piece that lies on page g of the window
+  auto page_index = [&](int k) { return FED ? k / 2 : 0; };     // which of them piece k lies on
+  int page1[PAGES], page2[PAGES], page3[PAGES], page4[PAGES];
+  if (feeds) {
+    int page0[PAGES];
+#pragma unroll
+    for (int g = 0; g < PAGES; ++g) {
+      page0[g] = page_of_chunk(geo, window_at(0), page_piece(g));
+      page1[g] = page_of_chunk(geo, window_at(1), page_piece(g));
+      page2[g] = page_of_chunk(geo, window_at(2), page_piece(g));
+      page3[g] = page_of_chunk(geo, window_at(3), page_piece(g));
+      page4[g] = page_of_chunk(geo, window_at(4), page_piece(g));
+    }
+#pragma unroll
+    for (int k = 0; k < MOVED; ++k) {
+      const int piece = piece_of(k);
+      fetch_keys<false>(kr[0][k], geo, window_at(0), lo_first, p_last, piece, lane, page0[page_index(k)]);
+      fetch_keys<false>(kr[1][k], geo, window_at(1), lo_first, p_last, piece, lane, page1[page_index(k)]);
+      fetch_values<false>(vr[0][k], geo, window_at(0), lo_first, p_last, piece, lane, page0[page_index(k)]);
+    }
   }
   // The value windows start as zeros: the first round multiplies one of them by probabilities
   // that are all zero, and what LDS held before could be anything.
-  for (int e = threadIdx.x * 8; e < 2 * V_TILE; e += STAGE_WAVES * TS_WAVE * 8)
+  for (int e = threadIdx.x * 8; e < 2 * V_TILE; e += blockDim.x * 8)
     *reinterpret_cast<u32x4*>(vs + e) = u32x4{0u, 0u, 0u, 0u};
-  stage_keys(ks, kr[0], wave, lane);
-  stage_keys(ks + K_TILE, kr[1], wave, lane);
-  fetch_keys(kr[0], geo, window_at(2), lo_first, p_last, wave, lane, page2);
+  if (feeds) {
+#pragma unroll
+    for (int k = 0; k < MOVED; ++k) {
+      stage_keys(ks, kr[0][k], piece_of(k), lane);
+      stage_keys(ks + K_TILE, kr[1][k], piece_of(k), lane);
+      fetch_keys<false>(kr[0][k], geo, window_at(2), lo_first, p_last, piece_of(k), lane, page2[page_index(k)]);
+    }
+  }
   __syncthreads();
   f32x16 s[2];  // the scores of the round's window and of the next, by parity of the round
-  wide_scores(s[0], ks, qf, col, half);
+  if (!feeder) wide_scores(s[0], ks, qf, col, half);
   __syncthreads();  // round 0 writes the window after next where these scores' keys were
   Frag8 pp0 = {0u, 0u, 0u, 0u}, pp1 = {0u, 0u, 0u, 0u};  // the probabilities of the round before
 
   // acc += V^T P^T for the value window staged at `vtile`.
-  auto accumulate_values = [&](const uint16_t* vtile, const Frag8 p0, const Frag8 p1) {
+  auto accumulate_values = [&](const uint16_t* vtile, const Frag8 p0, const Frag8 p1) __attribute__((always_inline)) {
     const uint16_t* vrow = vtile + col * V_ROW + 8 * half;
 #pragma unroll
     for (int t = 0; t < NT32; ++t) {
@@ -1135,44 +1234,72 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
     }
   };
 
-  auto round = [&](auto parity, int i) {
+  // (The lambdas are inlined by force: left as functions, everything they capture would live in
+  // memory.)
+  // Before a window's scores (held in s[A], window at `w`) become probabilities: keys a column
+  // must not see are masked, and where some column's largest score rises more than the slack
+  // above its reference, the values of the window before are accumulated at once, with the
+  // probabilities that belong to the old reference, the reference moves and everything so far is
+  // rescaled.  Lanes whose scores stayed below the slack keep their reference (a factor of exactly
+  // 1; a column that has seen nothing yet and sees nothing here must not form -inf - -inf).
+  auto look = [&](auto parity, auto steady, int w) __attribute__((always_inline)) {
+    constexpr int A = decltype(parity)::value;
+    constexpr int B = A ^ 1;
+    if (!decltype(steady)::value && !interior(w)) {
+      asm volatile("" ::: "memory");  // keeps this a branch: as selects it would cost every window 64 instructions
+      wide_mask(s[A], w, half, lo_col, p_col);
+    }
+    // The column's largest score here, over the lane's 16 and those of lane ^ 32
+    // (three at a time, as a tree: a chain of eight dependent instructions would be waited for).
+    float part[5];
+#pragma unroll
+    for (int e = 0; e < 5; ++e) part[e] = fmaxf(fmaxf(s[A][3 * e], s[A][3 * e + 1]), s[A][3 * e + 2]);
+    float mx = fmaxf(fmaxf(fmaxf(part[0], part[1]), part[2]), fmaxf(fmaxf(part[3], part[4]), s[A][15]));
+    float xa, xb;
+    swap_rows(mx, true, xa, xb);
+    mx = max_of_numbers(xa, xb) * scale_log2;  // the scale is positive: the maximum commutes with it
+    const bool moves_up = mx > m + WIDE_RESCALE_SLACK;
+    if (__any(moves_up)) {
+      accumulate_values(vs + B * V_TILE, pp0, pp1);
+      pp0 = pp1 = Frag8{0u, 0u, 0u, 0u};
+      const float alpha = moves_up ? fast_exp2(m - mx) : 1.f;  // 0 for a column that had seen nothing
+      m = moves_up ? mx : m;
+      l *= alpha;
+#pragma unroll
+      for (int t = 0; t < NT32; ++t) acc[t] *= alpha;
+    }
+  };
+  // One round.  MOVES: the wavefront fetches and stages.  COMPUTES: it has a head.  A self-fed
+  // wavefront does both.  STEADY: every window the round touches, W(i) .. W(i + 5), lies whole
+  // inside what every column of the block may see, so nothing is tested, clamped or masked.
+  auto round = [&](auto parity, auto steady, auto moves, auto computes, int i) __attribute__((always_inline)) {
     constexpr int A = decltype(parity)::value;  // i % 2
     constexpr int B = A ^ 1;
+    constexpr bool STEADY = decltype(steady)::value;
     const int w = begin + i * WINDOW_KEYS;
-    fetch_keys(kr[B], geo, window_at(i + 3), lo_first, p_last, wave, lane, page3);
-    fetch_values(vr[B], geo, window_at(i + 1), lo_first, p_last, wave, lane, page1);
-    page1 = page2;
-    page2 = page3;
-    page3 = page4;
-    page4 = page_of_chunk(geo, window_at(i + 5), wave);  // asked for now, used a round from now
-    if (wave_live) {
-      if (!interior(w)) {
-        asm volatile("" ::: "memory");  // keeps this a branch: as selects it would cost every window 64 instructions
-        wide_mask(s[A], w, half, lo_col, p_col);
-      }
-      // The column's largest score here, over the lane's 16 and those of lane ^ 32.
-      float mx = fmaxf(fmaxf(s[A][0], s[A][1]), s[A][2]);
+    auto at = [&](int k) { return STEADY ? w + k * WINDOW_KEYS : window_at(i + k); };
+    if constexpr (decltype(moves)::value) {
+      if constexpr (FED && STEADY) {
+        fetch_keys_halves(kr[B], geo, at(3), lane, page3);
+        fetch_values_halves(vr[B], geo, at(1), lane, page1);
+      } else {
 #pragma unroll
-      for (int e = 3; e < 15; e += 2) mx = fmaxf(fmaxf(mx, s[A][e]), s[A][e + 1]);
-      mx = fmaxf(mx, s[A][15]);
-      float xa, xb;
-      swap_rows(mx, true, xa, xb);
-      mx = max_of_numbers(xa, xb) * scale_log2;  // the scale is positive: the maximum commutes with it
-      const bool moves = mx > m + WIDE_RESCALE_SLACK;
-      if (__any(moves)) {
-        // Some column's reference moves: the values of the window before are accumulated at
-        // once, with the probabilities that belong to the old reference, then everything so far
-        // is rescaled.  Lanes whose scores stayed below the slack keep their reference (a factor
-        // of exactly 1; a column that has seen nothing yet and sees nothing here must not form
-        // -inf - -inf).
-        accumulate_values(vs + B * V_TILE, pp0, pp1);
-        pp0 = pp1 = Frag8{0u, 0u, 0u, 0u};
-        const float alpha = moves ? fast_exp2(m - mx) : 1.f;  // 0 for a column that had seen nothing
-        m = moves ? mx : m;
-        l *= alpha;
+        for (int k = 0; k < MOVED; ++k)
+          fetch_keys<STEADY>(kr[B][k], geo, at(3), lo_first, p_last, piece_of(k), lane, page3[page_index(k)]);
 #pragma unroll
-        for (int t = 0; t < NT32; ++t) acc[t] *= alpha;
+        for (int k = 0; k < MOVED; ++k)
+          fetch_values<STEADY>(vr[B][k], geo, at(1), lo_first, p_last, piece_of(k), lane, page1[page_index(k)]);
       }
+#pragma unroll
+      for (int g = 0; g < PAGES; ++g) {
+        page1[g] = page2[g];
+        page2[g] = page3[g];
+        page3[g] = page4[g];
+        page4[g] = page_of_chunk(geo, at(5), page_piece(g));  // asked for now, used a round from now
+      }
+    }
+    if (decltype(computes)::value && wave_live) {
+      look(parity, steady, w);
       // From here to the end of the round's products: no branch, so that the compiler may
       // interleave the three independent strands as asked below.  The two products alternate in
       // program order: the scores are one chain of dependent matrix instructions, the values'
@@ -1214,14 +1341,45 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
         __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // VALU
       }
     }
-    stage_keys(ks + A * K_TILE, kr[A], wave, lane);
-    stage_values(vs + A * V_TILE, vr[A], window_at(i), lo_first, p_last, wave, lane);
+    if constexpr (decltype(moves)::value) {
+#pragma unroll
+      for (int k = 0; k < MOVED; ++k) {
+        stage_keys(ks + A * K_TILE, kr[A][k], piece_of(k), lane);
+        stage_values<STEADY>(vs + A * V_TILE, vr[A][k], at(0), lo_first, p_last, piece_of(k), lane);
+      }
+    }
     __syncthreads();
   };
-  const int rounds = (end - begin + WINDOW_KEYS - 1) / WINDOW_KEYS;
-  for (int i = 0; i < rounds; i += 2) {
-    round(std::integral_constant<int, 0>{}, i);
-    if (i + 1 < rounds) round(std::integral_constant<int, 1>{}, i + 1);
+  // Rounds steady_from .. steady_to are steady: W(i) begins at or above the lowest key the last
+  // column sees, and W(i + 5) ends at or below the first column's own position.  Three loops,
+  // so that the steady one is a loop of its own to the compiler: general rounds up to an even
+  // round at or past steady_from, steady pairs of rounds, general rounds to the end.
+  const int steady_from = (lo_last - begin + WINDOW_KEYS - 1) / WINDOW_KEYS;
+  const int steady_to = cols == WIDE_ROWS ? (pos0 + 1 - begin) / WINDOW_KEYS - 6 : -1;
+  auto run = [&](auto moves, auto computes) __attribute__((always_inline)) {
+    constexpr std::integral_constant<int, 0> even{};
+    constexpr std::integral_constant<int, 1> odd{};
+    int i = 0;
+    for (; i < rounds && i < steady_from; i += 2) {
+      round(even, std::false_type{}, moves, computes, i);
+      if (i + 1 < rounds) round(odd, std::false_type{}, moves, computes, i + 1);
+    }
+    for (; i + 1 <= steady_to; i += 2) {
+      round(even, std::true_type{}, moves, computes, i);
+      round(odd, std::true_type{}, moves, computes, i + 1);
+    }
+    for (; i < rounds; i += 2) {
+      round(even, std::false_type{}, moves, computes, i);
+      if (i + 1 < rounds) round(odd, std::false_type{}, moves, computes, i + 1);
+    }
+  };
+  // Every wavefront of the workgroup meets the same barriers, whichever of these it runs.
+  if constexpr (!FED) {
+    run(std::true_type{}, std::true_type{});
+  } else if (feeder) {
+    run(std::true_type{}, std::false_type{});
+  } else {
+    run(std::false_type{}, std::true_type{});
   }
   // The last window's values are still to be accumulated.
   if (wave_live) accumulate_values(vs + ((rounds - 1) & 1) * V_TILE, pp0, pp1);
@@ -1247,14 +1405,10 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
                                const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
                                int table_width, const int* query_start_loc, const int* context_lens,
                                const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
-                               float scale_log2, int window) {
+                               float scale_log2, int window, int max_context) {
   constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
   static_assert(lds <= 64 * 1024, "two workgroups' staged windows must fit in LDS");
-  constexpr int HW = STAGE_WAVES;
   const int gsize = heads / kv_heads;
-  const int chunks = (gsize + HW - 1) / HW;
-  const long long total = (long long)num_blocks * kv_heads * chunks;
-  if (total > 0x7fffffffLL) return TS_ERR_SHAPE;
   static int compute_units = 0;
   if (compute_units == 0) {
     int device = 0;
@@ -1262,10 +1416,37 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
     if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return TS_ERR_LAUNCH;
     compute_units = prop.multiProcessorCount;
   }
+  // Fed workgroups take the KV head's query heads in equal shares of at most seven; with fewer
+  // than five heads beside the feeder a compute unit would be left half empty, and the self-fed
+  // form (two workgroups of four heads a compute unit) does better.  It also does better where
+  // its grid fills the device once to twice over at two workgroups a unit and the blocks are of
+  // very unequal length, so that a heavy and a light one are paired on each unit (see the kernel),
+  // while the fed grid, of one workgroup a unit, would leave units idle behind the heaviest block
+  // (a prompt of 2,048 tokens of the 7B shape: 66 against 73 us; at 4,096 tokens fed is ahead, 151
+  // against 182 us).  Blocks are of unequal length when no request has a context much longer than
+  // what the step brings in all: the longest context is no longer than the step's rows.
+  const int fed_chunks = (gsize + FED_MAX_HEADS - 1) / FED_MAX_HEADS;
+  const int fed_heads = (gsize + fed_chunks - 1) / fed_chunks;
+  const long long self_total = (long long)num_blocks * kv_heads * ((gsize + STAGE_WAVES - 1) / STAGE_WAVES);
+  const bool self_fits = self_total > compute_units && self_total <= 2LL * compute_units && max_context > 0 &&
+                         max_context <= (long long)num_blocks * WIDE_ROWS;
+  const bool fed = fed_heads >= FED_MIN_HEADS && shift >= 4 && !self_fits;
+  const int group_heads = fed ? fed_heads : STAGE_WAVES;
+  const int chunks = (gsize + group_heads - 1) / group_heads;
+  const long long total = (long long)num_blocks * kv_heads * chunks;
+  if (total > 0x7fffffffLL) return TS_ERR_SHAPE;
+  if (fed) {
+    // One workgroup fills a compute unit; blocks come heaviest first, so units that finish early
+    // take the lighter ones.
+    hipLaunchKernelGGL(prefill_wide_kernel<true>, dim3((unsigned)total), dim3((group_heads + 1) * TS_WAVE), lds, stream,
+                       out, q, q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens,
+                       blocks, num_blocks, 0, group_heads, heads, kv_heads, shift, scale_log2, window);
+    return ts_launch_status();
+  }
   const int pair_blocks = total <= 2LL * compute_units ? 1 : 0;
-  hipLaunchKernelGGL(prefill_wide_kernel, dim3((unsigned)total), dim3(HW * TS_WAVE), lds, stream, out, q, q_stride,
-                     k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks, num_blocks,
-                     pair_blocks, heads, kv_heads, shift, scale_log2, window);
+  hipLaunchKernelGGL(prefill_wide_kernel<false>, dim3((unsigned)total), dim3(STAGE_WAVES * TS_WAVE), lds, stream, out, q,
+                     q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks,
+                     num_blocks, pair_blocks, group_heads, heads, kv_heads, shift, scale_log2, window);
   return ts_launch_status();
 }
 #endif  // wide prefill
@@ -1310,7 +1491,8 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
 // Prefill attention for `num_blocks` blocks of `block_rows` consecutive rows (16 or 32: what
 // ts_attention_prefill_rows_d says for the geometry); blocks [num_blocks, 2] holds (request
 // index, first row) of each, rows being token rows of the step.  Writes the rows of
-// `out [T, heads * D]` the blocks cover.
+// `out [T, heads * D]` the blocks cover.  max_context: the longest context among the requests, or 0
+// if the caller does not know it (it only helps to choose a launch plan).
 // Rows per block that ts_attention_prefill_d<D> wants in `blocks` for this geometry.
 extern "C" int TS_SYM(ts_attention_prefill_rows_d)(int heads, int kv_heads) {
 #ifdef TS_WIDE_PREFILL
@@ -1324,7 +1506,8 @@ extern "C" int TS_SYM(ts_attention_prefill_rows_d)(int heads, int kv_heads) {
 extern "C" int TS_SYM(ts_attention_prefill_d)(
     void* out, const void* q, long q_stride, const void* k_pages, const void* v_pages, const int* block_table,
     int table_width, const int* query_start_loc, const int* context_lens, const int* blocks, int num_blocks,
-    int block_rows, int heads, int kv_heads, int block_size, float scale, int window, hipStream_t stream) {
+    int block_rows, int heads, int kv_heads, int block_size, float scale, int window, int max_context,
+    hipStream_t stream) {
   if (num_blocks == 0) return TS_OK;
   if (!out || !q || !k_pages || !v_pages || !block_table || !query_start_loc || !context_lens || !blocks)
     return TS_ERR_ARG;
@@ -1338,7 +1521,7 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   if (gsize >= 3)
     return launch_prefill_wide(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                (const uint16_t*)v_pages, block_table, table_width, query_start_loc, context_lens,
-                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window, max_context);
 #endif
   // Three or more query heads per KV head: workgroups of four wavefronts, one or two heads each,
   // share every window of keys and values through LDS.

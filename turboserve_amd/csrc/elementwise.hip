@@ -5,6 +5,8 @@
 // :290-302 (rotary, half-split pairs), :437-440 (SwiGLU) and
 // src/turboserve/engine/core/kv_cache.py:601-631 (cache write at slot = block * BS + offset).
 // Reductions, the residual sum and the rotation are computed in 32-bit whatever T is.
+#include <type_traits>
+
 #include "common.hpp"
 
 // ---------------------------------------------------------------------------------------------
@@ -323,10 +325,50 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
   Vec4Of<T>::store(out + t * inter + i, o);
 }
 
+// Eight outputs per thread with 16-byte loads and stores: bfloat16 in and out, one split, I a
+// multiple of 8 (the many-row case: a product of the library's, then this).  The same arithmetic
+// per element as above.
+__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gate_up, int inter,
+                                     size_t octets, int paired) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= octets) return;
+  const int per_row = inter / 8;
+  const size_t t = idx / per_row;
+  const int i = (int)(idx - t * per_row) * 8;
+  const bf16_t* row = gate_up + t * 2 * inter;
+  // paired: sixteen consecutive columns g0 u0 .. g7 u7; else eight of the gate and eight of the up half
+  const uint4 a = *reinterpret_cast<const uint4*>(paired ? row + 2 * i : row + i);
+  const uint4 b = *reinterpret_cast<const uint4*>(paired ? row + 2 * i + 8 : row + inter + i);
+  const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wb[4] = {b.x, b.y, b.z, b.w};
+  float g[8], u[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float a_lo = __uint_as_float(wa[e] << 16), a_hi = __uint_as_float(wa[e] & 0xffff0000u);
+    const float b_lo = __uint_as_float(wb[e] << 16), b_hi = __uint_as_float(wb[e] & 0xffff0000u);
+    if (paired) {
+      g[e] = a_lo; u[e] = a_hi; g[4 + e] = b_lo; u[4 + e] = b_hi;
+    } else {
+      g[2 * e] = a_lo; g[2 * e + 1] = a_hi; u[2 * e] = b_lo; u[2 * e + 1] = b_hi;
+    }
+  }
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  uint32_t w[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    w[e] = (uint32_t)from_float<bf16_t>(o[2 * e]).bits | ((uint32_t)from_float<bf16_t>(o[2 * e + 1]).bits << 16);
+  *reinterpret_cast<uint4*>(out + t * inter + i) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 template <typename T, typename P>
 static void launch_swiglu(void* out, const void* gate_up, int splits, long split_stride, int tokens, int inter,
                           int paired, hipStream_t stream) {
-  if (inter % 4 == 0) {
+  if (std::is_same<T, bf16_t>::value && std::is_same<P, bf16_t>::value && splits == 1 && inter % 8 == 0) {
+    const size_t octets = (size_t)tokens * (inter / 8);
+    hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
+                       (bf16_t*)out, (const bf16_t*)gate_up, inter, octets, paired);
+  } else if (inter % 4 == 0) {
     const size_t quads = (size_t)tokens * (inter / 4);
     hipLaunchKernelGGL((swiglu_vec4_kernel<T, P>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                        (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads, paired);

@@ -69,7 +69,7 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
                                              c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
         f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                              c_int, c_void_p],
+                                              c_int, c_int, c_void_p],
         f"ts_attention_prefill_rows_d{head_dim}": [c_int, c_int],
     }
 
@@ -490,7 +490,8 @@ class Ops:
         fn = getattr(lib, f"ts_attention_prefill_d{head_dim}")
         _check(fn(_ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                   block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), _ptr(blocks), blocks.shape[0],
-                  block_rows, heads, kv_heads, block_size, float(scale), int(window or 0), self.stream()),
+                  block_rows, heads, kv_heads, block_size, float(scale), int(window or 0), int(max_context),
+                  self.stream()),
                "ts_attention_prefill")
 
     #: Fewest keys worth a wavefront of its own.

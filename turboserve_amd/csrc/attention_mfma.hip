@@ -893,14 +893,15 @@ static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16
 
 // ---------------------------------------------------------------------------------------------
 // prefill, 32 tokens per wavefront (head sizes 32, 64, 96, 128; three or more query heads per
-// KV head): one workgroup of four wavefronts per (block of 32 rows, KV head, four of its query
-// heads), one head per wavefront.  S^T = K Q^T is a 32 x 32 tile of v_mfma_f32_32x32x16_bf16
+// KV head): one workgroup per (block of 32 rows, KV head, some of its query heads), one head per
+// wavefront: four wavefronts that also fetch the windows, or five to seven and one more that
+// does nothing but fetch (see WIDE_PIECES below).  S^T = K Q^T is a 32 x 32 tile of v_mfma_f32_32x32x16_bf16
 // (rows: the window's 32 keys, columns: the 32 tokens), O^T = V^T P^T four such tiles.  A column's
 // 32 scores lie in two lanes (l and l ^ 32), 16 registers each, so the softmax's maximum and sum
 // are taken inside a lane and crossed once; per score it costs under half the vector
 // instructions of the 16-column kernels, and a key row read from LDS serves 32 tokens.  Windows
-// are fetched and staged exactly as in prefill_shared_kernel (same LDS image but for the order
-// of the key rows, see wide_key_row).
+// are staged as in prefill_shared_kernel (the same LDS image but for the order of the key rows,
+// see wide_key_row).
 // ---------------------------------------------------------------------------------------------
 #if TS_HEAD_DIM % 32 == 0 && TS_HEAD_DIM <= 128
 #define TS_WIDE_PREFILL 1

@@ -143,7 +143,8 @@ def test_registry_maps_the_name_to_config_and_plan():
     config = arch.parse_config(QWEN2_RAW)
     plan = arch.build_plan(config)
     assert len(plan.layers) == 2 and [c.layer for c in plan.schedule] == [0, 1]
-    assert plan.layers[1].prefix == "model.layers.1" and plan.tie_head is False
+    assert plan.layers[1].prefix == "model.layers.1"
+    assert plan.embedding.kind == "token_table" and plan.head.kind == "norm_linear" and plan.head.params["tied_to"] is None
     mixer = plan.layers[0].block.params["mixer"]
     assert mixer.kind == "gqa_attention" and mixer.params["num_kv_heads"] == 2 and mixer.params["qkv_bias"] is True
     assert mixer.params["position"].kind == "rope" and mixer.params["position"].params["theta"] == 1000000.0

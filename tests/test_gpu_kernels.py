@@ -457,6 +457,40 @@ def test_attention_generic(ops, dtype, heads, kv_heads, dim, page, window):
     torch.testing.assert_close(got, case.expected, **tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 20])
+def test_attention_generic_with_a_bias_by_distance(ops, dtype, window):
+    """slopes[h] * (key - query position) is added to the scores before the softmax: with a steep
+    slope a head attends to its own position only, with slope 0 it is plain attention, and in
+    between it matches the formula written out."""
+    heads, kv_heads, dim, page = 6, 2, 32, 8
+    seqs = [(70, 5), (33, 33), (129, 2)]
+    case = PagedCase(dtype, heads, kv_heads, dim, page, seqs, window, seed=3)
+    slopes = torch.tensor([0.0, 0.03, 0.5, 1e4, 0.1, 2.0])
+    got = ops.paged_attention_generic(
+        case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.token_seq), case.ints(case.positions), heads, dim ** -0.5, window, slopes.to(DEV),
+    ).float().cpu().view(-1, heads, dim)
+    want = torch.empty_like(got)
+    row = 0
+    for s, (ctx, qlen) in enumerate(seqs):
+        pages = case.table[s, : -(-ctx // page)].long()
+        k = case.kp[pages].permute(0, 2, 1, 3).reshape(-1, kv_heads, dim)[:ctx].float()  # [ctx, Hkv, D]
+        v = case.vp[pages].permute(0, 3, 1, 2).reshape(-1, kv_heads, dim)[:ctx].float()
+        q = case.q[row:row + qlen].view(qlen, heads, dim).float()
+        qpos = torch.arange(ctx - qlen, ctx)
+        mask = plain.attention_mask(qpos, ctx, window)
+        distance = (torch.arange(ctx)[None, :] - qpos[:, None]).float()
+        for h in range(heads):
+            scores = (q[:, h] @ k[:, h // 3].T) * dim ** -0.5 + slopes[h] * distance
+            want[row:row + qlen, h] = torch.softmax(scores.masked_fill(~mask, float("-inf")), dim=-1) @ v[:, h // 3]
+            if h == 3:  # the steep head sees its own key only
+                torch.testing.assert_close(want[row:row + qlen, h], v[qpos, h // 3], rtol=0, atol=1e-6)
+        row += qlen
+    torch.testing.assert_close(got, want, **tol(dtype))
+    torch.testing.assert_close(got[:, 0].reshape(-1), case.expected.view(-1, heads, dim)[:, 0].reshape(-1), **tol(dtype))
+
+
 @pytest.mark.parametrize("heads,kv_heads,dim,page", ATTENTION_GEOMETRIES)
 @pytest.mark.parametrize("window", [None, 20, 300])
 def test_attention_decode_mfma(ops, heads, kv_heads, dim, page, window):

@@ -1,6 +1,7 @@
 """The parts of a model, alone and recombined: each built-in part against the plain
-implementation; a toy mixer with state of its own, a toy feed-forward with routing, a toy
-position encoding and a toy architecture made of them, all defined here and registered
+implementation; a toy mixer with state of its own, a toy feed-forward with routing, two toy
+position encodings (one added to queries and keys, one a bias inside the scores), a toy
+embedding, a toy head and a toy architecture made of them, all defined here and registered
 without touching the framework; a run order that names a layer twice and lets a
 layer read another layer's cache; long decoding and the first tokens of a sequence."""
 
@@ -136,7 +137,8 @@ def register_toy_architecture():
     from turboserve_amd.config import registry as arch_registry
     from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
     from turboserve_amd.parts import registry as part_registry
-    from turboserve_amd.parts.base import FeedForward, FixedState, Mixer, PartSpec, PositionEncoding, TensorSpec
+    from turboserve_amd.parts.base import (Embedding, FeedForward, FixedState, Head, Mixer, PartSpec, PositionEncoding,
+                                           TensorSpec)
 
     if "running_mean" not in part_registry.MIXERS:
 
@@ -235,6 +237,71 @@ def register_toy_architecture():
                 return ops.rope_store(qkv, cache.k, cache.v, None, None, ctx.positions, slots, num_heads, num_kv_heads,
                                       head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype)
 
+    if "distance_bias" not in part_registry.POSITION_ENCODINGS:
+
+        @part_registry.register_position_encoding("distance_bias")
+        class DistanceBias(PositionEncoding):
+            """A position encoding that leaves queries and keys as they are and acts inside the
+            scores: head h's score of a key ``d`` positions back is lowered by ``slopes[h] * d``."""
+
+            def __init__(self, prefix, runtime, *, slopes):
+                super().__init__(prefix, runtime)
+                self.slopes = torch.tensor(list(slopes), dtype=torch.float32, device=runtime.device)
+
+            def score_slopes(self, num_heads):
+                assert self.slopes.numel() == num_heads
+                return self.slopes
+
+            def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache):
+                ops = self.runtime.ops
+                slots = ctx.slot_mapping[cache.group] if cache.writable else None
+                return ops.rope_store(ops.dense(qkv, self.runtime.dtype), cache.k, cache.v, None, None, ctx.positions, slots,
+                                      num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1,
+                                      self.runtime.dtype)
+
+    if "scaled_table" not in part_registry.EMBEDDINGS:
+
+        @part_registry.register_embedding("scaled_table")
+        class ScaledTable(Embedding):
+            """Another embedding: the table's row times a constant."""
+
+            def __init__(self, prefix, runtime, *, vocab_size, hidden_size, multiplier):
+                super().__init__(prefix, runtime)
+                self.shape, self.multiplier, self.weight = (vocab_size, hidden_size), float(multiplier), None
+
+            def tensor_specs(self):
+                return {self.name("weight"): TensorSpec(self.shape)}
+
+            def load(self, tensors):
+                self.weight = tensors[self.name("weight")]
+
+            def forward(self, token_ids, ctx):
+                return self.runtime.ops.embed(self.weight, token_ids) * self.multiplier
+
+    if "biased_head" not in part_registry.HEADS:
+
+        @part_registry.register_head("biased_head")
+        class BiasedHead(Head):
+            """Another head: norm, a matrix of its own, a scale on the scores and a bias per token id."""
+
+            def __init__(self, prefix, runtime, *, vocab_size, hidden_size, norm, scale):
+                super().__init__(prefix, runtime)
+                self.vocab, self.hidden, self.scale = vocab_size, hidden_size, float(scale)
+                self.norm = part_registry.build_part("norm", norm, "model.norm", runtime)
+                self.weight = self.bias = None
+
+            def tensor_specs(self):
+                return {**self.norm.tensor_specs(), self.name("weight"): TensorSpec((self.vocab, self.hidden)),
+                        self.name("bias"): TensorSpec((self.vocab,))}
+
+            def load(self, tensors):
+                self.norm.load(tensors)
+                self.weight, self.bias = tensors[self.name("weight")], tensors[self.name("bias")].float()
+
+            def forward(self, stream, rows):
+                hidden = self.norm.forward_residual(stream, rows)
+                return self.runtime.ops.linear_float32_out(hidden, self.weight) * self.scale + self.bias
+
     if "ToyForCausalLM" not in arch_registry.ARCHITECTURES:
 
         def parse(data, name_or_path=""):
@@ -250,10 +317,12 @@ def register_toy_architecture():
                 "position": PartSpec("rope", {"head_dim": cfg["head_dim"], "theta": 1e4, "scaling_factor": 1.0, "max_positions": 256})})
             learned = PartSpec("gqa_attention", dict(attention.params, position=PartSpec(
                 "learned_positions", {"head_dim": cfg["head_dim"], "max_positions": 128})))
+            biased = PartSpec("gqa_attention", dict(attention.params, position=PartSpec(
+                "distance_bias", {"slopes": cfg["slopes"]})))
             toy = PartSpec("running_mean", {"hidden_size": hidden})
             routed = PartSpec("top1_experts", {"hidden_size": hidden, "intermediate_size": cfg["intermediate_size"],
                                                "num_experts": cfg["experts"]})
-            mixers = {"attention": attention, "attention_learned": learned, "state": toy}
+            mixers = {"attention": attention, "attention_learned": learned, "attention_biased": biased, "state": toy}
             layers = []
             for index, kind in enumerate(cfg["mixers"]):  # mixer and feed-forward are chosen layer by layer
                 block = PartSpec("prenorm", {"mixer": mixers[kind],
@@ -261,8 +330,12 @@ def register_toy_architecture():
                                              "mixer_norm": norm, "ff_norm": norm})
                 layers.append(LayerSpec(f"model.layers.{index}", block))
             schedule = tuple(LayerCall(layer, cache_of) for layer, cache_of in cfg["schedule"])
+            embedding = PartSpec("scaled_table", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden,
+                                                  "multiplier": cfg["embedding_multiplier"]})
+            head = PartSpec("biased_head", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden, "norm": norm,
+                                            "scale": cfg["logit_scale"]})
             return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=hidden, layers=tuple(layers), schedule=schedule,
-                             final_norm=norm, tie_head=True)
+                             embedding=embedding, head=head)
 
         arch_registry.register_architecture("ToyForCausalLM", parse, plan)
 
@@ -271,8 +344,9 @@ def toy_plain_logits(cfg, tensors, tokens):
     """The toy model by the plain functions: whole sequence, no cache."""
     values = {"heads": cfg["heads"], "kv_heads": cfg["kv_heads"], "head_dim": cfg["head_dim"], "theta": 1e4,
               "rope_factor": 1.0, "eps": cfg["eps"]}
-    h = tensors["model.embed_tokens.weight"][torch.tensor(tokens)]
+    h = tensors["model.embed_tokens.weight"][torch.tensor(tokens)] * cfg["embedding_multiplier"]
     pos = torch.arange(len(tokens))
+    distance = (pos[None, :] - pos[:, None]).float()  # [query, key]: key position less query position
     kv_of_call = {}
     for call, (layer, cache_of) in enumerate(cfg["schedule"]):
         p = f"model.layers.{layer}"
@@ -282,6 +356,8 @@ def toy_plain_logits(cfg, tensors, tokens):
             if cfg["mixers"][layer] == "attention":
                 angles = plain.rope_angles(pos, dim, 1e4)
                 encode = lambda t: plain.apply_rope(t, angles)
+            elif cfg["mixers"][layer] == "attention_biased":
+                encode = lambda t: t
             else:
                 table = tensors[f"{p}.self_attn.position_table"]
                 encode = lambda t: t + table[pos][:, None, :]
@@ -292,7 +368,16 @@ def toy_plain_logits(cfg, tensors, tokens):
                 v = (x @ tensors[f"{p}.self_attn.v_proj.weight"].T + tensors[f"{p}.self_attn.v_proj.bias"]).view(-1, kvh, dim)
                 kv_of_call[call] = (encode(k), v)
             k, v = kv_of_call[call if cache_of is None else cache_of]
-            mixed = plain.attention(q, k, v, plain.attention_mask(pos, len(tokens), None), dim ** -0.5)
+            if cfg["mixers"][layer] == "attention_biased":
+                # scores + slope * (key - query), written out: the plain attention has no such term
+                mask = plain.attention_mask(pos, len(tokens), None)
+                mixed = torch.empty_like(q)
+                for head in range(heads):
+                    scores = (q[:, head] @ k[:, head // (heads // kvh)].T) * dim ** -0.5 + cfg["slopes"][head] * distance
+                    probs = torch.softmax(scores.masked_fill(~mask, float("-inf")), dim=-1)
+                    mixed[:, head] = probs @ v[:, head // (heads // kvh)]
+            else:
+                mixed = plain.attention(q, k, v, plain.attention_mask(pos, len(tokens), None), dim ** -0.5)
             mixed = mixed.reshape(len(tokens), -1) @ tensors[f"{p}.self_attn.o_proj.weight"].T
         else:
             mean = torch.cumsum(x, dim=0) / torch.arange(1, len(tokens) + 1)[:, None]
@@ -308,18 +393,20 @@ def toy_plain_logits(cfg, tensors, tokens):
         else:
             h = h + plain.swiglu_mlp(x, *(tensors[f"{p}.mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
     h = plain.rms_norm(h, tensors["model.norm.weight"], cfg["eps"])
-    return h @ tensors["model.embed_tokens.weight"].T
+    return (h @ tensors["lm_head.weight"].T) * cfg["logit_scale"] + tensors["lm_head.bias"]
 
 
 TOY_CONFIG = {
     "architectures": ["ToyForCausalLM"], "hidden_size": 40, "intermediate_size": 56, "vocab_size": 97, "heads": 5,
     "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "experts": 3,
-    "mixers": ["attention", "state", "attention", "attention_learned"],
-    "feed_forwards": ["swiglu", "routed", "swiglu", "routed"],
+    "embedding_multiplier": 1.5, "logit_scale": 0.5, "slopes": [0.5, 0.25, 0.125, 0.0625, 0.03125],
+    "mixers": ["attention", "state", "attention", "attention_learned", "attention_biased"],
+    "feed_forwards": ["swiglu", "routed", "swiglu", "routed", "swiglu"],
     # layer 0, the stateful layer (with a routed feed-forward), layer 0 AGAIN (weights reused, a
     # cache of its own), layer 2 reading the cache of the first call instead of keeping one, then
-    # a layer whose attention takes learned positions instead of rotation.
-    "schedule": [[0, None], [1, None], [0, None], [2, 0], [3, None]],
+    # a layer whose attention takes learned positions instead of rotation, then one whose position
+    # encoding is a bias on the scores.
+    "schedule": [[0, None], [1, None], [0, None], [2, 0], [3, None], [4, None]],
 }
 
 
@@ -337,12 +424,13 @@ def test_toy_model_is_data(toy_folder):
 
     _, model = describe_model(TOY_CONFIG)
     layout = CacheLayout.from_model(model)
-    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads", "pages"]
-    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2, 4) and layout.state_entries[0][0] == 1
+    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads", "pages", "pages"]
+    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2, 4, 5) and layout.state_entries[0][0] == 1
     names = list(model.tensor_specs())
     assert "model.layers.1.self_attn.mix.weight" in names and "model.layers.2.self_attn.q_proj.weight" in names
     assert "model.layers.1.mlp.experts.2.down_proj.weight" in names and "model.layers.1.mlp.router.weight" in names
     assert "model.layers.3.self_attn.position_table" in names and "model.layers.0.mlp.gate_proj.weight" in names
+    assert "lm_head.bias" in names and "model.norm.weight" in names and names[0] == "model.embed_tokens.weight"
 
 
 @pytest.mark.parametrize("cut", ["whole", "prefix_then_single", "portions", "mixed"])
@@ -382,7 +470,7 @@ def test_toy_architecture_generates_through_the_engine_and_the_command_line(toy_
     if dtype == "bfloat16":
         # Without the routed feed-forward: a router's near-tie may fall to another expert in
         # bfloat16, which is a different function, not a rounding error.
-        dense = {**TOY_CONFIG, "feed_forwards": ["swiglu"] * 4}
+        dense = {**TOY_CONFIG, "feed_forwards": ["swiglu"] * 5}
         folder = write_random_model(dense, tmp_path / "toy_bf16", seed=5, dtype=torch.bfloat16, std=0.1)
     raw, tensors = tiny.read_model_dir(folder)
     prompts = [tiny.random_tokens(97, n, 40 + n) for n in (3, 12, 29)]

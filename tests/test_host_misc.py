@@ -12,6 +12,7 @@ from turboserve_amd.engine.detokenizer import IncrementalDetokenizer, StopString
 from turboserve_amd.engine.sequence import Sequence
 from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
 from turboserve_amd.parts.base import PartSpec
+from turboserve_amd.parts.ends import standard_ends
 from turboserve_amd.sampling.params import FinishReason, SamplingParams
 
 
@@ -228,15 +229,17 @@ def test_command_line_options_are_the_references():
 def test_the_run_order_is_data():
     norm = PartSpec("rmsnorm", {"size": 8, "eps": 1e-6})
     layers = (LayerSpec("model.layers.0", PartSpec("prenorm", {})), LayerSpec("model.layers.1", PartSpec("prenorm", {})))
-    plan = ModelPlan(vocab_size=10, hidden_size=8, layers=layers, final_norm=norm, tie_head=True,
+    ends = standard_ends(10, 8, norm, tie_head=True)
+    assert ends["head"].params["tied_to"] == "model.embed_tokens.weight"
+    plan = ModelPlan(vocab_size=10, hidden_size=8, layers=layers, **ends,
                      schedule=(LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(1, cache_of=1)))
     assert [c.layer for c in plan.schedule] == [0, 1, 0, 1]  # a layer may run twice, or read an earlier call's cache
     with pytest.raises(ValueError, match="not earlier"):
-        ModelPlan(10, 8, layers, (LayerCall(0, cache_of=0),), norm, True)
+        ModelPlan(10, 8, layers, (LayerCall(0, cache_of=0),), **ends)
     with pytest.raises(ValueError, match="names layer"):
-        ModelPlan(10, 8, layers, (LayerCall(2),), norm, True)
+        ModelPlan(10, 8, layers, (LayerCall(2),), **ends)
     with pytest.raises(ValueError, match="owns none"):
-        ModelPlan(10, 8, layers, (LayerCall(0), LayerCall(1, cache_of=0), LayerCall(0, cache_of=1)), norm, True)
+        ModelPlan(10, 8, layers, (LayerCall(0), LayerCall(1, cache_of=0), LayerCall(0, cache_of=1)), **ends)
 
 
 def test_bench_contract_on_the_host():

@@ -125,7 +125,7 @@ def test_tied_checkpoint_may_carry_the_head(tmp_path):
     model = cpu_model(config)
     report = load_model_weights(model, folder)
     assert report.ok and report.ignored == ["lm_head.weight"]
-    assert model.head is model.embedding
+    assert model.head.weight is model.embedding.weight  # one tensor, as a tied head shares the table
 
 
 def test_random_model_is_a_function_of_config_and_seed(tmp_path):

@@ -25,7 +25,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                const int* __restrict__ block_table, int table_width,
                                const int* __restrict__ token_seq, const int* __restrict__ positions,
                                int heads, int kv_heads, int dim, int block_size, float scale,
-                               int window) {
+                               int window, const float* __restrict__ slopes) {
   __shared__ float qs[ATTN_MAX_DIM];
   __shared__ float ps[ATTN_TILE];
   __shared__ long long rows[ATTN_TILE];  // per key of the tile: offset of its value column
@@ -38,6 +38,8 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int* table = block_table + (size_t)seq * table_width;
+  // A position encoding may bias the scores by the distance: + slope[h] * (key - p), in 32-bit.
+  const float slope = slopes ? slopes[h] : 0.f;
 
   const T* qrow = q + (size_t)t * q_stride + (size_t)h * dim;
   for (int d = lane; d < dim; d += ATTN_TILE) qs[d] = to_float(qrow[d]) * scale;
@@ -62,7 +64,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       const T* krow = k_pages + head_base + (long long)(key % block_size) * dim;
       float s = 0.f;
       for (int d = 0; d < dim; ++d) s = fmaf(qs[d], to_float(krow[d]), s);
-      score = s;
+      score = slopes ? fmaf(slope, (float)(key - p), s) : s;
     }
     const float m_new = fmaxf(m_run, wave_max(score));
     const float alpha = expf(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
@@ -96,21 +98,24 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
 }
 
 // out [T, Hq, D] contiguous; q rows are q_stride elements apart (the fused projection output).
+// slopes [Hq] (32-bit) or null: the score of key j for the query at position p gets
+// slopes[h] * (j - p) added.
 extern "C" int ts_paged_attention_generic(void* out, const void* q, long q_stride,
                                           const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_width,
                                           const int* token_seq, const int* positions, int tokens,
                                           int heads, int kv_heads, int dim, int block_size,
-                                          float scale, int window, int dtype, hipStream_t stream) {
+                                          float scale, int window, const float* slopes, int dtype,
+                                          hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !q || !k_pages || !v_pages || !block_table || !token_seq || !positions) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dim < 1 || dim > ATTN_MAX_DIM || block_size < 1 || table_width < 1) return TS_ERR_SHAPE;
   dim3 grid(tokens, heads), block(ATTN_TILE);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, block_size, scale, window);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, block_size, scale, window, slopes);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, block_size, scale, window);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, block_size, scale, window, slopes);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -49,7 +49,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_int, c_void_p],
+                                       c_float, c_int, c_void_p, c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -350,12 +350,19 @@ class Ops:
         heads: int,
         scale: float,
         window: int | None,
+        slopes: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """Attention of every token over the keys ``lo..position`` of its request.
 
         ``q`` is the tensor whose first ``heads * D`` elements of each ``q_stride``-long row
-        are the (already encoded) queries.  Returns ``[T, heads * D]``."""
+        are the (already encoded) queries.  ``slopes [heads]`` (32-bit), if given, biases the
+        score of key ``j`` for a query at position ``p`` by ``slopes[h] * (j - p)``.  Returns
+        ``[T, heads * D]``."""
         _gpu(q, k_pages, v_pages, block_table, token_seq, positions)
+        if slopes is not None:
+            _gpu(slopes)
+            _need(slopes.dtype == torch.float32 and slopes.is_contiguous() and slopes.numel() == heads,
+                  "slopes must be contiguous float32 [heads]")
         _i32(block_table, "block_table")
         _i32(token_seq, "token_seq")
         _i32(positions, "positions")
@@ -371,7 +378,8 @@ class Ops:
         _check(self.core.ts_paged_attention_generic(
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim,
-            block_size, float(scale), int(window or 0), dtype_code(q.dtype), self.stream()),
+            block_size, float(scale), int(window or 0), _ptr(slopes) if slopes is not None else None,
+            dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
 

@@ -1,6 +1,7 @@
-"""A decoder assembled from a plan: embedding, layers, the order they run in, final norm, head.
+"""A decoder assembled from a plan: embedding, layers, the order they run in, head.
 
-The plan is data.  ``layers`` describes each layer's block and parts; ``schedule`` is the list
+The plan is data.  ``embedding`` and ``head`` are parts like any other (for the usual pair see
+``parts.ends.standard_ends``); ``layers`` describes each layer's block and parts; ``schedule`` is the list
 of layer calls of one forward pass: it may name a layer twice (the layer's weights run twice,
 each call with a cache of its own) and a call may read the cache of an earlier call instead of
 owning one.  The reference runs its layers once each, in order, with one cache kind
@@ -19,6 +20,8 @@ from turboserve_amd.parts.base import (
     Block,
     CacheNeed,
     CacheView,
+    Embedding,
+    Head,
     PartSpec,
     ResidualStream,
     Runtime,
@@ -50,11 +53,10 @@ class ModelPlan:
     hidden_size: int
     layers: tuple[LayerSpec, ...]
     schedule: tuple[LayerCall, ...]
-    final_norm: PartSpec
-    tie_head: bool
-    embedding_name: str = "model.embed_tokens"
-    final_norm_name: str = "model.norm"
-    head_name: str = "lm_head"
+    embedding: PartSpec
+    head: PartSpec
+    embedding_prefix: str = "model.embed_tokens"
+    head_prefix: str = "lm_head"
 
     def __post_init__(self) -> None:
         for index, call in enumerate(self.schedule):
@@ -77,37 +79,34 @@ class DecoderModel:
         self.blocks: list[Block] = [
             build_part("block", layer.block, layer.prefix, runtime) for layer in plan.layers
         ]
-        self.final_norm = build_part("norm", plan.final_norm, plan.final_norm_name, runtime)
-        self.embedding: torch.Tensor | None = None
-        self.head: torch.Tensor | None = None
+        self.embedding: Embedding = build_part("embedding", plan.embedding, plan.embedding_prefix, runtime)
+        self.head: Head = build_part("head", plan.head, plan.head_prefix, runtime)
 
     # -- weights ------------------------------------------------------------------------------
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         """Every checkpoint tensor the model expects, in model order."""
-        plan = self.plan
-        specs: dict[str, TensorSpec] = {
-            f"{plan.embedding_name}.weight": TensorSpec((plan.vocab_size, plan.hidden_size))
-        }
+        specs: dict[str, TensorSpec] = dict(self.embedding.tensor_specs())
         for block in self.blocks:
             specs.update(block.tensor_specs())
-        specs.update(self.final_norm.tensor_specs())
-        if not plan.tie_head:
-            specs[f"{plan.head_name}.weight"] = TensorSpec((plan.vocab_size, plan.hidden_size))
+        for name, spec in self.head.tensor_specs().items():
+            # A head may name a tensor of another part (a tied head: the token table) and then
+            # shares it; both must expect the same thing there.
+            if name in specs and specs[name] != spec:
+                raise ValueError(f"the head expects {spec} under {name!r}, another part {specs[name]}")
+            specs[name] = spec
         return specs
 
     def ignorable_names(self) -> set[str]:
-        """Names a checkpoint may hold that the model does not read: a tied model's copy of the
-        head (the reference shares one parameter, src/turboserve/engine/model/model.py:139-142)."""
-        return {f"{self.plan.head_name}.weight"} if self.plan.tie_head else set()
+        """Names a checkpoint may hold that the model does not read (a tied head's own copy of
+        the matrix)."""
+        return self.head.ignorable_names()
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        plan = self.plan
-        self.embedding = tensors[f"{plan.embedding_name}.weight"].contiguous()
+        self.embedding.load(tensors)
         for block in self.blocks:
             block.load(tensors)
-        self.final_norm.load(tensors)
-        self.head = self.embedding if plan.tie_head else tensors[f"{plan.head_name}.weight"].contiguous()
+        self.head.load(tensors)
 
     def num_parameters(self) -> int:
         total = 0
@@ -128,7 +127,7 @@ class DecoderModel:
         plan = self.plan
         stream = tokens * plan.hidden_size * (4 + 4)
         layer = max((block.activation_bytes(tokens, itemsize) for block in self.blocks), default=0)
-        layer += self.final_norm.activation_bytes(tokens, itemsize)
+        layer += self.head.activation_bytes(tokens, itemsize)
         return 2 * (stream + layer) + requests * plan.vocab_size * 4 * 2
 
     # -- caches -------------------------------------------------------------------------------
@@ -136,7 +135,8 @@ class DecoderModel:
     def is_capturable(self) -> bool:
         """Whether single-token steps of this model may be recorded into HIP graphs: every
         part says so (``Part.capturable``)."""
-        return all(block.is_capturable() for block in self.blocks) and self.final_norm.is_capturable()
+        return (all(block.is_capturable() for block in self.blocks) and self.embedding.is_capturable()
+                and self.head.is_capturable())
 
     def cache_needs(self) -> list[CacheNeed]:
         """What each schedule entry needs a cache for (``None``: nothing, or it reads another's)."""
@@ -153,12 +153,11 @@ class DecoderModel:
         (model.py:105-107).  ``caches[i]`` is the view of schedule entry ``i``."""
         if len(caches) != len(self.plan.schedule):
             raise ValueError(f"{len(caches)} cache views for {len(self.plan.schedule)} scheduled layer calls")
-        stream = ResidualStream(self.runtime.ops.embed(self.embedding, token_ids))
+        stream = ResidualStream(self.embedding.forward(token_ids, ctx))
         for call, cache in zip(self.plan.schedule, caches):
             stream = self.blocks[call.layer].forward(stream, ctx, cache)
         return stream
 
     def logits(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
-        """Final norm and head at ``rows`` only -> 32-bit ``[n, V]`` (model.py:108, 237-244)."""
-        hidden = self.final_norm.forward_residual(stream, rows)
-        return self.runtime.ops.linear_float32_out(hidden, self.head)
+        """The head at ``rows`` only -> 32-bit ``[n, V]`` (model.py:108, 237-244)."""
+        return self.head.forward(stream, rows)

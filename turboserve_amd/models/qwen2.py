@@ -11,6 +11,7 @@ from __future__ import annotations
 from turboserve_amd.config.model_config import Qwen2Config
 from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
 from turboserve_amd.parts.base import PartSpec
+from turboserve_amd.parts.ends import standard_ends
 
 
 def qwen2_plan(config: Qwen2Config) -> ModelPlan:
@@ -53,6 +54,5 @@ def qwen2_plan(config: Qwen2Config) -> ModelPlan:
         hidden_size=config.hidden_size,
         layers=tuple(layers),
         schedule=tuple(LayerCall(i) for i in range(config.num_hidden_layers)),
-        final_norm=norm,
-        tie_head=config.tie_word_embeddings,
+        **standard_ends(config.vocab_size, config.hidden_size, norm, tie_head=config.tie_word_embeddings),
     )

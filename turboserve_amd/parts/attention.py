@@ -109,10 +109,12 @@ class GroupedQueryAttention(Mixer):
 
         bfloat16 runs use the matrix-core kernels where the geometry allows: one launch for the
         multi-token requests at the front of the batch, one for the single-token requests
-        behind them; every 32-bit run and any other geometry goes through the generic kernel."""
+        behind them; every 32-bit run, any other geometry and any position encoding that biases
+        the scores goes through the generic kernel."""
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
-        fast = ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
+        slopes = self.position.score_slopes(self.num_heads)
+        fast = slopes is None and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
         if fast:
             out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
             if ctx.num_prefill_seqs > 0:
@@ -134,5 +136,5 @@ class GroupedQueryAttention(Mixer):
             return out
         return ops.paged_attention_generic(
             qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
-            self.num_heads, self.scale, self.window,
+            self.num_heads, self.scale, self.window, slopes,
         )

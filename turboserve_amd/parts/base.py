@@ -198,6 +198,35 @@ class PositionEncoding(Part):
         returns the tensor holding the encoded queries with its row stride."""
         raise NotImplementedError
 
+    def score_slopes(self, num_heads: int) -> torch.Tensor | None:
+        """An encoding may (also, or instead) act inside the scores: ``[num_heads]`` 32-bit
+        slopes ``m`` on the device, for which the score of key ``j`` for the query at position
+        ``p`` of head ``h`` gets ``m[h] * (j - p)`` added before the softmax; ``None``: no such
+        bias.  The attention mixer hands them to a kernel that takes them."""
+        return None
+
+
+class Embedding(Part):
+    """Token ids -> what the first layer's residual stream starts as."""
+
+    def forward(self, token_ids: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+        """``token_ids [T]`` int32 -> 32-bit ``[T, H]``."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    """The residual stream after the last layer, at the rows whose scores are wanted -> 32-bit
+    scores over the vocabulary.  A head that shares a tensor with another part (a tied head
+    shares the embedding's table) names that tensor in its ``tensor_specs`` like any other."""
+
+    def forward(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        """``rows [n]`` int32 -> ``[n, V]`` 32-bit; the stream is left as it is."""
+        raise NotImplementedError
+
+    def ignorable_names(self) -> set[str]:
+        """Tensor names a checkpoint may hold for this part that it does not read."""
+        return set()
+
 
 class Mixer(Part):
     """Mixes information between the tokens of a request (attention, or anything with state)."""

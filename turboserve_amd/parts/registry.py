@@ -1,7 +1,8 @@
 """Registries from a part's kind name to its class, one per interface.
 
-A layer description names its parts by kind; adding a mixer, feed-forward, norm, position
-encoding or block arrangement is one ``register_*`` call and needs no change elsewhere.
+A layer description names its parts by kind, and so does a model for its embedding and its
+head; adding a mixer, feed-forward, norm, position encoding, block arrangement, embedding or head
+is one ``register_*`` call and needs no change elsewhere.
 """
 
 from __future__ import annotations
@@ -18,6 +19,8 @@ FEED_FORWARDS: dict[str, type] = {}
 NORMS: dict[str, type] = {}
 POSITION_ENCODINGS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
+EMBEDDINGS: dict[str, type] = {}
+HEADS: dict[str, type] = {}
 
 _TABLES = {
     "mixer": MIXERS,
@@ -25,6 +28,8 @@ _TABLES = {
     "norm": NORMS,
     "position_encoding": POSITION_ENCODINGS,
     "block": BLOCKS,
+    "embedding": EMBEDDINGS,
+    "head": HEADS,
 }
 
 
@@ -58,9 +63,17 @@ def register_block(kind: str) -> Callable[[type[T]], type[T]]:
     return _register(BLOCKS, "block", kind)
 
 
+def register_embedding(kind: str) -> Callable[[type[T]], type[T]]:
+    return _register(EMBEDDINGS, "embedding", kind)
+
+
+def register_head(kind: str) -> Callable[[type[T]], type[T]]:
+    return _register(HEADS, "head", kind)
+
+
 def build_part(role: str, spec: PartSpec, prefix: str, runtime: Runtime, **extra: Any) -> Any:
     """Instantiate ``spec`` from the registry of ``role`` (``"mixer"``, ``"feed_forward"``,
-    ``"norm"``, ``"position_encoding"`` or ``"block"``)."""
+    ``"norm"``, ``"position_encoding"``, ``"block"``, ``"embedding"`` or ``"head"``)."""
     table = _TABLES[role]
     try:
         cls = table[spec.kind]

@@ -93,6 +93,9 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--kernel-shares", metavar="TRACE.csv", default=None,
                    help="print the per-kernel table of a rocprofv3 kernel trace of a run of this program and exit")
     p.add_argument("--shares-steps", type=int, default=4, help="steps at the end of the trace that the table covers")
+    p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
+                   help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
+                        "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
     return p.parse_args()
 
 
@@ -254,6 +257,43 @@ def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True)
     return best
 
 
+def run_attention_prefill(shape: dict, tokens: int, context: int, launches: int = 15) -> dict:
+    """The prefill attention kernel alone (no model): ``tokens`` rows of one request at the end of
+    ``context`` keys on scrambled pages, random queries, keys and values; the best of ``launches``
+    launches by device events.  Flops: causal attention of the rows over what they see."""
+    import torch
+
+    from turboserve_amd.kernels.ops import Ops
+
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    dim = shape["hidden_size"] // heads
+    ops = Ops("cuda:0")
+    pages = -(-context // PAGE)
+    generator = torch.Generator(device="cuda").manual_seed(0)
+    k_pages = torch.randn(pages, kv_heads, PAGE, dim, device="cuda", generator=generator).bfloat16()
+    v_pages = torch.randn(pages, kv_heads, dim, PAGE, device="cuda", generator=generator).bfloat16()
+    q = torch.randn(tokens, heads * dim, device="cuda", generator=generator).bfloat16()
+    table = torch.randperm(pages, device="cuda", generator=generator).int().view(1, -1)
+    starts = torch.tensor([0, tokens], dtype=torch.int32, device="cuda")
+    contexts = torch.tensor([context], dtype=torch.int32, device="cuda")
+    rows = ops.prefill_block_rows(dim, heads, kv_heads)
+    blocks = ops.prefill_blocks([tokens], [context], rows)
+    out = torch.empty(tokens, heads * dim, dtype=torch.bfloat16, device="cuda")
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    for _ in range(launches):
+        start.record()
+        ops.attention_prefill(out, q, heads * dim, k_pages, v_pages, table, starts, contexts, blocks, heads, dim ** -0.5,
+                              None, context, rows)
+        stop.record()
+        stop.synchronize()
+        best = min(best, start.elapsed_time(stop) * 1e-3)
+    flops = 4.0 * heads * dim * (tokens * (context - tokens) + tokens * tokens / 2)
+    return {"kernel": "prefill attention", "tokens": tokens, "context": context, "heads": heads, "kv_heads": kv_heads,
+            "head_dim": dim, "us": round(best * 1e6, 1), "tflops": round(flops / best / 1e12, 1),
+            "frac": round(flops / best / PEAK_FLOPS["bf16"], 4)}
+
+
 def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
     """Bytes a decode step has to read: every weight it uses once (all but the embedding
     table, of which it reads one row per request) and the cache of the live requests."""
@@ -281,6 +321,10 @@ def main() -> int:
         from turboserve_amd.profiling import format_shares, step_shares
 
         print(format_shares(step_shares(args.kernel_shares, steps=args.shares_steps)))
+        return 0
+    if args.attention_prefill:
+        sizes = [int(v) for v in args.attention_prefill.split(",")]
+        print(json.dumps(run_attention_prefill(SHAPES[args.shape][1], sizes[0], sizes[-1])))
         return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU by design)")

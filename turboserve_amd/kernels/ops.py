@@ -568,11 +568,8 @@ class Ops:
     resident_small_bytes = 64 << 20
 
     def _tiled_plan(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int]:
-        """(iterations of 128 per split, splits, tile) of the tiled product.  The cost of a
-        choice is what the busiest compute unit has to stream: workgroups it is handed (one at
-        a time for the larger tiles, whose LDS fills a compute unit; two for the smallest) x
-        rows of a tile x iterations, one more iteration per workgroup for starting up, with
-        small corrections fitted to measurements at the 7B sizes."""
+        """(iterations of 128 per split, splits, tile) of the tiled product: the cheapest by
+        :meth:`_tiled_cost`."""
         key = (m, n, k, max_splits)
         known = self._tiled_plans.get(key)
         if known is not None:
@@ -581,25 +578,49 @@ class Ops:
         limit = min(iters, max_splits or 32)
         best = None
         for tile in (5, 4, 2):
-            rows = 32 * tile
-            tiles = -(-n // rows)
             for want in range(1, limit + 1):
                 per_split = -(-iters // want)
                 splits = -(-iters // per_split)
                 if splits != want:
                     continue  # the same grid as a smaller `want`
-                groups = -(-tiles * splits // self.compute_units)
-                cost = groups * rows * (per_split + 1)
-                cost *= 1.0 + 2.0 * splits * m / k  # partial sums written here and read by the consumer
-                cost *= 1.0 + 0.12 * m / rows       # activations a workgroup stages, relative to its weights
-                if tile == 2:
-                    cost *= 0.95                    # two workgroups share a compute unit and fill each other's waits
-                resident = self.compute_units * (2 if tile == 2 else 1)
-                cost *= 1.0 + 0.1 * (-(-tiles * splits // resident) - 1)  # later rounds start on a busy device, unevenly
+                cost = self._tiled_cost(m, n, k, per_split, splits, tile)
                 if best is None or cost < best[0] * 0.999:
                     best = (cost, per_split, splits, tile)
         self._tiled_plans[key] = (best[1], best[2], best[3])
         return self._tiled_plans[key]
+
+    def _tiled_cost(self, m: int, n: int, k: int, per_split: int, splits: int, tile: int) -> float:
+        """What a grid of the tiled product costs, in weight rows x iterations streamed by a
+        compute unit one after the other.  A compute unit holds one workgroup of the larger tiles
+        (their LDS fills it) or, up to 64 activation rows, two of the smallest, and streams the
+        faster the more weight rows it has in flight: 64 rows (one small workgroup) count as 1,
+        two small workgroups as 1.25, a tile of 128 as 1.21, of 160 as 1.27.  With more than 32
+        distinct activation rows two workgroups on a unit get in each other's way (at 64 rows the
+        pair is slower than one after the other).  Workgroups beyond what the device holds at
+        once wait for a later round, which starts on a busy device, unevenly.  Every workgroup
+        pays one more iteration for starting up; partial sums are written here and read by the
+        consumer.  Fitted to steps of the 7B and 14B shapes at 8, 32 and 64 rows, measured
+        through the engine with each product's grid varied in turn, and to kernel traces of them."""
+        rows = 32 * tile
+        units = self.compute_units
+        workgroups = -(-n // rows) * splits
+        stretch = rows * (per_split + 1)
+        pairs = tile == 2 and m <= 64  # else the activation rows' LDS leaves room for one workgroup
+        pair_extra = 0.6 if m <= 32 else 0.6 + 0.6 * (m - 32) / 32  # a pair costs 1 + this of a single one
+
+        def round_cost(count: int) -> float:
+            if tile == 2:
+                doubled = max(0, count - units) / units if pairs else 0.0  # share of the units that hold two
+                return stretch * (1.0 + pair_extra * doubled)
+            return stretch / (1.21 if tile == 4 else 1.27)
+
+        held = units * (2 if pairs else 1)
+        full, rest = divmod(workgroups, held)
+        cost = full * round_cost(held) + (round_cost(rest) if rest else 0.0)
+        rounds = full + (1 if rest else 0)
+        cost *= 1.0 + 0.1 * (rounds - 1)
+        cost *= 1.0 + 3.0 * splits * m / k
+        return cost
 
     def gemm_tiled(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                    *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None,

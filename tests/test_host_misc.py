@@ -339,3 +339,26 @@ def test_kernel_shares_of_a_trace(tmp_path):
     assert "| `gemm_tiled_kernel<5, 2>` | 60672, 1, 1 | 2 | 50.0 | 100.0 | 80.0% |" in text and "1 other kernels" in text
     with pytest.raises(ValueError, match="not enough"):
         step_shares(trace, steps=3)
+
+
+def test_tiled_product_plans_are_the_ones_measured_best():
+    """The cost model of the tiled decode product is fitted to measurements on a device of 256
+    compute units; these are the grids that were fastest inside the step there ((iterations of
+    128 per range of K, ranges, tile)), so that a change to the model that loses one shows."""
+    from turboserve_amd.kernels.ops import Ops
+
+    class Planner(Ops):
+        def __init__(self):  # the plan needs the device's size only
+            self.compute_units = 256
+            self._tiled_plans = {}
+
+    plan = Planner()._tiled_plan
+    h7, i7, h14, i14 = 3584, 18944, 5120, 13824
+    assert plan(8, 2 * i7, h7, None) == (28, 1, 5)        # 7B gate+up: one workgroup of 160 rows a unit, one range
+    assert plan(8, h7, i7, None) == (17, 9, 2)            # 7B down: pairs of small workgroups, nine ranges
+    assert plan(64, h7, i7, None) == (17, 9, 4)           # at 64 rows a pair is no longer ahead of a tile of 128
+    assert plan(8, 152064, h7, 1) == (28, 1, 5)           # the head: one range, in rounds
+    assert plan(8, h14, i14, None)[1:] in ((6, 2), (8, 5))  # 14B down: six ranges in pairs or eight of 160 rows, not three
+    assert plan(8, 7168, h14, None) == (10, 4, 2)         # 14B qkv: four ranges, two workgroups a unit
+    assert plan(8, 2 * i14, h14, None) == (40, 1, 2)      # 14B gate+up: 432 small workgroups
+    assert plan(128, h7, i7, None)[2] != 2                # above 64 rows LDS holds one workgroup: no pairs to count on

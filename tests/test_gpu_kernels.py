@@ -727,6 +727,80 @@ def test_sampler_stages_against_plain(ops, vocab):
         assert low - 1e-5 <= u <= high + 1e-5, f"row {i} {settings[i % len(settings)]}: u={u} not in [{low}, {high}]"
 
 
+def kept_after_truncation(logits: torch.Tensor, temperature: float, top_k: int, top_p: float) -> torch.Tensor:
+    """The plain truncation rules (``plain.top_k_filter``, ``plain.top_p_filter``) for a long row:
+    the same sets, found with a sort and cumulative sums instead of a loop over the vocabulary."""
+    work = logits.double() / temperature
+    keep = torch.ones_like(work, dtype=torch.bool)
+    if 0 < top_k < work.numel():
+        keep = work >= torch.sort(work, descending=True).values[top_k - 1]
+    if top_p < 1.0:
+        filtered = work.masked_fill(~keep, float("-inf"))
+        probs = torch.softmax(filtered, dim=-1)
+        values, inverse = torch.unique(filtered, sorted=True, return_inverse=True)
+        per_value = torch.zeros(values.numel(), dtype=torch.float64).index_add_(0, inverse, probs)
+        above = per_value.sum() - torch.cumsum(per_value, dim=0)  # mass strictly above each distinct value
+        keep = keep & (above[inverse] <= top_p)
+    return keep
+
+
+def test_truncation_helper_is_the_plain_rule():
+    g = torch.Generator().manual_seed(9)
+    for quantum in (None, 0.5):
+        logits = torch.randn(300, generator=g) * 3
+        if quantum:
+            logits = torch.round(logits / quantum) * quantum  # many equal values
+        for top_k, top_p in ((0, 0.7), (7, 1.0), (20, 0.5), (3, 0.9)):
+            want = torch.isfinite(plain.top_p_filter(plain.top_k_filter(logits / 0.8, top_k), top_p))
+            assert torch.equal(kept_after_truncation(logits, 0.8, top_k, top_p), want)
+
+
+@pytest.mark.parametrize("vocab", [152064, 40001])
+def test_sampler_on_a_long_row_with_equal_logits(ops, vocab):
+    """A vocabulary of real size (rows that are and are not 16-byte aligned), smooth logits and
+    logits on a grid of 0.25 (thousands of equal values, keys whose low bits are zero): the token
+    lies in what the plain truncation keeps, and its cumulative interval holds the uniform number."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    g = torch.Generator().manual_seed(vocab)
+    settings = [dict(temperature=0.8), dict(temperature=0.8, top_k=50, top_p=0.9), dict(temperature=1.0, top_p=0.6),
+                dict(temperature=1.3, top_k=5), dict(temperature=0.7, top_k=2000, top_p=0.95), dict(temperature=1.0, top_p=0.05)]
+    rows = 2 * len(settings) * 2
+    logits = torch.randn(rows, vocab, generator=g) * 2.5
+    logits[rows // 2:] = torch.round(logits[rows // 2:] * 4) / 4
+    params = [SamplingParams(**settings[i % len(settings)]) for i in range(rows)]
+    seeds = [77 + i * 104729 for i in range(rows)]
+    draws = [i for i in range(rows)]
+    out = sample_rows(ops, logits, params, seeds, draws)
+    for i, p in enumerate(params):
+        token = out.token_ids[i]
+        keep = kept_after_truncation(logits[i], p.temperature, p.top_k, p.top_p)
+        assert bool(keep[token]), f"row {i} {settings[i % len(settings)]}: token {token} is outside the kept set of {int(keep.sum())}"
+        probs = torch.softmax((logits[i].double() / p.temperature).masked_fill(~keep, float("-inf")), dim=-1)
+        cdf = torch.cumsum(probs, dim=-1)
+        u = plain.philox_uniform(seeds[i], draws[i])
+        low = float(cdf[token - 1]) if token > 0 else 0.0
+        assert low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"row {i}: u={u} not in [{low}, {float(cdf[token])}]"
+
+
+def test_sampler_keeps_equal_logits_together(ops):
+    """Five equal logits at the edge of top-k 3 are all kept (the plain rule: below the k-th
+    largest is cut) and all drawn; a nucleus that ends inside a group of equal logits keeps the group."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    logits = torch.full((1, 64), -4.0)
+    logits[0, [3, 9]] = 2.0
+    logits[0, [11, 20, 31, 40, 63]] = 1.0  # the third largest value, five times
+    many = logits.repeat(600, 1)
+    out = sample_rows(ops, many, [SamplingParams(temperature=1.0, top_k=3)] * 600, [5] * 600, list(range(600)))
+    assert set(out.token_ids) == {3, 9, 11, 20, 31, 40, 63}
+    # mass above the 1.0 group is 2 e^2 / (2 e^2 + 5 e + 57 e^-4) = 0.5024 <= 0.6: the group stays; 0.5 cuts it
+    out = sample_rows(ops, many, [SamplingParams(temperature=1.0, top_p=0.6)] * 600, [6] * 600, list(range(600)))
+    assert set(out.token_ids) == {3, 9, 11, 20, 31, 40, 63}
+    out = sample_rows(ops, many, [SamplingParams(temperature=1.0, top_p=0.5)] * 600, [7] * 600, list(range(600)))
+    assert set(out.token_ids) == {3, 9}
+
+
 def test_sampler_rows_are_independent(ops):
     """A batch equals its rows one by one, and a row does not depend on its neighbours
     (tests/unit/test_sampler.py:131-149, 198-215)."""

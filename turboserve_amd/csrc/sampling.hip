@@ -6,8 +6,9 @@
 // The draw is this engine's own rule, because a kernel cannot follow torch.multinomial's
 // stream (sampler.py:285-296): u = Philox-4x32-10(key = seed, counter = draw index) in [0, 1),
 // and the token is the first one, in vocabulary order, whose cumulative probability exceeds u.
-// top-k and top-p are applied as value thresholds found by bisection over the ordered bit
-// patterns of the logits, so equal logits are kept or dropped together.
+// top-k and top-p are applied as value thresholds on the ordered bit patterns of the logits (the
+// k-th largest pattern; the largest pattern whose mass strictly above exceeds p), so equal logits
+// are kept or dropped together.
 #include "common.hpp"
 #include "ts_no_alloc.h"
 
@@ -53,18 +54,51 @@ __device__ __forceinline__ float philox_uniform(uint32_t seed_lo, uint32_t seed_
   return (float)(c0 >> 8) * (1.0f / 16777216.0f);
 }
 
+// f(index, value) for every element of the row, each thread of the block taking every
+// blockDim-th group of four (or every blockDim-th element where the row is not 16-byte aligned).
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ row, int vocab, F f) {
+  const int tid = threadIdx.x;
+  const int step = blockDim.x;
+  if ((reinterpret_cast<uintptr_t>(row) & 15u) == 0) {
+    const float4* quads = reinterpret_cast<const float4*>(row);
+    const int count = vocab >> 2;
+    int i = tid;
+    for (; i + 3 * step < count; i += 4 * step) {
+      const float4 a = quads[i], b = quads[i + step], c = quads[i + 2 * step], d = quads[i + 3 * step];
+      f(4 * i, a.x); f(4 * i + 1, a.y); f(4 * i + 2, a.z); f(4 * i + 3, a.w);
+      f(4 * (i + step), b.x); f(4 * (i + step) + 1, b.y); f(4 * (i + step) + 2, b.z); f(4 * (i + step) + 3, b.w);
+      f(4 * (i + 2 * step), c.x); f(4 * (i + 2 * step) + 1, c.y); f(4 * (i + 2 * step) + 2, c.z);
+      f(4 * (i + 2 * step) + 3, c.w);
+      f(4 * (i + 3 * step), d.x); f(4 * (i + 3 * step) + 1, d.y); f(4 * (i + 3 * step) + 2, d.z);
+      f(4 * (i + 3 * step) + 3, d.w);
+    }
+    for (; i < count; i += step) {
+      const float4 a = quads[i];
+      f(4 * i, a.x); f(4 * i + 1, a.y); f(4 * i + 2, a.z); f(4 * i + 3, a.w);
+    }
+    for (int j = 4 * count + tid; j < vocab; j += step) f(j, row[j]);
+  } else {
+    int i = tid;
+    for (; i + 3 * step < vocab; i += 4 * step) {
+      const float a = row[i], b = row[i + step], c = row[i + 2 * step], d = row[i + 3 * step];
+      f(i, a); f(i + step, b); f(i + 2 * step, c); f(i + 3 * step, d);
+    }
+    for (; i < vocab; i += step) f(i, row[i]);
+  }
+}
+
 // Lowest index among the largest values of a row.
 __device__ __forceinline__ int block_argmax(const float* __restrict__ row, int vocab, float* fscratch,
                                             int* iscratch) {
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
-    if (best_i == 0x7fffffff || v > best) {  // i only grows, so the first of equal values stays
+  for_each_logit(row, vocab, [&](int i, float v) {  // indices come in no particular order
+    if (best_i == 0x7fffffff || v > best || (v == best && i < best_i)) {
       best = v;
       best_i = i;
     }
-  }
+  });
 #pragma unroll
   for (int off = TS_WAVE / 2; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best, off, TS_WAVE);
@@ -188,6 +222,36 @@ extern "C" int ts_argmax_static(int* tokens, const float* logits, int rows, int 
   return ts_argmax(tokens, logits, address, rows, vocab, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The sampling kernel proper.  A row of a large vocabulary is read a dozen times, so every
+// pass matters: rows are visited with 16-byte loads, several in flight per thread; the two
+// truncations pick their thresholds eight bits at a time from histograms in LDS (four passes
+// each instead of 32); the draw scans partial sums in parallel.  Everything is a function of
+// the row alone and is added up in a fixed order (histograms hold integers), so a row's token
+// does not depend on its neighbours or on the run.
+// ---------------------------------------------------------------------------------------------
+#define SAMPLE_WAVES (SAMPLE_THREADS / TS_WAVE)
+#define MASS_COPIES 4  // histograms of mass per workgroup (wavefront w adds to copy w % 4)
+// Probability mass as an integer: exp((x - max) / T) <= 1 in units of 2^-32.  Sums of a whole
+// vocabulary stay far below 2^64, integer sums do not depend on their order, and a token whose
+// mass is below 2^-33 of the likeliest one's counts as none.
+__device__ __forceinline__ unsigned long long mass_units(float x, float m, float inv_temp) {
+  return (unsigned long long)(expf((x - m) * inv_temp) * 4294967296.0f);
+}
+
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* scratch) {
+  const int lane = threadIdx.x & (TS_WAVE - 1);
+  const int wave = threadIdx.x / TS_WAVE;
+#pragma unroll
+  for (int off = TS_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TS_WAVE);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  unsigned long long total = 0;
+  for (int w = 0; w < SAMPLE_WAVES; ++w) total += scratch[w];
+  return total;
+}
+
 // Per-row parameters, all device arrays of `rows` entries:
 //   temperature (0 = greedy), top_k (0 = off), top_p (1 = off), penalty (1 = off),
 //   seed_lo / seed_hi / draw_index (Philox key and counter).
@@ -203,39 +267,50 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
               const int* __restrict__ history_start) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
-  __shared__ float partial[SAMPLE_THREADS];
+  __shared__ unsigned long long lscratch[SAMPLE_WAVES];
+  __shared__ unsigned int counts[SAMPLE_WAVES][256];             // top-k: keys per digit, one histogram a wavefront
+  __shared__ unsigned long long mass[MASS_COPIES][256];          // top-p: mass per digit
+  __shared__ unsigned long long mass_exact[MASS_COPIES][256];    // of which: keys whose lower digits are all zero
+  __shared__ unsigned int picked[2];                             // what thread 0 decided in a round
+  __shared__ unsigned long long carried;
+  __shared__ float wave_total[SAMPLE_WAVES];
   __shared__ int chosen;
 
   const int r = blockIdx.x;
   const int tid = threadIdx.x;
+  const int lane = tid & (TS_WAVE - 1);
+  const int wave = tid / TS_WAVE;
   const float* src = logits + (size_t)r * vocab;
-  float* row = work + (size_t)r * vocab;
   const float temp = temperature[r];
   const float pen = penalty[r];
 
-  // 1. penalised copy.  Reading the untouched logits makes a repeated history token harmless.
-  for (int i = tid; i < vocab; i += blockDim.x) row[i] = src[i];
-  __syncthreads();
+  // 1. penalised copy (only where there is a penalty; else the logits themselves are read).
+  // Reading the untouched logits makes a repeated history token harmless.
+  const float* row = src;
   if (pen != 1.0f) {
+    float* copy = work + (size_t)r * vocab;
+    for (int i = tid; i < vocab; i += blockDim.x) copy[i] = src[i];
+    __syncthreads();
     const int h0 = history_start[r], h1 = history_start[r + 1];
     for (int j = h0 + tid; j < h1; j += blockDim.x) {
       const int tok = history[j];
       if (tok >= 0 && tok < vocab) {
         const float v = src[tok];
-        row[tok] = v < 0.f ? v * pen : v / pen;
+        copy[tok] = v < 0.f ? v * pen : v / pen;
       }
     }
     __syncthreads();
+    row = copy;
   }
 
   // 2. log-softmax terms of the penalised logits (before temperature).
   float base_max = 0.f, base_lse = 0.f;
   if (logprobs) {
     float m = -INFINITY;
-    for (int i = tid; i < vocab; i += blockDim.x) m = fmaxf(m, row[i]);
+    for_each_logit(row, vocab, [&](int, float v) { m = fmaxf(m, v); });
     base_max = block_max(m, fscratch);
     float s = 0.f;
-    for (int i = tid; i < vocab; i += blockDim.x) s += expf(row[i] - base_max);
+    for_each_logit(row, vocab, [&](int, float v) { s += expf(v - base_max); });
     base_lse = logf(block_sum(s, fscratch));
   }
 
@@ -244,82 +319,202 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
     token = block_argmax(row, vocab, fscratch, iscratch);
   } else {
     const float inv_temp = 1.0f / temp;
-    // 3. top-k: the k-th largest key, by bisection on the bit pattern.
+    // 3. top-k: the k-th largest key, found eight bits at a time: the digit whose keys, with
+    // those of higher digits, reach k, then the same among the keys that share it.
     uint32_t threshold = 0u;
     const int k = top_k[r];
     if (k > 0 && k < vocab) {
-      uint32_t t = 0u;
-      for (int bit = 31; bit >= 0; --bit) {
-        const uint32_t cand = t | (1u << bit);
-        int count = 0;
-        for (int i = tid; i < vocab; i += blockDim.x) count += ordered_key(row[i]) >= cand;
-        if (block_sum_int(count, iscratch) >= k) t = cand;
+      uint32_t prefix = 0u;
+      unsigned int wanted = (unsigned int)k;  // among the keys that share `prefix`
+      for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = tid; i < SAMPLE_WAVES * 256; i += blockDim.x) (&counts[0][0])[i] = 0u;
+        __syncthreads();
+        const uint32_t high_mask = shift == 24 ? 0u : ~0u << (shift + 8);
+        for_each_logit(row, vocab, [&](int, float v) {
+          const uint32_t key = ordered_key(v);
+          if ((key & high_mask) == prefix) atomicAdd(&counts[wave][(key >> shift) & 255u], 1u);
+        });
+        __syncthreads();
+        if (tid < 256) {  // one histogram, in counts[0]
+          unsigned int total = 0u;
+          for (int w = 0; w < SAMPLE_WAVES; ++w) total += counts[w][tid];
+          counts[0][tid] = total;
+        }
+        __syncthreads();
+        if (tid == 0) {
+          unsigned int above = 0u;
+          int digit = 255;
+          for (; digit > 0; --digit) {
+            if (above + counts[0][digit] >= wanted) break;
+            above += counts[0][digit];
+          }
+          picked[0] = (unsigned int)digit;
+          picked[1] = wanted - above;
+        }
+        __syncthreads();
+        prefix |= picked[0] << shift;
+        wanted = picked[1];
+        __syncthreads();
       }
-      threshold = t;
+      threshold = prefix;
     }
     // Softmax terms of the scaled logits over what top-k kept.
     float m = -INFINITY;
-    for (int i = tid; i < vocab; i += blockDim.x)
-      if (ordered_key(row[i]) >= threshold) m = fmaxf(m, row[i]);
+    for_each_logit(row, vocab, [&](int, float v) {
+      if (ordered_key(v) >= threshold) m = fmaxf(m, v);
+    });
     m = block_max(m, fscratch);
-    // 4. top-p: keep a token while the mass strictly above it is <= p.
+    // 4. top-p: keep a token while the mass strictly above it is <= p.  T is the largest key whose
+    // mass strictly above still exceeds the limit, again eight bits at a time: for a candidate whose
+    // lower digits are zero, the mass above it is that of the higher digits plus that of its own
+    // digit less the keys that equal the candidate itself.
     const float p = top_p[r];
     if (p < 1.0f) {
-      float z = 0.f;
-      for (int i = tid; i < vocab; i += blockDim.x)
-        if (ordered_key(row[i]) >= threshold) z += expf((row[i] - m) * inv_temp);
-      z = block_sum(z, fscratch);
-      const float limit = p * z;
-      uint32_t t = 0u;  // the largest key whose mass above still exceeds the limit
-      for (int bit = 31; bit >= 0; --bit) {
-        const uint32_t cand = t | (1u << bit);
-        float above = 0.f;
-        for (int i = tid; i < vocab; i += blockDim.x) {
-          const uint32_t key = ordered_key(row[i]);
-          if (key > cand && key >= threshold) above += expf((row[i] - m) * inv_temp);
+      unsigned long long z = 0ull;
+      for_each_logit(row, vocab, [&](int, float v) {
+        if (ordered_key(v) >= threshold) z += mass_units(v, m, inv_temp);
+      });
+      z = block_sum_u64(z, lscratch);
+      const unsigned long long limit = (unsigned long long)((double)p * (double)z);
+      uint32_t prefix = 0u;
+      unsigned long long above = 0ull;  // mass of the keys whose higher digits exceed the prefix's
+      for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = tid; i < MASS_COPIES * 256; i += blockDim.x) {
+          (&mass[0][0])[i] = 0ull;
+          (&mass_exact[0][0])[i] = 0ull;
         }
-        if (block_sum(above, fscratch) > limit) t = cand;
+        __syncthreads();
+        const uint32_t high_mask = shift == 24 ? 0u : ~0u << (shift + 8);
+        const uint32_t low_mask = shift == 0 ? 0u : ~0u >> (32 - shift);
+        for_each_logit(row, vocab, [&](int, float v) {
+          const uint32_t key = ordered_key(v);
+          if (key >= threshold && (key & high_mask) == prefix) {
+            const unsigned long long units = mass_units(v, m, inv_temp);
+            const uint32_t digit = (key >> shift) & 255u;
+            atomicAdd(&mass[wave % MASS_COPIES][digit], units);
+            if ((key & low_mask) == 0u) atomicAdd(&mass_exact[wave % MASS_COPIES][digit], units);
+          }
+        });
+        __syncthreads();
+        if (tid < 256) {
+          unsigned long long total = 0ull, exact = 0ull;
+          for (int c = 0; c < MASS_COPIES; ++c) {
+            total += mass[c][tid];
+            exact += mass_exact[c][tid];
+          }
+          mass[0][tid] = total;
+          mass_exact[0][tid] = exact;
+        }
+        __syncthreads();
+        if (tid == 0) {
+          unsigned long long higher = above;  // mass of the digits above the candidate's
+          int digit = 255;
+          for (; digit > 0; --digit) {
+            if (higher + (mass[0][digit] - mass_exact[0][digit]) > limit) break;
+            higher += mass[0][digit];
+          }
+          picked[0] = (unsigned int)digit;
+          carried = higher;
+        }
+        __syncthreads();
+        prefix |= picked[0] << shift;
+        above = carried;
+        __syncthreads();
       }
-      if (t + 1u > threshold) threshold = t + 1u;
+      // prefix is T only if the mass above it does exceed the limit; otherwise nothing is cut here
+      // (every digit fell through to 0: T = 0, as the search bit by bit would leave it).
+      if (prefix + 1u > threshold) threshold = prefix + 1u;
     }
-    // 5. draw: contiguous chunks per thread, scan of the chunk sums, walk inside one chunk.
-    const int chunk = (vocab + blockDim.x - 1) / blockDim.x;
-    const int c0 = tid * chunk;
-    const int c1 = (c0 + chunk < vocab) ? c0 + chunk : vocab;
-    float local = 0.f;
-    for (int i = c0; i < c1; ++i)
-      if (ordered_key(row[i]) >= threshold) local += expf((row[i] - m) * inv_temp);
-    partial[tid] = local;
+    // 5. draw.  The vocabulary is cut into one stretch per wavefront, a stretch into blocks of 256
+    // tokens, four consecutive ones per lane.  Cumulative mass is added up in a fixed order (a
+    // lane's four, the lanes of a block by a scan, blocks and stretches one after the other); every
+    // interval ends where the next begins by construction, so exactly one stretch, block, lane
+    // and token take the target, and where rounding lets a walk end below it, the last token
+    // with mass does.
+    const int block_tokens = 4 * TS_WAVE;
+    const int blocks_total = (vocab + block_tokens - 1) / block_tokens;
+    const int blocks_per_wave = (blocks_total + SAMPLE_WAVES - 1) / SAMPLE_WAVES;
+    const int first_block = wave * blocks_per_wave;
+    const int last_block = min(first_block + blocks_per_wave, blocks_total);  // exclusive
+    auto lane_masses = [&](int block, float (&e)[4]) {
+      const int at = block * block_tokens + 4 * lane;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = at + j;
+        const float v = i < vocab ? row[i] : -INFINITY;
+        e[j] = (i < vocab && ordered_key(v) >= threshold) ? expf((v - m) * inv_temp) : 0.f;
+      }
+    };
+    auto wave_inclusive = [&](float v) {  // sum over lanes 0 .. lane, always by the same additions
+#pragma unroll
+      for (int off = 1; off < TS_WAVE; off <<= 1) {
+        const float other = __shfl_up(v, off, TS_WAVE);
+        if (lane >= off) v += other;
+      }
+      return v;
+    };
+    float stretch = 0.f;
+    for (int block = first_block; block < last_block; ++block) {
+      float e[4];
+      lane_masses(block, e);
+      stretch += __shfl(wave_inclusive((e[0] + e[1]) + (e[2] + e[3])), TS_WAVE - 1, TS_WAVE);
+    }
+    if (lane == 0) wave_total[wave] = stretch;
     if (tid == 0) chosen = -1;
     __syncthreads();
-    if (tid == 0) {
-      float running = 0.f;
-      for (int i = 0; i < (int)blockDim.x; ++i) {
-        const float v = partial[i];
-        partial[i] = running;  // exclusive prefix
-        running += v;
-      }
-      fscratch[0] = running;
+    float before = 0.f, after = 0.f, total = 0.f;  // cumulative mass where this stretch begins and ends, and all of it
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+      if (w == wave) before = total;
+      total += wave_total[w];
+      if (w == wave) after = total;
     }
-    __syncthreads();
-    const float total = fscratch[0];
     const float u = philox_uniform(seed_lo[r], seed_hi[r], draw_index[r]);
     float target = u * total;
     const float below_total = __uint_as_float(__float_as_uint(total) - 1u);
     if (target > below_total) target = below_total;
-    const float prefix = partial[tid];
-    if (local > 0.f && prefix <= target && target < prefix + local) {
-      // Same order of additions as `local`, so prefix + inner ends at prefix + local > target.
-      float inner = 0.f;
-      int pick = -1;
-      for (int i = c0; i < c1; ++i) {
-        if (ordered_key(row[i]) >= threshold) {
-          inner += expf((row[i] - m) * inv_temp);
-          pick = i;
-          if (prefix + inner > target) break;
+    if (before <= target && target < after) {  // true in one wavefront, for all of its lanes
+      float sum = before;
+      int fallback_block = -1;
+      bool found = false;
+      for (int block = first_block; block < last_block && !found; ++block) {
+        float e[4];
+        lane_masses(block, e);
+        const float mine = (e[0] + e[1]) + (e[2] + e[3]);
+        const float through = wave_inclusive(mine);
+        float upto_previous = __shfl_up(through, 1, TS_WAVE);
+        if (lane == 0) upto_previous = 0.f;
+        const unsigned long long with_mass = __ballot(mine > 0.f);
+        const unsigned long long over = __ballot(mine > 0.f && sum + through > target);
+        if (over != 0ull) {
+          if (lane == __ffsll((long long)over) - 1) {
+            float inner = sum + upto_previous;
+            int pick = -1;
+            for (int j = 0; j < 4; ++j) {
+              if (e[j] > 0.f) {
+                inner += e[j];
+                pick = block * block_tokens + 4 * lane + j;
+                if (inner > target) break;
+              }
+            }
+            chosen = pick;
+          }
+          found = true;
+        } else if (with_mass != 0ull) {
+          fallback_block = block;
+        }
+        sum += __shfl(through, TS_WAVE - 1, TS_WAVE);
+      }
+      if (!found && fallback_block >= 0) {
+        float e[4];
+        lane_masses(fallback_block, e);
+        const unsigned long long with_mass = __ballot((e[0] + e[1]) + (e[2] + e[3]) > 0.f);
+        if (lane == 63 - __clzll((long long)with_mass)) {
+          int pick = -1;
+          for (int j = 0; j < 4; ++j)
+            if (e[j] > 0.f) pick = fallback_block * block_tokens + 4 * lane + j;
+          chosen = pick;
         }
       }
-      chosen = pick;
     }
     __syncthreads();
     token = chosen;

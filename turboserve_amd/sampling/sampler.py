@@ -111,7 +111,8 @@ class Sampler:
             dtype=np.float32,
         )
         seeds64 = np.asarray([int(s) & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64)
-        ints = np.concatenate([
+        packed = np.concatenate([
+            floats.reshape(-1).view(np.int32),
             np.asarray([p.top_k for p in params], dtype=np.int32),
             (seeds64 & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32),
             (seeds64 >> np.uint64(32)).astype(np.uint32).view(np.int32),
@@ -119,14 +120,21 @@ class Sampler:
             np.asarray(history_start, dtype=np.int32),
             np.asarray(flat_history, dtype=np.int32),
         ])
+        # One copy, from pinned memory and queued on the stream: a copy from pageable memory
+        # would make the host wait for everything the stream holds, a step launched ahead included.
         device = logits.device
-        fdev = torch.from_numpy(floats).to(device)
-        idev = torch.from_numpy(ints).to(device)
-        top_k, seed_lo, seed_hi, draw, hstart, hist = torch.split(
-            idev, [rows, rows, rows, rows, rows + 1, len(flat_history)]
+        if device.type == "cuda":
+            staged = torch.empty(packed.shape, dtype=torch.int32, pin_memory=True)
+            staged.numpy()[:] = packed
+            on_device = staged.to(device, non_blocking=True)
+        else:
+            on_device = torch.from_numpy(packed).to(device)
+        temperature, top_p, penalty, top_k, seed_lo, seed_hi, draw, hstart, hist = torch.split(
+            on_device, [rows, rows, rows, rows, rows, rows, rows, rows + 1, len(flat_history)]
         )
         tokens, logprobs = self.ops.sample(
-            logits, fdev[0], top_k, fdev[1], fdev[2], seed_lo, seed_hi, draw, hist, hstart, want_logprobs
+            logits, temperature.view(torch.float32), top_k, top_p.view(torch.float32), penalty.view(torch.float32),
+            seed_lo, seed_hi, draw, hist, hstart, want_logprobs
         )
         return PendingSample(tokens, logprobs, list(params))
 

@@ -75,12 +75,13 @@ class ToySampler:
         return PendingSample(logits.argmax(dim=1).to(torch.int32), None, [seq.sampling for seq in sequences])
 
 
-def make_engine(run_ahead: bool, *, num_blocks: int = 64, max_num_seqs: int = 8, budget: int = 32, page: int = 4):
+def make_engine(run_ahead: bool, *, num_blocks: int = 64, max_num_seqs: int = 8, budget: int = 32, page: int = 4,
+                sampler=None):
     cfg = SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget, block_size=page, num_blocks=num_blocks)
     scheduler = Scheduler(cfg, CacheManager([None], num_blocks, page, max_num_seqs))
     runner = ToyRunner()
     engine = LLMEngine(EngineConfig(model="/nonexistent", scheduler=cfg, run_ahead=run_ahead), model=object(),
-                       scheduler=scheduler, runner=runner, sampler=ToySampler())
+                       scheduler=scheduler, runner=runner, sampler=sampler or ToySampler())
     return engine, runner
 
 
@@ -182,6 +183,36 @@ def test_a_step_is_not_launched_ahead_of_a_request_that_ends_by_length_or_has_a_
     while engine.has_unfinished():
         engine.step()
     assert runner.steps == 6 and runner.steps_ahead == 0  # the penalty needs the tokens on the host
+
+    class UnreadSampler(ToySampler):
+        """A sampler that can be given the token the host has not read (as the real one can)."""
+
+        takes_unread = True
+
+        def __init__(self):
+            self.seen = []
+
+        def launch_sequences(self, logits, sequences, unread=None):
+            if unread is not None:
+                tokens, places = unread
+                assert len(places) == len(sequences)
+                assert all(seq.output_token_ids[-1] == seq.UNREAD_TOKEN for seq in sequences)
+                self.seen.append([int(tokens[place]) for place in places])
+            return super().launch_sequences(logits, sequences)
+
+    sampler = UnreadSampler()
+    engine, runner = make_engine(True, sampler=sampler)
+    params = SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True, repetition_penalty=1.2)
+    engine.add_request("b", [5, 6, 7], params)
+    engine.add_request("d", [9, 3], params)
+    outputs = []
+    while engine.has_unfinished():
+        outputs.extend(engine.step())
+    assert runner.steps_ahead == 5  # with such a sampler a penalty does not keep a step from being launched ahead
+    tokens = {rid: [t for o in outputs if o.request_id == rid for t in o.new_token_ids] for rid in ("b", "d")}
+    assert tokens["b"] == continuation([5, 6, 7], params) and tokens["d"] == continuation([9, 3], params)
+    # every launch ahead named, for each request, that request's own token of the launch before
+    assert sampler.seen == [[tokens["b"][i], tokens["d"][i]] for i in range(5)]
     engine, runner = make_engine(True)
     engine.add_request("c", [5, 6, 7], SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
     while engine.has_unfinished():

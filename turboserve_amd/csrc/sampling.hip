@@ -256,6 +256,9 @@ __device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v
 //   temperature (0 = greedy), top_k (0 = off), top_p (1 = off), penalty (1 = off),
 //   seed_lo / seed_hi / draw_index (Philox key and counter).
 // history tokens of row r: history[history_start[r] .. history_start[r + 1]).
+// unread_tokens / unread_row (both may be null): a row whose request has one more token that
+// the host has not read yet (it was sampled by a launch still in flight) names that token's
+// place in `unread_tokens`, or -1; it counts as part of the row's history.
 // work [rows, vocab]: scratch for the penalised logits.  logprobs may be null.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
@@ -264,7 +267,8 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
               const float* __restrict__ top_p, const float* __restrict__ penalty,
               const uint32_t* __restrict__ seed_lo, const uint32_t* __restrict__ seed_hi,
               const uint32_t* __restrict__ draw_index, const int* __restrict__ history,
-              const int* __restrict__ history_start) {
+              const int* __restrict__ history_start, const int* __restrict__ unread_tokens,
+              const int* __restrict__ unread_row) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ unsigned long long lscratch[SAMPLE_WAVES];
@@ -294,6 +298,13 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
     const int h0 = history_start[r], h1 = history_start[r + 1];
     for (int j = h0 + tid; j < h1; j += blockDim.x) {
       const int tok = history[j];
+      if (tok >= 0 && tok < vocab) {
+        const float v = src[tok];
+        copy[tok] = v < 0.f ? v * pen : v / pen;
+      }
+    }
+    if (tid == 0 && unread_tokens && unread_row && unread_row[r] >= 0) {
+      const int tok = unread_tokens[unread_row[r]];
       if (tok >= 0 && tok < vocab) {
         const float v = src[tok];
         copy[tok] = v < 0.f ? v * pen : v / pen;
@@ -530,13 +541,13 @@ extern "C" int ts_sample(int* tokens, float* logprobs, const float* logits, floa
                          int vocab, const float* temperature, const int* top_k, const float* top_p,
                          const float* penalty, const uint32_t* seed_lo, const uint32_t* seed_hi,
                          const uint32_t* draw_index, const int* history, const int* history_start,
-                         hipStream_t stream) {
+                         const int* unread_tokens, const int* unread_row, hipStream_t stream) {
   if (rows == 0) return TS_OK;
   if (!tokens || !logits || !work || vocab < 1 || !temperature || !top_k || !top_p || !penalty ||
       !seed_lo || !seed_hi || !draw_index || !history_start)
     return TS_ERR_ARG;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, tokens, logprobs,
                      logits, work, vocab, temperature, top_k, top_p, penalty, seed_lo, seed_hi,
-                     draw_index, history, history_start);
+                     draw_index, history, history_start, unread_tokens, unread_row);
   return ts_launch_status();
 }

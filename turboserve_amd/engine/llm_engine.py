@@ -260,13 +260,20 @@ class LLMEngine:
         else:  # only a runner that said it takes them (`takes_tokens_from`) is asked to
             logits = self.runner.step(entries, fresh_state_slots=scheduled.fresh_state_slots, tokens_from=tokens_from)
         sampled = scheduled.sampled()
-        pending = self._launch_sampler(logits, [item.seq for item in sampled]) if sampled else None
+        unread = None
+        if tokens_from is not None and sampled and getattr(self.sampler, "takes_unread", False):
+            # Every request of a step launched ahead has its last token still on the device; a
+            # repetition penalty must see it.
+            tokens, patch = tokens_from
+            row_of = {id(item): index for index, item in enumerate(scheduled.scheduled)}
+            unread = (tokens, [patch.get(row_of[id(item)], -1) for item in sampled])
+        pending = self._launch_sampler(logits, [item.seq for item in sampled], unread) if sampled else None
         return _InFlight(sampled, pending)
 
-    def _launch_sampler(self, logits, sequences):
+    def _launch_sampler(self, logits, sequences, unread=None):
         launch = getattr(self.sampler, "launch_sequences", None)
         if launch is not None:
-            return launch(logits, sequences)
+            return launch(logits, sequences, unread) if unread is not None else launch(logits, sequences)
         return _Sampled(self.sampler.sample_sequences(logits, sequences))  # a stand-in sampler without a launch/read split
 
     def _run_ahead(self, flight: "_InFlight", outputs: list[RequestOutput], *, now: float) -> "_InFlight | None":
@@ -274,7 +281,7 @@ class LLMEngine:
 
         Possible when that step is known without the tokens' values: the unfinished requests of
         ``flight`` all sample and are all the running requests, nothing waits to be admitted,
-        none needs its own history for a penalty, and the step replays as a graph.  Each request
+        and the step replays as a graph (a repetition penalty gets the unread token on the device).  Each request
         gets a place for its unread token (unless that token is its last by ``max_tokens``: then
         it has no part in the next step); the step's token ids are copied on the device from the
         sampler's result.  A request that then turns out to have ended (a stop token, a stop
@@ -287,8 +294,8 @@ class LLMEngine:
         takes = getattr(self.runner, "takes_tokens_from", None)
         if takes is None or not takes(len(live)) or not self.scheduler.only_running(live):
             return None
-        if any(seq.sampling.repetition_penalty != 1.0 for seq in live):
-            return None
+        if any(seq.sampling.repetition_penalty != 1.0 for seq in live) and not getattr(self.sampler, "takes_unread", False):
+            return None  # the penalty needs the unread token, and this sampler cannot be given it
         for seq in live:
             # A request that reaches max_tokens with the token in flight takes no place: it has
             # nothing to compute in the next step and ends when its token is read.

@@ -58,7 +58,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                     c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
 }
 
@@ -773,10 +773,15 @@ class Ops:
         history: torch.Tensor,
         history_start: torch.Tensor,
         want_logprobs: bool,
+        unread_tokens: torch.Tensor | None = None,
+        unread_row: torch.Tensor | None = None,
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
         """One token per row of ``logits [n, V]``; parameter tensors are per row (see
-        ``csrc/sampling.hip``).  Returns ``(tokens int32 [n], logprobs float32 [n] | None)``."""
-        _gpu(logits, temperature, top_k, top_p, penalty, seed_lo, seed_hi, draw_index, history, history_start)
+        ``csrc/sampling.hip``).  ``unread_tokens`` (int32, on the device) with ``unread_row [n]``
+        (a place in it per row, or -1): one more token of a row's history that only the device
+        knows yet.  Returns ``(tokens int32 [n], logprobs float32 [n] | None)``."""
+        _gpu(logits, temperature, top_k, top_p, penalty, seed_lo, seed_hi, draw_index, history, history_start,
+             unread_tokens, unread_row)
         _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(),
               "logits must be contiguous float32 [n, V]")
         rows, vocab = logits.shape
@@ -788,11 +793,17 @@ class Ops:
         _i32(history, "history")
         _i32(history_start, "history_start")
         _need(history_start.numel() == rows + 1, "history_start must have n + 1 entries")
+        _need((unread_tokens is None) == (unread_row is None), "unread_tokens and unread_row come together")
+        if unread_row is not None:
+            _i32(unread_tokens, "unread_tokens")
+            _i32(unread_row, "unread_row")
+            _need(unread_row.numel() == rows and unread_tokens.is_contiguous() and unread_row.is_contiguous(),
+                  "unread_row must have n entries")
         tokens = torch.empty((rows,), dtype=torch.int32, device=logits.device)
         logprobs = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_logprobs else None
         work = torch.empty_like(logits)
         _check(self.core.ts_sample(_ptr(tokens), _ptr(logprobs), _ptr(logits), _ptr(work), rows, vocab,
                                    _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(penalty), _ptr(seed_lo),
                                    _ptr(seed_hi), _ptr(draw_index), _ptr(history), _ptr(history_start),
-                                   self.stream()), "ts_sample")
+                                   _ptr(unread_tokens), _ptr(unread_row), self.stream()), "ts_sample")
         return tokens, logprobs

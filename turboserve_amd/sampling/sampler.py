@@ -61,6 +61,9 @@ class PendingSample:
 
 
 class Sampler:
+    #: ``launch`` takes ``unread``: a row's history may end in a token only the device knows yet.
+    takes_unread = True
+
     def __init__(self, ops) -> None:
         self.ops = ops
 
@@ -86,14 +89,20 @@ class Sampler:
         seeds: SequenceABC[int],
         draw_indices: SequenceABC[int],
         histories: SequenceABC[SequenceABC[int]] | None = None,
+        unread: tuple[torch.Tensor, SequenceABC[int]] | None = None,
     ) -> PendingSample:
         """``sample`` without the wait: the kernels are launched and the tokens stay on the
-        device until ``PendingSample.read``."""
+        device until ``PendingSample.read``.  ``unread``: the tokens of a launch whose result has
+        not been read (int32 on the device) and, per row, the place in them of the row's own last
+        token, or -1; a row with a repetition penalty counts that token into its history (where
+        its ``histories`` entry has a negative stand-in)."""
         rows = int(logits.shape[0])
         if len(params) != rows or len(seeds) != rows or len(draw_indices) != rows:
             raise ValueError(f"{len(params)} params / {len(seeds)} seeds / {len(draw_indices)} counters for {rows} rows")
         if histories is not None and len(histories) != rows:
             raise ValueError(f"{len(histories)} histories for {rows} rows of logits")
+        if unread is not None and len(unread[1]) != rows:
+            raise ValueError(f"{len(unread[1])} places of unread tokens for {rows} rows of logits")
         if rows == 0:
             return PendingSample(None, None)
         if all(p.is_plain_greedy for p in params):
@@ -118,6 +127,7 @@ class Sampler:
             (seeds64 >> np.uint64(32)).astype(np.uint32).view(np.int32),
             np.asarray([int(d) & 0xFFFFFFFF for d in draw_indices], dtype=np.uint32).view(np.int32),
             np.asarray(history_start, dtype=np.int32),
+            np.asarray(unread[1] if unread is not None else [-1] * rows, dtype=np.int32),
             np.asarray(flat_history, dtype=np.int32),
         ])
         # One copy, from pinned memory and queued on the stream: a copy from pageable memory
@@ -129,12 +139,14 @@ class Sampler:
             on_device = staged.to(device, non_blocking=True)
         else:
             on_device = torch.from_numpy(packed).to(device)
-        temperature, top_p, penalty, top_k, seed_lo, seed_hi, draw, hstart, hist = torch.split(
-            on_device, [rows, rows, rows, rows, rows, rows, rows, rows + 1, len(flat_history)]
+        temperature, top_p, penalty, top_k, seed_lo, seed_hi, draw, hstart, unread_row, hist = torch.split(
+            on_device, [rows, rows, rows, rows, rows, rows, rows, rows + 1, rows, len(flat_history)]
         )
         tokens, logprobs = self.ops.sample(
             logits, temperature.view(torch.float32), top_k, top_p.view(torch.float32), penalty.view(torch.float32),
-            seed_lo, seed_hi, draw, hist, hstart, want_logprobs
+            seed_lo, seed_hi, draw, hist, hstart, want_logprobs,
+            unread_tokens=unread[0] if unread is not None else None,
+            unread_row=unread_row.contiguous() if unread is not None else None,
         )
         return PendingSample(tokens, logprobs, list(params))
 
@@ -143,12 +155,15 @@ class Sampler:
         only if a penalty is set, the token history of each (sampler.py:240-256)."""
         return self.launch_sequences(logits, sequences).read()
 
-    def launch_sequences(self, logits: torch.Tensor, sequences: SequenceABC[Sequence]) -> PendingSample:
-        """``sample_sequences`` without the wait."""
+    def launch_sequences(self, logits: torch.Tensor, sequences: SequenceABC[Sequence],
+                         unread: tuple[torch.Tensor, SequenceABC[int]] | None = None) -> PendingSample:
+        """``sample_sequences`` without the wait.  ``unread``: see ``launch`` (a request whose last
+        token is an unread one has ``Sequence.UNREAD_TOKEN`` there)."""
         return self.launch(
             logits,
             [seq.sampling for seq in sequences],
             [seq.sample_seed for seq in sequences],
             [seq.num_output_tokens for seq in sequences],
             [seq.token_ids if seq.sampling.repetition_penalty != 1.0 else () for seq in sequences],
+            unread,
         )

@@ -93,6 +93,11 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--kernel-shares", metavar="TRACE.csv", default=None,
                    help="print the per-kernel table of a rocprofv3 kernel trace of a run of this program and exit")
     p.add_argument("--shares-steps", type=int, default=4, help="steps at the end of the trace that the table covers")
+    p.add_argument("--closed-loop", type=int, default=0, metavar="C",
+                   help="the reference's serving profile offline: 256 requests of 128..1024 input and 64..512 output "
+                        "tokens, C of them live at a time; prints output tokens/s, time to first token and time between tokens")
+    p.add_argument("--sampled", action="store_true",
+                   help="with --closed-loop: temperature 0.7, top-p 0.8, top-k 20, repetition penalty 1.05 instead of greedy")
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
@@ -257,6 +262,66 @@ def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True)
     return best
 
 
+def run_closed_loop(model, config, concurrency: int, *, sampled: bool, requests: int = 256, tune: bool = True) -> dict:
+    """The workload shape of the reference's serving benchmark (configs/bench/profiles.yaml:26-40:
+    256 requests, 128 to 1,024 input tokens, 64 to 512 output tokens, a fixed number in flight),
+    driven offline: a request is added the moment one ends.  Lengths and token ids are seeded
+    uniform draws; every request runs to its output length."""
+    import random
+
+    import torch
+
+    from turboserve_amd.sampling.params import SamplingParams
+
+    rng = random.Random(1)
+    shapes = [(rng.randint(128, 1024), rng.randint(64, 512)) for _ in range(requests)]
+    engine = make_engine(model, config, max_num_seqs=concurrency, budget=PREFILL_TOKENS,
+                         tokens_per_request=1024 + 512 + PAGE, tune_tokens=(PREFILL_TOKENS,) if tune else ())
+    prompts = [random_prompts(config, 1, length, 100 + index)[0] for index, (length, _) in enumerate(shapes)]
+
+    def params(index: int) -> "SamplingParams":
+        if sampled:
+            return SamplingParams(max_tokens=shapes[index][1], temperature=0.7, top_p=0.8, top_k=20,
+                                  repetition_penalty=1.05, seed=index, ignore_eos=True)
+        return SamplingParams(max_tokens=shapes[index][1], temperature=0.0, ignore_eos=True)
+
+    sequences, live, produced, steps = [], 0, 0, 0
+
+    def admit() -> None:
+        nonlocal live
+        while live < concurrency and len(sequences) < requests:
+            index = len(sequences)
+            sequences.append(engine.add_request(f"r{index}", prompts[index], params(index)))
+            live += 1
+
+    admit()
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    while engine.has_unfinished():
+        for output in engine.step():
+            produced += len(output.new_token_ids)
+            live -= bool(output.finished)
+        admit()
+        steps += 1
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - started
+    preemptions = int(engine.stats()["num_preemptions"])
+    engine.close()
+
+    def median(values: list[float]) -> float:
+        ordered = sorted(values)
+        return ordered[len(ordered) // 2]
+
+    first = [seq.timing.t_first_token - seq.timing.t_arrival for seq in sequences]
+    between = [(seq.timing.t_finished - seq.timing.t_first_token) / max(1, seq.num_output_tokens - 1) for seq in sequences]
+    return {"metric": f"closed loop, {requests} requests of 128..1024 in / 64..512 out, {concurrency} in flight "
+                      f"(through LLMEngine, {'sampled' if sampled else 'greedy'})",
+            "value": round(produced / seconds, 1), "unit": "output tokens/s", "seconds": round(seconds, 2), "steps": steps,
+            "ms_per_step": round(seconds / steps * 1e3, 3), "output_tokens": produced,
+            "input_tokens": sum(length for length, _ in shapes), "first_token_ms_p50": round(median(first) * 1e3, 1),
+            "between_tokens_ms_p50": round(median(between) * 1e3, 2), "preemptions": preemptions}
+
+
 def run_attention_prefill(shape: dict, tokens: int, context: int, launches: int = 15) -> dict:
     """The prefill attention kernel alone (no model): ``tokens`` rows of one request at the end of
     ``context`` keys on scrambled pages, random queries, keys and values; the best of ``launches``
@@ -350,6 +415,11 @@ def main() -> int:
     tune = not args.no_gemm_tuning and dtype == torch.bfloat16
     run_ahead = not args.no_run_ahead
 
+    if args.closed_loop:
+        record = run_closed_loop(model, config, args.closed_loop, sampled=args.sampled, tune=tune)
+        record.update({"dtype": dtype_key, "layers": layers, "model": f"{shape_name} shape"})
+        print(json.dumps(record))
+        return 0
     if args.only_prefill:
         seconds = run_prefill(model, config, PREFILL_TOKENS, tune=tune)
         print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}))

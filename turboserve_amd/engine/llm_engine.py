@@ -249,7 +249,7 @@ class LLMEngine:
             flight = self._launch(scheduled)
         if self.config.run_ahead:
             self._in_flight = self._run_ahead(flight, outputs, now=timestamp)
-        outputs.extend(self._collect(flight, now=timestamp))
+        outputs.extend(self._collect(flight, now=now))
         return outputs
 
     def _launch(self, scheduled: SchedulerOutput, tokens_from=None) -> "_InFlight":
@@ -312,12 +312,14 @@ class LLMEngine:
             patch[index] = source[item.seq.seq_id]
         return self._launch(scheduled, tokens_from=(tokens, patch))
 
-    def _collect(self, flight: "_InFlight", *, now: float) -> list[RequestOutput]:
+    def _collect(self, flight: "_InFlight", *, now: float | None) -> list[RequestOutput]:
         """Wait for a launched step's tokens and feed them back: stop checks, text, per-request
         deltas (engine.py:366-410)."""
         if flight.pending is None:
             return []
         result = flight.pending.read()
+        if now is None:  # the tokens exist from here on, not from when the call began
+            now = time.perf_counter()
         tokens, logprobs = result.token_ids, result.logprobs
         outputs = []
         for index, (item, token) in enumerate(zip(flight.sampled, tokens)):

@@ -111,7 +111,7 @@ def tuning_file() -> str:
 
 
 def make_engine(model, config, *, max_num_seqs: int, budget: int, tokens_per_request: int, fill_hbm: bool = False,
-                tune_tokens: tuple[int, ...] = (), run_ahead: bool = True):
+                tune_tokens: tuple[int, ...] = (), run_ahead: bool = True, step_sizes: bool = False):
     """An ``LLMEngine`` around the already loaded model, with a cache pool for ``max_num_seqs``
     requests of ``tokens_per_request`` tokens (or, with ``fill_hbm``, 90% of the free memory)."""
     import torch
@@ -126,7 +126,7 @@ def make_engine(model, config, *, max_num_seqs: int, budget: int, tokens_per_req
         num_blocks = max(num_blocks, int(free * 0.9) // page_bytes)
     engine_config = EngineConfig(
         model="(random weights)", dtype="bfloat16" if model.runtime.dtype == torch.bfloat16 else "float32", seed=0,
-        tune_gemm_tokens=tune_tokens, gemm_tuning_file=tuning_file(), run_ahead=run_ahead,
+        tune_gemm_tokens=tune_tokens, tune_gemm_step_sizes=step_sizes, gemm_tuning_file=tuning_file(), run_ahead=run_ahead,
         scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=budget, block_size=PAGE,
                                   num_blocks=num_blocks),
     )
@@ -278,7 +278,7 @@ def run_closed_loop(model, config, concurrency: int, *, sampled: bool, requests:
     rng = random.Random(1)
     shapes = [(rng.randint(128, 1024), rng.randint(64, 512)) for _ in range(requests)]
     engine = make_engine(model, config, max_num_seqs=concurrency, budget=PREFILL_TOKENS,
-                         tokens_per_request=1024 + 512 + PAGE, tune_tokens=(PREFILL_TOKENS,) if tune else ())
+                         tokens_per_request=1024 + 512 + PAGE, step_sizes=tune)
     prompts = [random_prompts(config, 1, length, 100 + index)[0] for index, (length, _) in enumerate(shapes)]
 
     def params(index: int) -> "SamplingParams":

@@ -302,6 +302,41 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
         torch.cuda.tunable.enable(False)
 
 
+def test_library_products_at_timed_step_sizes(model, tmp_path):
+    """An engine told to run the library's products at a few timed sizes: prompts of lengths
+    between the sizes, alone and cut into portions beside decoded tokens, give the plain
+    implementation's log-probabilities, and their products did run at the sizes."""
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    prompts = [tiny.random_tokens(model["vocab"], length, 900 + length) for length in (131, 203, 250, 390)]
+    sampling = SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True, logprobs=True)
+    engine = LLMEngine(EngineConfig(
+        model=str(model["bf16_folder"]), dtype="bfloat16", tune_gemm_step_sizes=True, gemm_tuning_file=str(tmp_path / "choices.csv"),
+        scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=300, block_size=model["page"], num_blocks=96),
+    ))
+    lengths = []
+    mm, addmm = torch.mm, torch.addmm
+    try:
+        ops = engine.model.runtime.ops
+        assert ops.library_buckets == (32, 64, 96, 128, 160, 192, 224, 256, 300)
+        torch.mm = lambda a, *rest, **kw: (lengths.append(a.shape[0]), mm(a, *rest, **kw))[1]
+        torch.addmm = lambda c, a, *rest, **kw: (lengths.append(a.shape[0]), addmm(c, a, *rest, **kw))[1]
+        outs = engine.generate(prompts[:1], sampling) + engine.generate(prompts[1:2], sampling)
+        assert set(lengths) == {160, 224}, "131 and 203 tokens, each at the next size up"
+        outs += engine.generate(prompts[2:], sampling)
+    finally:
+        torch.mm, torch.addmm = mm, addmm
+        engine.close()
+        torch.cuda.tunable.enable(False)
+    assert set(lengths) <= set(ops.library_buckets), sorted(set(lengths))
+    for prompt, out in zip(prompts, outs):
+        sequence = prompt + out.new_token_ids
+        logits = plain.forward_logits(model["bf16_raw"], model["bf16_tensors"], sequence)
+        check_logprobs(logits[len(prompt) - 1:], out)
+
+
 @pytest.mark.parametrize("count", [40, 100])
 def test_many_requests_decode_together(model, count):
     """40 and 100 requests decoding in one batch (recorded steps of 64 and 128 rows, the tiled

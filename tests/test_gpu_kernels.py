@@ -200,6 +200,44 @@ def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
             x.to(DEV), w.to(DEV), torch.zeros(2 * inter).bfloat16().to(DEV), plan=plan, gated=True)
 
 
+def test_library_product_at_a_larger_size_ignores_the_rows_behind(ops):
+    """With sizes set for the library's products, a step's activations are allocated up to the
+    next size and the product runs that long; the rows behind the step's own (not-a-numbers
+    here) reach no row of the result, and a buffer without the room runs at its own size."""
+    from turboserve_amd.kernels.ops import Ops
+
+    sized = Ops(DEV)
+    sized.library_buckets = (192, 256)
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(150, 264, generator=g).bfloat16()
+    w = (torch.randn(136, 264, generator=g) / 16).bfloat16()
+    b = torch.randn(136, generator=g).bfloat16()
+    ref = x.float() @ w.float().t()
+    buffer = sized.rows_buffer(150, 264, torch.bfloat16, DEV)
+    assert buffer.shape == (150, 264) and buffer.untyped_storage().nbytes() == 192 * 264 * 2
+    buffer.as_strided((192, 264), (264, 1)).fill_(float("nan"))
+    buffer.copy_(x)
+    lengths = []
+    mm, addmm = torch.mm, torch.addmm
+    try:
+        torch.mm = lambda a, *rest, **kw: (lengths.append(a.shape[0]), mm(a, *rest, **kw))[1]
+        torch.addmm = lambda c, a, *rest, **kw: (lengths.append(a.shape[0]), addmm(c, a, *rest, **kw))[1]
+        got = sized.linear(buffer, w.to(DEV))
+        biased = sized.linear(buffer, w.to(DEV), b.to(DEV))
+        wide = sized.linear_float32_out(buffer, w.to(DEV))
+        tight = sized.linear(x.to(DEV), w.to(DEV))
+        unsized = ops.linear(buffer, w.to(DEV))
+    finally:
+        torch.mm, torch.addmm = mm, addmm
+    assert lengths == [192, 192, 192, 150, 150]
+    for result in (got, tight, unsized):
+        assert result.shape == (150, 136)
+        torch.testing.assert_close(result.float().cpu(), ref, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(biased.float().cpu(), ref + b.float(), rtol=2e-2, atol=3e-2)
+    assert wide.dtype == torch.float32 and wide.shape == (150, 136)
+    torch.testing.assert_close(wide.cpu(), ref, rtol=2e-2, atol=2e-2)
+
+
 def test_gemm_skinny_rows_do_not_depend_on_the_batch(ops):
     """A row's sums are the same bits whatever else is in the batch, for a given grid of the
     tiled kernel and within the resident kernel; between grids the ranges of K differ, so only

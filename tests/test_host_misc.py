@@ -5,6 +5,7 @@ from __future__ import annotations
 
 import numpy as np
 import pytest
+import torch
 
 from turboserve_amd.cli import build_parser
 from turboserve_amd.engine.batch import StepEntry, StepLayout, StepLimits, build_context, check_packed, pack_step, validate_entries
@@ -362,3 +363,34 @@ def test_tiled_product_plans_are_the_ones_measured_best():
     assert plan(8, 7168, h14, None) == (10, 4, 2)         # 14B qkv: four ranges, two workgroups a unit
     assert plan(8, 2 * i14, h14, None) == (40, 1, 2)      # 14B gate+up: 432 small workgroups
     assert plan(128, h7, i7, None)[2] != 2                # above 64 rows LDS holds one workgroup: no pairs to count on
+
+
+def test_library_products_run_at_a_few_sizes():
+    """The sizes at which the BLAS library's products are run when they are all timed: a step is
+    at most a quarter longer than it had to be, the token budget is a size itself, decode-sized
+    steps keep their own size, and a buffer is seen longer only if its storage reaches that far."""
+    from turboserve_amd.kernels.ops import Ops
+
+    class Sized(Ops):
+        def __init__(self, sizes):
+            self.library_buckets = sizes
+
+    sizes = Ops.bucket_sizes(2000)
+    assert sizes[-1] == 2000 and list(sizes) == sorted(set(sizes))
+    assert {32, 256, 320, 512, 640, 1024, 1280, 1792}.issubset(sizes) and 288 not in sizes and 576 not in sizes
+    assert Ops.bucket_sizes(100) == (32, 64, 96, 100)
+    ops = Sized(sizes)
+    assert ops.library_rows(1) == 1 and ops.library_rows(128) == 128, "decode-sized steps use the engine's own products"
+    for rows in range(129, 2001):
+        at = ops.library_rows(rows)
+        assert at in sizes and rows <= at <= rows * 1.25
+    assert ops.library_rows(2001) == 2001, "beyond the largest size a step keeps its own"
+    assert Sized(()).library_rows(777) == 777
+    buffer = ops.rows_buffer(130, 8, torch.float32, "cpu")
+    assert buffer.shape == (130, 8) and buffer.is_contiguous()
+    seen = Ops._with_room(buffer, 160)
+    assert seen.shape == (160, 8) and seen.data_ptr() == buffer.data_ptr()
+    assert Ops._with_room(torch.empty(130, 8), 160) is None, "no room behind it"
+    assert Ops._with_room(torch.empty(160, 16)[:130, :8], 160) is None, "rows that are not dense"
+    assert Ops._with_room(torch.empty(4, 160, 8)[1, :130], 160).shape == (160, 8)
+    assert Ops._with_room(torch.empty(4, 160, 8)[3, 10:140], 160) is None, "it would run past the end"

@@ -38,6 +38,9 @@ def _add_engine_options(p: argparse.ArgumentParser, *, max_num_seqs: int) -> Non
     p.set_defaults(prefix_caching=False)
     p.add_argument("--tune-gemm", action="store_true",
                    help="time the BLAS library's kernels for a full step of prompt tokens at start-up and keep the fastest")
+    p.add_argument("--tune-gemm-step-sizes", action="store_true",
+                   help="run every step's BLAS products at one of a few sizes and time the library's kernels at all of them "
+                        "at start-up (a minute or two the first time; kept in a per-user file)")
     p.add_argument("--run-ahead", dest="run_ahead", action="store_true",
                    help="launch each decode step before the host has read the tokens of the step before it (the default)")
     p.add_argument("--no-run-ahead", dest="run_ahead", action="store_false",
@@ -98,6 +101,7 @@ def _generate(args: argparse.Namespace) -> int:
     config = EngineConfig(
         model=args.model, device=args.device, dtype=args.dtype, seed=args.seed,
         tune_gemm_tokens=(args.max_num_batched_tokens,) if args.tune_gemm else (),
+        tune_gemm_step_sizes=getattr(args, "tune_gemm_step_sizes", False),
         run_ahead=getattr(args, "run_ahead", True),
         scheduler=SchedulerConfig(
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,

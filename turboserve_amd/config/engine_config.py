@@ -66,6 +66,12 @@ class EngineConfig:
     #: timed at start-up and the fastest kept (bfloat16 only; a few seconds per size).  Empty:
     #: the library's own heuristic picks.  No counterpart in the reference.
     tune_gemm_tokens: tuple[int, ...] = ()
+    #: Run the library products of every step at one of a few sizes (the next one up: multiples
+    #: of 32 tokens to 256, of 64 to 512, of 128 to 1,024, of 256 beyond, and the token budget)
+    #: and time the library's kernels at all of them at start-up, so that every step, not only
+    #: one of a listed size, runs on timed kernels (bfloat16 only; a minute or two the first
+    #: time, read from ``gemm_tuning_file`` afterwards).  No counterpart in the reference.
+    tune_gemm_step_sizes: bool = False
     #: Where the timed choices are kept between runs; None is a per-user cache file.
     gemm_tuning_file: str | None = None
     #: Launch a decode step before the host has read the tokens of the step before it (they

@@ -129,7 +129,7 @@ class LLMEngine:
         self.scheduler = scheduler
         self.runner = runner if runner is not None else ModelRunner(model, storage)
         self.sampler = sampler if sampler is not None else Sampler(model.runtime.ops)
-        if config.tune_gemm_tokens and runner is None:
+        if (config.tune_gemm_tokens or config.tune_gemm_step_sizes) and runner is None:
             self._tune_library_products()
         self._decoders: dict[str, StreamingDecoder] = {}
         self._seed = config.seed if config.seed is not None else time.time_ns() & 0xFFFFFFFF
@@ -154,13 +154,17 @@ class LLMEngine:
         from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
 
         budget = self.config.scheduler.max_num_batched_tokens
+        sizes = {min(t, budget) for t in self.config.tune_gemm_tokens}
+        if self.config.tune_gemm_step_sizes:
+            ops = self.model.runtime.ops
+            ops.library_buckets = ops.bucket_sizes(budget)
+            sizes.update(size for size in ops.library_buckets if size > ops.skinny_max_rows)
         started = time.perf_counter()
         with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
-            for tokens in sorted({min(t, budget) for t in self.config.tune_gemm_tokens}):
+            for tokens in sorted(sizes):
                 self.runner.dry_run(tokens)
         logger.info("library products timed for steps of %s tokens in %.1f s (%d choices kept in %s)",
-                    list(self.config.tune_gemm_tokens), time.perf_counter() - started, tuning.num_results(),
-                    tuning.results_file)
+                    sorted(sizes), time.perf_counter() - started, tuning.num_results(), tuning.results_file)
 
     def _resolve_eos_token_ids(self) -> frozenset[int]:
         """Every id that ends a generation: the checkpoint configuration's and the tokenizer's

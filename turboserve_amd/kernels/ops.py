@@ -236,7 +236,7 @@ class Ops:
         if pending is not None:
             is_f32, splits, stride = self._partials(pending, tokens, hidden, weight.dtype, "pending")
         out_rows = tokens if rows is None else rows.numel()
-        y = torch.empty((out_rows, hidden), dtype=weight.dtype, device=residual.device)
+        y = self.rows_buffer(out_rows, hidden, weight.dtype, residual.device)
         _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight),
                                         _ptr(rows), float(eps), out_rows, hidden, dtype_code(weight.dtype),
                                         self.stream()), "ts_add_rmsnorm")
@@ -255,7 +255,7 @@ class Ops:
             _need(dtype is not None, "partial sums need the output dtype")
         is_f32, splits, stride = self._partials(gate_up, tokens, width, out_dtype, "gate_up")
         inter = width // 2
-        out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
+        out = self.rows_buffer(tokens, inter, out_dtype, gate_up.device)
         _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
                                    1 if paired else 0, dtype_code(out_dtype), self.stream()), "ts_swiglu")
         return out
@@ -690,6 +690,52 @@ class Ops:
             return True
         return m <= self.resident_wide_rows and -(-n // 160) >= 200
 
+    #: Row counts that steps of more rows than the decode products take are run at by the BLAS
+    #: library (ascending; empty: every step at its own size).  The library's choice of kernel is
+    #: only as good as its heuristic unless a shape has been timed, and a serving engine meets
+    #: every row count; with a short list of sizes all of them can be timed at start-up
+    #: (``LLMEngine`` sets the list when it is asked to time them).  A step runs at the next size
+    #: up: its activation buffers are allocated that long (``rows_buffer``) and the rows beyond the
+    #: step's own hold whatever was there; products are row by row, so nothing of it reaches a
+    #: row that is read.
+    library_buckets: tuple[int, ...] = ()
+
+    @staticmethod
+    def bucket_sizes(limit: int) -> tuple[int, ...]:
+        """The sizes up to ``limit`` (which is one itself): multiples of 32 to 256, of 64 to 512,
+        of 128 to 1,024, of 256 beyond, so that a step is at most a quarter longer than it had
+        to be."""
+        sizes = {limit}
+        for step, end in ((32, 256), (64, 512), (128, 1024), (256, limit)):
+            sizes.update(range(step, min(end, limit) + 1, step))
+        return tuple(sorted(sizes))
+
+    def library_rows(self, rows: int) -> int:
+        """The row count a library product of ``rows`` rows is run at."""
+        if rows <= self.skinny_max_rows:
+            return rows
+        for size in self.library_buckets:
+            if size >= rows:
+                return size
+        return rows
+
+    def rows_buffer(self, rows: int, width: int, dtype: torch.dtype, device) -> torch.Tensor:
+        """``[rows, width]`` for a step's activations, with room behind it up to the size a
+        library product of these rows is run at."""
+        return torch.empty((self.library_rows(rows), width), dtype=dtype, device=device)[:rows]
+
+    @staticmethod
+    def _with_room(x: torch.Tensor, rows: int) -> torch.Tensor | None:
+        """``x`` seen ``rows`` long, if its rows are dense and its storage reaches that far."""
+        if rows == x.shape[0]:
+            return x
+        if x.dim() != 2 or x.stride(1) != 1 or x.stride(0) != x.shape[1]:
+            return None
+        needed = (x.storage_offset() + rows * x.shape[1]) * x.element_size()
+        if needed > x.untyped_storage().nbytes():
+            return None
+        return x.as_strided((rows, x.shape[1]), (x.shape[1], 1))
+
     #: Products with fewer multiply-adds than this never use a timed choice of the BLAS library's
     #: kernels, only its default: timing them is noise, and one of the library's candidates for
     #: such a shape ([200, 64] x [256, 64]) returned garbage once in about eight processes.
@@ -697,7 +743,12 @@ class Ops:
 
     def _library_product(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
                          out_dtype: torch.dtype | None) -> torch.Tensor:
-        """``x @ weight^T (+ bias)`` by the BLAS library behind torch."""
+        """``x @ weight^T (+ bias)`` by the BLAS library behind torch, at the row count of
+        :meth:`library_rows` when ``x`` has the room (see ``library_buckets``)."""
+        rows = x.shape[0]
+        roomy = self._with_room(x, self.library_rows(rows))
+        if roomy is not None and roomy.shape[0] != rows:
+            return self._library_product(roomy, weight, bias, out_dtype)[:rows]
         tunable = torch.cuda.tunable
         small = x.shape[0] * weight.shape[0] * weight.shape[1] < self.library_tuning_min_work
         paused = small and tunable.is_enabled()

@@ -116,7 +116,7 @@ class GroupedQueryAttention(Mixer):
         slopes = self.position.score_slopes(self.num_heads)
         fast = slopes is None and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
         if fast:
-            out = torch.empty((ctx.num_tokens, self.q_size), dtype=qkv.dtype, device=qkv.device)
+            out = ops.rows_buffer(ctx.num_tokens, self.q_size, qkv.dtype, qkv.device)
             if ctx.num_prefill_seqs > 0:
                 # The launch's list of row blocks is the same for every layer with this geometry.
                 rows = ops.prefill_block_rows(self.head_dim, self.num_heads, self.num_kv_heads)

@@ -344,7 +344,7 @@ def run_attention_prefill(shape: dict, tokens: int, context: int, launches: int 
     starts = torch.tensor([0, tokens], dtype=torch.int32, device="cuda")
     contexts = torch.tensor([context], dtype=torch.int32, device="cuda")
     rows = ops.prefill_block_rows(dim, heads, kv_heads)
-    blocks = ops.prefill_blocks([tokens], [context], rows)
+    blocks = ops.prefill_blocks([tokens], [context], rows, heads=heads, kv_heads=kv_heads, head_dim=dim, block_size=PAGE)
     out = torch.empty(tokens, heads * dim, dtype=torch.bfloat16, device="cuda")
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     best = float("inf")

@@ -645,6 +645,80 @@ def test_attention_prefill_mfma_every_launch_plan(ops, heads, kv_heads, dim, tok
     torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
 
 
+def shared_out_work(case, seqs, window, shares_wanted):
+    """A work list in which every block of 32 rows with two or more windows of keys is shared out
+    over up to ``shares_wanted`` workgroups, written out from the entry point's description."""
+    from turboserve_amd.kernels.ops import PrefillWork, prefill_block_windows
+
+    blocks, ranges, combine, slot = [], [], [], 0
+    for s, (ctx, qlen) in enumerate(seqs):
+        for offset in range(0, qlen, 32):
+            here = min(32, qlen - offset)
+            windows = prefill_block_windows(ctx - qlen + offset, here, window or 0)
+            shares = min(shares_wanted, windows)
+            if shares < 2:
+                blocks.append((s, case.qsl[s] + offset))
+                ranges.append((0, 0, -1))
+                continue
+            each = -(-windows // shares)
+            shares = -(-windows // each)
+            combine.append((case.qsl[s] + offset, here, slot, shares))
+            for share in range(shares):
+                blocks.append((s, case.qsl[s] + offset))
+                ranges.append((share * each, min(each, windows - share * each), slot))
+                slot += 1
+    order = list(range(len(blocks)))
+    random.Random(5).shuffle(order)
+    return PrefillWork(case.ints([blocks[i] for i in order]), case.ints([ranges[i] for i in order]),
+                       case.ints(combine), slot)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,page", [g for g in ATTENTION_GEOMETRIES if g[0] // g[1] >= 3 and g[2] % 32 == 0 and g[2] <= 128])
+@pytest.mark.parametrize("window", [None, 20, 300])
+@pytest.mark.parametrize("shares", [2, 3, 16])
+def test_attention_prefill_mfma_with_shared_out_blocks(ops, heads, kv_heads, dim, page, window, shares):
+    """The keys of a block shared out over two, three and sixteen workgroups (fewer where a block
+    has fewer windows; a share of one window included), whole blocks beside them, ragged last
+    blocks, windows that cut shares off from some rows: the combined result is the plain one."""
+    seqs = [(70, 70), (33, 2), (600, 77), (129, 16), (257, 17), (48, 48), (2, 2), (515, 33), (1000, 64)]
+    case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, window, seed=dim + 5)
+    assert ops.prefill_block_rows(dim, heads, kv_heads) == 32
+    work = shared_out_work(case, seqs, window, shares)
+    assert work.slots >= 4
+    out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(
+        out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+        case.ints(case.qsl), case.ints([c for c, _ in seqs]), work, heads, dim ** -0.5, window,
+        max(c for c, _ in seqs), 32,
+    )
+    torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+
+
+def test_attention_prefill_mfma_shares_by_the_planner(ops, monkeypatch):
+    """The work lists :meth:`Ops.prefill_blocks` makes itself: a short portion at the end of a
+    long context beside another request's (every long block shared out several times) with a far
+    key that carries the result, a prompt of 5,000 tokens on one KV head (a quarter of the
+    workgroups: long shares), and prompts that fill the device or are short (nothing shared
+    out); each against the plain attention."""
+    heads, kv_heads, dim, page = 28, 4, 128, 16
+    for seqs, spike, shared in (([(6000, 96), (300, 40)], 77, True), ([(2048, 2048)], None, False),
+                                ([(500, 500), (90, 90)], None, False), ([(5000, 5000)], None, True)):
+        if seqs[0][0] == 5000:
+            heads, kv_heads = 7, 1  # (and the plain attention on the host takes a quarter of the time)
+        case = PagedCase(torch.bfloat16, heads, kv_heads, dim, page, seqs, None, seed=21, spike=spike)
+        work = ops.prefill_blocks([q for _, q in seqs], [c for c, _ in seqs], 32, heads=heads, kv_heads=kv_heads,
+                                  head_dim=dim, block_size=page)
+        assert (work.ranges is not None) == shared, seqs
+        out = torch.zeros(case.qsl[-1], heads * dim, dtype=torch.bfloat16, device=DEV)
+        ops.attention_prefill(
+            out, case.dev(case.q), heads * dim, case.dev(case.kp), case.dev(case.vp), case.dev(case.table),
+            case.ints(case.qsl), case.ints([c for c, _ in seqs]), work, heads, dim ** -0.5, None, max(c for c, _ in seqs), 32,
+        )
+        torch.testing.assert_close(out.float().cpu(), case.expected, **tol(torch.bfloat16))
+        if spike is not None:
+            assert float(case.expected[:96].abs().mean()) > 4.0
+
+
 def test_attention_prefill_mfma_far_key(ops):
     heads, kv_heads, dim, page = 28, 4, 128, 16
     seqs = [(3000, 40), (2100, 2100)]

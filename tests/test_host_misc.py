@@ -394,3 +394,71 @@ def test_library_products_run_at_a_few_sizes():
     assert Ops._with_room(torch.empty(160, 16)[:130, :8], 160) is None, "rows that are not dense"
     assert Ops._with_room(torch.empty(4, 160, 8)[1, :130], 160).shape == (160, 8)
     assert Ops._with_room(torch.empty(4, 160, 8)[3, 10:140], 160) is None, "it would run past the end"
+
+
+def test_prefill_work_list_shares_out_long_blocks():
+    """The planner of the prefill attention's work list: every window of every block is taken by
+    exactly one entry, shares of a block lie in consecutive slots, nothing is shared out where
+    the device is busy anyway or a block is short, and what it picks is no slower, played
+    through, than whole blocks."""
+    from turboserve_amd.kernels.ops import prefill_block_list, prefill_block_windows, prefill_share_list
+
+    assert prefill_block_windows(0, 32, 0) == 1 and prefill_block_windows(31, 2, 0) == 2
+    assert prefill_block_windows(2016, 32, 0) == 64 and prefill_block_windows(2016, 32, 100) == 5
+    assert prefill_block_windows(100, 1, 33) == 2  # keys 68..100: windows 64.. and 96..
+
+    def check(query_lens, context_lens, window, per_block, places, min_windows=16):
+        blocks, ranges, combine = prefill_share_list(query_lens, context_lens, 32, window, per_block, places, min_windows)
+        if not ranges:
+            assert blocks == prefill_block_list(query_lens, context_lens, 32) and combine == []
+            return blocks, ranges, combine
+        assert len(blocks) == len(ranges)
+        taken, first_row, sizes = {}, 0, []
+        starts = []
+        for count in query_lens:
+            starts.append(first_row)
+            first_row += count
+        for (request, row), (first, windows, slot) in zip(blocks, ranges):
+            offset = row - starts[request]
+            here = min(32, query_lens[request] - offset)
+            total = prefill_block_windows(context_lens[request] - query_lens[request] + offset, here, window)
+            span = range(total) if slot < 0 else range(first, first + windows)
+            assert slot >= 0 or (first, windows) == (0, 0)
+            assert windows >= 1 or slot < 0
+            sizes.append(len(span))
+            for w in span:
+                assert 0 <= w < total and (request, row, w) not in taken
+                taken[(request, row, w)] = slot
+        covered = sum(prefill_block_windows(c - q + o, min(32, q - o), window)
+                      for q, c in zip(query_lens, context_lens) for o in range(0, q, 32))
+        assert len(taken) == covered
+        assert sizes == sorted(sizes, reverse=True), "the longest entries start first"
+        slots_seen = sorted(slot for _, _, slot in ranges if slot >= 0)
+        assert slots_seen == list(range(len(slots_seen)))
+        for row, rows, first_slot, shares in combine:
+            assert 2 <= shares <= 16 and 1 <= rows <= 32
+            members = [(b, r) for b, r in zip(blocks, ranges) if first_slot <= r[2] < first_slot + shares]
+            assert len(members) == shares and all(b[1] == row for b, _ in members)
+            assert sorted(r[0] for _, r in members) == [r[0] for _, r in sorted(members, key=lambda m: m[1][2])]
+        assert sum(c[3] for c in combine) == len(slots_seen)
+        return blocks, ranges, combine
+
+    # a short portion at the end of a long context: every block several times, all at once
+    blocks, ranges, combine = check([512], [8192], 0, 4, 256)
+    assert len(combine) == 16 and all(c[3] == 4 for c in combine) and len(blocks) * 4 == 256
+    blocks, ranges, combine = check([128], [16384], 0, 4, 256)
+    assert len(combine) == 4 and all(c[3] == 16 for c in combine)
+    # whole blocks that fill the device stay whole (a second workgroup's start costs more than
+    # the shorter blocks save), and so do blocks too short to be worth putting together
+    assert check([2048], [2048], 0, 4, 256)[1] == []
+    assert check([8192], [8192], 0, 4, 256)[1] == []
+    assert check([2048], [8192], 0, 4, 256)[1] == []
+    assert check([600, 40], [600, 900], 0, 4, 256)[1] == []
+    # a sliding window makes every block short
+    assert check([512], [8192], 128, 4, 256)[1] == []
+    # shares and whole blocks of several requests; a window that leaves long blocks
+    blocks, ranges, combine = check([300, 100, 33], [4000, 150, 2000], 0, 8, 512, min_windows=4)
+    assert combine and any(r[2] < 0 for r in ranges)
+    assert check([64, 64], [3000, 4000], 1024, 4, 256, min_windows=8)[1]
+    check([5], [5], 0, 4, 256)
+    check([], [], 0, 4, 256)

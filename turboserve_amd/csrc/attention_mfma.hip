@@ -1107,7 +1107,8 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
                     const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
                     const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
                     int pair_blocks, int group_heads, int heads, int kv_heads, int block_shift, float scale_log2,
-                    int window) {
+                    int window, const int* __restrict__ ranges, float* __restrict__ partial_acc,
+                    float* __restrict__ partial_ml) {
   extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
   uint16_t* ks = staged;
   uint16_t* vs = staged + 2 * K_TILE;
@@ -1140,10 +1141,36 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   const int lo_col = (window > 0 && p_col - window + 1 > 0) ? p_col - window + 1 : 0;
   const int p_last = pos0 + cols - 1;
   const int lo_first = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-  const int begin = lo_first & ~(WINDOW_KEYS - 1);
-  const int end = p_last + 1;
+  int begin = lo_first & ~(WINDOW_KEYS - 1);
+  int end = p_last + 1;
+  // A block whose keys are shared out over several workgroups: this one takes `count` windows
+  // from the block's window `first` on and leaves its sums, not yet divided, in slot `slot` for
+  // prefill_combine_kernel.  What a column may see is still decided by its own position.
+  int slot = -1;
+  if (ranges) {
+    const int first = ranges[3 * block];
+    const int count = ranges[3 * block + 1];
+    slot = ranges[3 * block + 2];
+    if (count > 0) {
+      begin += first * WINDOW_KEYS;
+      end = min(end, begin + count * WINDOW_KEYS);
+    }
+  }
   const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
   auto interior = [&](int w) { return cols == WIDE_ROWS && w >= lo_last && w + WINDOW_KEYS - 1 <= pos0; };
+  if (begin >= end) {
+    // A share that lies past the block's keys (no work list of this library's makes one): it
+    // has seen nothing, and says so.  The whole workgroup leaves here, before any barrier.
+    if (slot >= 0 && wave_live) {
+      const size_t entry = ((size_t)slot * heads + kvh * gsize + hg) * WIDE_ROWS + col;
+      for (int d = 4 * half; d < D; d += 8) *reinterpret_cast<f32x4*>(partial_acc + entry * D + d) = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (half == 0) {
+        partial_ml[entry * 2] = -INFINITY;
+        partial_ml[entry * 2 + 1] = 0.f;
+      }
+    }
+    return;
+  }
 
   PageGeometry geo{k_pages, v_pages, block_table + (size_t)seq * table_width, table_width, kv_heads, kvh, block_shift,
                    (1 << block_shift) - 1};
@@ -1356,7 +1383,9 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   // so that the steady one is a loop of its own to the compiler: general rounds up to an even
   // round at or past steady_from, steady pairs of rounds, general rounds to the end.
   const int steady_from = (lo_last - begin + WINDOW_KEYS - 1) / WINDOW_KEYS;
-  const int steady_to = cols == WIDE_ROWS ? (pos0 + 1 - begin) / WINDOW_KEYS - 6 : -1;
+  // (a workgroup with a share of the block's windows ends before the block does: its last rounds
+  // ask for windows past its share, which exist and are dropped.)
+  const int steady_to = cols == WIDE_ROWS ? min((pos0 + 1 - begin) / WINDOW_KEYS - 6, rounds - 1) : -1;
   auto run = [&](auto moves, auto computes) __attribute__((always_inline)) {
     constexpr std::integral_constant<int, 0> even{};
     constexpr std::integral_constant<int, 1> odd{};
@@ -1387,6 +1416,25 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
 
   float la, lb;
   swap_rows(l, true, la, lb);
+  if (slot >= 0) {
+    // A share of a block: the sums as they are, with the reference they were taken against.
+    // Columns past the block's rows saw nothing (m = -inf, zeros) and are written like the rest.
+    if (wave_live) {
+      const size_t entry = ((size_t)slot * heads + kvh * gsize + hg) * WIDE_ROWS + col;
+      float* arow = partial_acc + entry * D + 4 * half;
+#pragma unroll
+      for (int t = 0; t < NT32; ++t)
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          *reinterpret_cast<f32x4*>(arow + 32 * t + 8 * a) =
+              f32x4{acc[t][4 * a], acc[t][4 * a + 1], acc[t][4 * a + 2], acc[t][4 * a + 3]};
+      if (half == 0) {
+        partial_ml[entry * 2] = m;
+        partial_ml[entry * 2 + 1] = la + lb;
+      }
+    }
+    return;
+  }
   if (col_valid && wave_live) {
     const float inv = 1.f / (la + lb);
     uint16_t* orow = out + ((size_t)(row0 + col) * heads + kvh * gsize + hg) * D + 4 * half;
@@ -1402,11 +1450,55 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   }
 }
 
+// The blocks whose keys were shared out: combine[4 c ..] = (first row, rows, first slot, shares)
+// of block c, whose shares lie in consecutive slots.  out = sum_s acc_s 2^(m_s - M) / sum_s l_s
+// 2^(m_s - M) with M the largest reference among the shares, as in decode_reduce_kernel.
+// grid (blocks to combine, heads), 256 threads: a thread takes four head dimensions of one row.
+constexpr int COMBINE_THREADS = 256;
+constexpr int PREFILL_MAX_SHARES = 16;
+
+__global__ void __launch_bounds__(COMBINE_THREADS)
+prefill_combine_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_acc,
+                       const float* __restrict__ partial_ml, const int* __restrict__ combine, int heads) {
+  const int row0 = combine[4 * blockIdx.x];
+  const int rows = combine[4 * blockIdx.x + 1];
+  const int first_slot = combine[4 * blockIdx.x + 2];
+  const int shares = combine[4 * blockIdx.x + 3];
+  const int head = blockIdx.y;
+  for (int c = threadIdx.x; c < rows * (D / 4); c += COMBINE_THREADS) {
+    const int col = c / (D / 4);
+    const int d = 4 * (c % (D / 4));
+    float m[PREFILL_MAX_SHARES], l[PREFILL_MAX_SHARES];
+    f32x4 part[PREFILL_MAX_SHARES];
+    float m_max = -INFINITY;
+#pragma unroll
+    for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
+      const size_t entry = ((size_t)(first_slot + min(sh, shares - 1)) * heads + head) * WIDE_ROWS + col;
+      m[sh] = sh < shares ? partial_ml[entry * 2] : -INFINITY;
+      l[sh] = partial_ml[entry * 2 + 1];
+      part[sh] = *reinterpret_cast<const f32x4*>(partial_acc + entry * D + d);
+      m_max = fmaxf(m_max, m[sh]);
+    }
+    float den = 0.f;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
+      const float wgt = (m[sh] == -INFINITY) ? 0.f : exp2f(m[sh] - m_max);  // a share that saw nothing, or none
+      den += l[sh] * wgt;
+      sum += part[sh] * wgt;
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    *reinterpret_cast<u32x2*>(out + ((size_t)(row0 + col) * heads + head) * D + d) =
+        Frag4{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
+  }
+}
+
 static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t* q, long q_stride,
                                const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
                                int table_width, const int* query_start_loc, const int* context_lens,
                                const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
-                               float scale_log2, int window, int max_context) {
+                               float scale_log2, int window, int max_context, const int* ranges,
+                               float* partial_acc, float* partial_ml, const int* combine, int num_combine) {
   constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
   static_assert(lds <= 64 * 1024, "two workgroups' staged windows must fit in LDS");
   const int gsize = heads / kv_heads;
@@ -1429,8 +1521,9 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
   const int fed_chunks = (gsize + FED_MAX_HEADS - 1) / FED_MAX_HEADS;
   const int fed_heads = (gsize + fed_chunks - 1) / fed_chunks;
   const long long self_total = (long long)num_blocks * kv_heads * ((gsize + STAGE_WAVES - 1) / STAGE_WAVES);
-  const bool self_fits = self_total > compute_units && self_total <= 2LL * compute_units && max_context > 0 &&
-                         max_context <= (long long)num_blocks * WIDE_ROWS;
+  // (A work list with shared-out blocks was balanced for the fed form where the geometry has it.)
+  const bool self_fits = !ranges && self_total > compute_units && self_total <= 2LL * compute_units &&
+                         max_context > 0 && max_context <= (long long)num_blocks * WIDE_ROWS;
   const bool fed = fed_heads >= FED_MIN_HEADS && shift >= 4 && !self_fits;
   const int group_heads = fed ? fed_heads : STAGE_WAVES;
   const int chunks = (gsize + group_heads - 1) / group_heads;
@@ -1441,14 +1534,32 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
     // take the lighter ones.
     hipLaunchKernelGGL(prefill_wide_kernel<true>, dim3((unsigned)total), dim3((group_heads + 1) * TS_WAVE), lds, stream,
                        out, q, q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens,
-                       blocks, num_blocks, 0, group_heads, heads, kv_heads, shift, scale_log2, window);
-    return ts_launch_status();
+                       blocks, num_blocks, 0, group_heads, heads, kv_heads, shift, scale_log2, window, ranges,
+                       partial_acc, partial_ml);
+  } else {
+    const int pair_blocks = (!ranges && total <= 2LL * compute_units) ? 1 : 0;
+    hipLaunchKernelGGL(prefill_wide_kernel<false>, dim3((unsigned)total), dim3(STAGE_WAVES * TS_WAVE), lds, stream, out,
+                       q, q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks,
+                       num_blocks, pair_blocks, group_heads, heads, kv_heads, shift, scale_log2, window, ranges,
+                       partial_acc, partial_ml);
   }
-  const int pair_blocks = total <= 2LL * compute_units ? 1 : 0;
-  hipLaunchKernelGGL(prefill_wide_kernel<false>, dim3((unsigned)total), dim3(STAGE_WAVES * TS_WAVE), lds, stream, out, q,
-                     q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, context_lens, blocks,
-                     num_blocks, pair_blocks, group_heads, heads, kv_heads, shift, scale_log2, window);
+  const int status = ts_launch_status();
+  if (status != TS_OK || num_combine == 0) return status;
+  hipLaunchKernelGGL(prefill_combine_kernel, dim3(num_combine, heads), dim3(COMBINE_THREADS), 0, stream, out, partial_acc,
+                     partial_ml, combine, heads);
   return ts_launch_status();
+}
+
+// Workgroups a block of the work list becomes for this geometry (KV heads x chunks of their query
+// heads) and how many of them a compute unit runs at a time, in the form launch_prefill_wide
+// takes for a list with shared-out blocks: what a caller needs to balance such a list.
+static void prefill_wide_shape(int heads, int kv_heads, int shift, int* per_block, int* per_unit) {
+  const int gsize = heads / kv_heads;
+  const int fed_chunks = (gsize + FED_MAX_HEADS - 1) / FED_MAX_HEADS;
+  const int fed_heads = (gsize + fed_chunks - 1) / fed_chunks;
+  const bool fed = fed_heads >= FED_MIN_HEADS && shift >= 4;
+  *per_block = kv_heads * (fed ? fed_chunks : (gsize + STAGE_WAVES - 1) / STAGE_WAVES);
+  *per_unit = fed ? 1 : 2;
 }
 #endif  // wide prefill
 
@@ -1494,6 +1605,13 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
 // index, first row) of each, rows being token rows of the step.  Writes the rows of
 // `out [T, heads * D]` the blocks cover.  max_context: the longest context among the requests, or 0
 // if the caller does not know it (it only helps to choose a launch plan).
+// ranges (may be null; blocks of 32 rows only): [num_blocks, 3] = (first window, windows, slot) of
+// each entry of `blocks`.  An entry with slot -1 is a whole block (windows 0: all of them).  The
+// others are shares of a block's windows of 32 keys, counted from the block's first window (the
+// one that holds the lowest key its first row sees); a block may appear in `blocks` once per share.
+// Shares leave their sums in partial_acc [slots, heads, 32, D] and partial_ml [slots, heads, 32, 2]
+// (32-bit), and combine [num_combine, 4] = (first row, rows, first slot, shares <= 16) names the
+// blocks to put together afterwards, a block's shares lying in consecutive slots.
 // Rows per block that ts_attention_prefill_d<D> wants in `blocks` for this geometry.
 extern "C" int TS_SYM(ts_attention_prefill_rows_d)(int heads, int kv_heads) {
 #ifdef TS_WIDE_PREFILL
@@ -1504,13 +1622,29 @@ extern "C" int TS_SYM(ts_attention_prefill_rows_d)(int heads, int kv_heads) {
   return 16;
 }
 
+// For a work list with shares (see ts_attention_prefill_d): the workgroups one entry becomes and
+// how many workgroups a compute unit runs at a time; 0, 0 where blocks are not shared out.
+extern "C" void TS_SYM(ts_attention_prefill_shape_d)(int heads, int kv_heads, int block_size, int* per_block,
+                                                     int* per_unit) {
+  *per_block = *per_unit = 0;
+#ifdef TS_WIDE_PREFILL
+  if (kv_heads < 1 || heads % kv_heads != 0 || heads / kv_heads < 3 || block_size < 8) return;
+  int shift = 0;
+  while ((1 << shift) < block_size) ++shift;
+  prefill_wide_shape(heads, kv_heads, shift, per_block, per_unit);
+#endif
+}
+
 extern "C" int TS_SYM(ts_attention_prefill_d)(
     void* out, const void* q, long q_stride, const void* k_pages, const void* v_pages, const int* block_table,
     int table_width, const int* query_start_loc, const int* context_lens, const int* blocks, int num_blocks,
     int block_rows, int heads, int kv_heads, int block_size, float scale, int window, int max_context,
+    const int* ranges, void* partial_acc, void* partial_ml, const int* combine, int num_combine,
     hipStream_t stream) {
   if (num_blocks == 0) return TS_OK;
   if (!out || !q || !k_pages || !v_pages || !block_table || !query_start_loc || !context_lens || !blocks)
+    return TS_ERR_ARG;
+  if (ranges ? (!partial_acc || !partial_ml || num_combine < 0 || (num_combine > 0 && !combine)) : num_combine != 0)
     return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0) return TS_ERR_SHAPE;
   if (block_size < 8 || (block_size & (block_size - 1))) return TS_ERR_SHAPE;
@@ -1522,8 +1656,10 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   if (gsize >= 3)
     return launch_prefill_wide(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                (const uint16_t*)v_pages, block_table, table_width, query_start_loc, context_lens,
-                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window, max_context);
+                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window, max_context, ranges,
+                               (float*)partial_acc, (float*)partial_ml, combine, num_combine);
 #endif
+  if (ranges) return TS_ERR_ARG;  // only blocks of 32 rows are shared out
   // Three or more query heads per KV head: workgroups of four wavefronts, one or two heads each,
   // share every window of keys and values through LDS.
   if (gsize >= 3) {

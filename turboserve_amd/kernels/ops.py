@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
+from dataclasses import dataclass
 
 import torch
 
@@ -69,8 +70,9 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
                                              c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
         f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                              c_int, c_int, c_void_p],
+                                              c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         f"ts_attention_prefill_rows_d{head_dim}": [c_int, c_int],
+        f"ts_attention_prefill_shape_d{head_dim}": [c_int, c_int, c_int, c_void_p, c_void_p],
     }
 
 
@@ -144,6 +146,92 @@ def prefill_block_list(query_lens, context_lens, rows: int) -> list[list[int]]:
         first_row += count
     blocks.sort(key=lambda b: -b[0])
     return [[block[1], block[2]] for block in blocks]
+
+
+#: Keys a round of the prefill attention kernel for blocks of 32 rows takes (its "window").
+PREFILL_WINDOW_KEYS = 32
+#: Most workgroups that share the keys of one block.
+PREFILL_MAX_SHARES = 16
+
+
+def prefill_block_windows(first_position: int, rows: int, window: int) -> int:
+    """Windows of 32 keys that a block of ``rows`` rows, the first at ``first_position``, runs
+    over: from the window that holds the lowest key its first row sees to its last row's own."""
+    lowest = max(0, first_position - window + 1) if window > 0 else 0
+    begin = lowest - lowest % PREFILL_WINDOW_KEYS
+    return -(-(first_position + rows - begin) // PREFILL_WINDOW_KEYS)
+
+
+def prefill_share_list(query_lens, context_lens, rows: int, window: int, per_block: int, places: int,
+                       min_windows: int, *, combine_cost: int = 20):
+    """The work list of the prefill attention with the keys of long blocks shared out over several
+    workgroups, where that shortens the launch: ``(blocks, ranges, combine)`` as lists of
+    ``[request, first row]``, ``[first window, windows, slot]`` (slot -1, windows 0: a whole block) and
+    ``[first row, rows, first slot, shares]``; ``ranges`` and ``combine`` are empty where nothing
+    is shared out and the list is :func:`prefill_block_list`'s.
+
+    An entry becomes ``per_block`` workgroups, ``places`` of which run at a time.  Sharing pays
+    where whole blocks leave places idle (a short portion at the end of a long context: 512
+    tokens behind 7,680 take 84 us instead of 187 on an MI355X), and only as far as every
+    workgroup still has a place at once: a second workgroup's start on a compute unit costs
+    about what ten windows take, so a prompt of 2,048 tokens alone, whose whole blocks fill the
+    device, is slower with its long blocks in two (77 against 66 us).  So the smallest share
+    size (from ``min_windows`` up; a block's windows are spread evenly over its shares) is taken
+    at which all workgroups run at once, if the longest entry gets shorter by more than putting
+    the shares together costs (``combine_cost`` windows: the second kernel and the sums' way
+    through memory)."""
+    whole, first_row = [], 0
+    for index, (count, context) in enumerate(zip(query_lens, context_lens)):
+        for offset in range(0, count, rows):
+            here = min(rows, count - offset)
+            whole.append((prefill_block_windows(context - count + offset, here, window), index, first_row + offset, here))
+        first_row += count
+    plain = prefill_block_list(query_lens, context_lens, rows)
+    longest = max((block[0] for block in whole), default=0)
+    if (rows != PREFILL_WINDOW_KEYS or per_block < 1 or longest < 2 * min_windows
+            or (len(whole) + 1) * per_block > places):
+        return plain, [], []
+
+    def shares_of(windows: int, size: int) -> int:
+        return 1 if windows <= size else min(PREFILL_MAX_SHARES, -(-windows // size))
+
+    def fits(size: int) -> bool:
+        return sum(shares_of(block[0], size) for block in whole) * per_block <= places
+
+    low, high = min_windows, longest  # whole blocks (size = longest) fit
+    while low < high:
+        size = (low + high) // 2
+        if fits(size):
+            high = size
+        else:
+            low = size + 1
+    size = low
+    if max(-(-block[0] // shares_of(block[0], size)) for block in whole) + combine_cost >= longest:
+        return plain, [], []
+    entries, combine, slot = [], [], 0
+    for windows, index, row, here in whole:
+        shares = shares_of(windows, size)
+        if shares == 1:
+            entries.append((windows, index, row, 0, 0, -1))
+            continue
+        each = -(-windows // shares)
+        shares = -(-windows // each)  # no empty share
+        combine.append([row, here, slot, shares])
+        for share in range(shares):
+            entries.append((min(each, windows - share * each), index, row, share * each, min(each, windows - share * each), slot))
+            slot += 1
+    entries.sort(key=lambda entry: -entry[0])
+    return [[e[1], e[2]] for e in entries], [[e[3], e[4], e[5]] for e in entries], combine
+
+
+@dataclass
+class PrefillWork:
+    """The work list of one prefill attention launch on the device (see :meth:`Ops.prefill_blocks`)."""
+
+    blocks: torch.Tensor                 # int32 [n, 2]: request index, first row
+    ranges: torch.Tensor | None = None   # int32 [n, 3]: first window, windows, slot; None: whole blocks only
+    combine: torch.Tensor | None = None  # int32 [c, 4]: first row, rows, first slot, shares
+    slots: int = 0
 
 
 class Ops:
@@ -449,14 +537,37 @@ class Ops:
         lib = load_module(build.attention_module(head_dim))
         return int(getattr(lib, f"ts_attention_prefill_rows_d{head_dim}")(heads, kv_heads))
 
-    def prefill_blocks(self, query_lens, context_lens, rows: int) -> torch.Tensor:
+    #: Fewest windows of 32 keys worth a workgroup of their own when a block's keys are shared out,
+    #: and what putting the shares together costs, in windows (see :func:`prefill_share_list`).
+    prefill_share_min_windows = 16
+    prefill_share_combine_cost = 20
+
+    def prefill_blocks(self, query_lens, context_lens, rows: int, *, heads: int = 0, kv_heads: int = 0,
+                       head_dim: int = 0, block_size: int = 0, window: int | None = None) -> PrefillWork:
         """The work list of :meth:`attention_prefill` for the multi-token requests at the front
-        of a step (their numbers of new tokens and their contexts after the step): int32
-        ``[n, 2]`` on the device, (request index, first row) of every block of ``rows`` rows
-        (:meth:`prefill_block_rows`), those that see the most keys first, so the long ones start
-        early and the short ones fill the tail of the launch."""
-        blocks = prefill_block_list(query_lens, context_lens, rows)
-        return torch.tensor(blocks, dtype=torch.int32).view(-1, 2).to(self.device)
+        of a step (their numbers of new tokens and their contexts after the step): (request
+        index, first row) of every block of ``rows`` rows (:meth:`prefill_block_rows`), those
+        that see the most keys first, so the long ones start early and the short ones fill the
+        tail of the launch.  Given the geometry (and the layer's window), the keys of long
+        blocks are shared out over several workgroups where whole blocks would leave compute
+        units idle (:func:`prefill_share_list`): a short portion at the end of a long context."""
+        ranges, combine = [], []
+        if heads and kv_heads and head_dim and block_size and rows == PREFILL_WINDOW_KEYS:
+            per_block, per_unit = c_int(0), c_int(0)
+            lib = load_module(build.attention_module(head_dim))
+            getattr(lib, f"ts_attention_prefill_shape_d{head_dim}")(heads, kv_heads, block_size, ctypes.byref(per_block),
+                                                                   ctypes.byref(per_unit))
+            blocks, ranges, combine = prefill_share_list(
+                query_lens, context_lens, rows, int(window or 0), per_block.value, per_unit.value * self.compute_units,
+                self.prefill_share_min_windows, combine_cost=self.prefill_share_combine_cost)
+        else:
+            blocks = prefill_block_list(query_lens, context_lens, rows)
+        work = PrefillWork(torch.tensor(blocks, dtype=torch.int32).view(-1, 2).to(self.device))
+        if ranges:
+            work.ranges = torch.tensor(ranges, dtype=torch.int32).view(-1, 3).to(self.device)
+            work.combine = torch.tensor(combine, dtype=torch.int32).view(-1, 4).to(self.device)
+            work.slots = sum(entry[3] for entry in combine)
+        return work
 
     def attention_prefill(
         self,
@@ -468,7 +579,7 @@ class Ops:
         block_table: torch.Tensor,
         query_start_loc: torch.Tensor,
         context_lens: torch.Tensor,
-        blocks: torch.Tensor,
+        blocks: "torch.Tensor | PrefillWork",
         heads: int,
         scale: float,
         window: int | None,
@@ -476,13 +587,18 @@ class Ops:
         block_rows: int = 16,
     ) -> None:
         """Matrix-core attention for blocks of ``block_rows`` consecutive rows of multi-token
-        requests (what :meth:`prefill_block_rows` says for the geometry): ``blocks [n, 2]`` holds
-        (request index, first row) of each; writes those rows of ``out [T, heads * D]``."""
-        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens, blocks)
+        requests (what :meth:`prefill_block_rows` says for the geometry): ``blocks`` is the work
+        list of :meth:`prefill_blocks` (made for this ``window``), or ``[n, 2]`` (request index,
+        first row) of whole blocks; writes those rows of ``out [T, heads * D]``."""
+        work = blocks if isinstance(blocks, PrefillWork) else PrefillWork(blocks)
+        blocks = work.blocks
+        _gpu(out, q, k_pages, v_pages, block_table, query_start_loc, context_lens, blocks, work.ranges, work.combine)
         _i32(block_table, "block_table")
         _i32(query_start_loc, "query_start_loc")
         _i32(context_lens, "context_lens")
         _i32(blocks, "blocks")
+        _i32(work.ranges, "ranges")
+        _i32(work.combine, "combine")
         _check_pages(k_pages, v_pages, torch.bfloat16)
         _, kv_heads, block_size, head_dim = k_pages.shape
         _need(self.mfma_attention_supported(q.dtype, head_dim, block_size), "geometry not taken by the matrix-core kernels")
@@ -494,11 +610,22 @@ class Ops:
         _need(max_context <= block_table.shape[1] * block_size, "block table does not cover the context")
         _need(block_rows == self.prefill_block_rows(head_dim, heads, kv_heads),
               f"blocks of {block_rows} rows are not what the kernel for this geometry takes")
+        partial_acc = partial_ml = None
+        num_combine = 0
+        if work.ranges is not None:
+            _need(block_rows == PREFILL_WINDOW_KEYS, "only blocks of 32 rows are shared out")
+            _need(tuple(work.ranges.shape) == (blocks.shape[0], 3), "ranges must be [n, 3] beside blocks [n, 2]")
+            _need(work.combine is not None and work.combine.dim() == 2 and work.combine.shape[1] == 4 and work.slots >= 1,
+                  "a work list with shares names the blocks to combine")
+            num_combine = work.combine.shape[0]
+            partial_acc = torch.empty((work.slots, heads, PREFILL_WINDOW_KEYS, head_dim), dtype=torch.float32, device=out.device)
+            partial_ml = torch.empty((work.slots, heads, PREFILL_WINDOW_KEYS, 2), dtype=torch.float32, device=out.device)
         lib = load_module(build.attention_module(head_dim))
         fn = getattr(lib, f"ts_attention_prefill_d{head_dim}")
         _check(fn(_ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                   block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), _ptr(blocks), blocks.shape[0],
                   block_rows, heads, kv_heads, block_size, float(scale), int(window or 0), int(max_context),
+                  _ptr(work.ranges), _ptr(partial_acc), _ptr(partial_ml), _ptr(work.combine), num_combine,
                   self.stream()),
                "ts_attention_prefill")
 

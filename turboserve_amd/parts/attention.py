@@ -120,8 +120,10 @@ class GroupedQueryAttention(Mixer):
             if ctx.num_prefill_seqs > 0:
                 # The launch's list of row blocks is the same for every layer with this geometry.
                 rows = ops.prefill_block_rows(self.head_dim, self.num_heads, self.num_kv_heads)
-                blocks = ctx.derive(("attention_prefill_blocks", rows), lambda step: ops.prefill_blocks(
-                    step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs], rows))
+                geometry = dict(heads=self.num_heads, kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+                                block_size=cache.block_size, window=self.window)
+                blocks = ctx.derive(("attention_prefill_blocks", rows, *geometry.values()), lambda step: ops.prefill_blocks(
+                    step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs], rows, **geometry))
                 ops.attention_prefill(
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len, rows,

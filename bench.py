@@ -25,7 +25,8 @@ TFLOP/s.
 Other runs: ``--shape 14b --batch 32 --mixed-prefill 2048`` (every step holds the decode tokens
 and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool of all the
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
-requests of 128..1,024 tokens in and 64..512 out, C in flight), ``--attention-prefill T[,CTX]`` (the
+requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
+few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
 prefill attention kernel alone), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """

@@ -216,11 +216,19 @@ def test_trace_run_program(case, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("trial", range(10))
-def test_random_configurations_replay_like_plain(trial, tmp_path):
+def test_random_configurations_replay_like_plain(trial, tmp_path, monkeypatch):
     """Seeded random configurations beyond the three fixed ones: head sizes that are and are not
     multiples of 16 or 32, one to sixteen query heads per KV head (every attention kernel variant),
-    page sizes 8 to 64, windows, tied and untied heads; mixed and portion-wise cutting, both dtypes."""
+    page sizes 8 to 64, windows, tied and untied heads; mixed and portion-wise cutting, both dtypes.
+    Every other trial shares out the keys of every attention block that has two windows of keys
+    or more (serving does so only for long contexts)."""
     import random
+
+    from turboserve_amd.kernels.ops import Ops
+
+    if trial % 2:
+        monkeypatch.setattr(Ops, "prefill_share_min_windows", 1)
+        monkeypatch.setattr(Ops, "prefill_share_combine_cost", 0)
 
     rng = random.Random(9000 + trial)
     kv_heads = rng.choice([1, 1, 2, 3, 4])

@@ -1453,8 +1453,11 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
 // The blocks whose keys were shared out: combine[4 c ..] = (first row, rows, first slot, shares)
 // of block c, whose shares lie in consecutive slots.  out = sum_s acc_s 2^(m_s - M) / sum_s l_s
 // 2^(m_s - M) with M the largest reference among the shares, as in decode_reduce_kernel.
-// grid (blocks to combine, heads), 256 threads: a thread takes four head dimensions of one row.
-constexpr int COMBINE_THREADS = 256;
+// grid (blocks to combine, heads, 4 groups of 8 rows); a thread takes four head dimensions of one
+// row and asks for all of its shares' sums before it adds any (the launch is short and lives on
+// how many loads are under way).
+constexpr int COMBINE_ROWS = 8;
+constexpr int COMBINE_THREADS = COMBINE_ROWS * (D / 4);
 constexpr int PREFILL_MAX_SHARES = 16;
 
 __global__ void __launch_bounds__(COMBINE_THREADS)
@@ -1463,34 +1466,41 @@ prefill_combine_kernel(uint16_t* __restrict__ out, const float* __restrict__ par
   const int row0 = combine[4 * blockIdx.x];
   const int rows = combine[4 * blockIdx.x + 1];
   const int first_slot = combine[4 * blockIdx.x + 2];
-  const int shares = combine[4 * blockIdx.x + 3];
+  const int shares = min(combine[4 * blockIdx.x + 3], PREFILL_MAX_SHARES);
   const int head = blockIdx.y;
-  for (int c = threadIdx.x; c < rows * (D / 4); c += COMBINE_THREADS) {
-    const int col = c / (D / 4);
-    const int d = 4 * (c % (D / 4));
-    float m[PREFILL_MAX_SHARES], l[PREFILL_MAX_SHARES];
-    f32x4 part[PREFILL_MAX_SHARES];
-    float m_max = -INFINITY;
+  const int col = COMBINE_ROWS * blockIdx.z + threadIdx.x / (D / 4);
+  const int d = 4 * (threadIdx.x % (D / 4));
+  if (col >= rows) return;
+  const size_t first = ((size_t)first_slot * heads + head) * WIDE_ROWS + col;
+  const size_t step = (size_t)heads * WIDE_ROWS;  // from a share's entry to the next share's
+  float m[PREFILL_MAX_SHARES], l[PREFILL_MAX_SHARES];
+  f32x4 part[PREFILL_MAX_SHARES];
 #pragma unroll
-    for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
-      const size_t entry = ((size_t)(first_slot + min(sh, shares - 1)) * heads + head) * WIDE_ROWS + col;
-      m[sh] = sh < shares ? partial_ml[entry * 2] : -INFINITY;
+  for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
+    m[sh] = -INFINITY;
+    l[sh] = 0.f;
+    part[sh] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (sh < shares) {
+      const size_t entry = first + sh * step;
+      m[sh] = partial_ml[entry * 2];
       l[sh] = partial_ml[entry * 2 + 1];
       part[sh] = *reinterpret_cast<const f32x4*>(partial_acc + entry * D + d);
-      m_max = fmaxf(m_max, m[sh]);
     }
-    float den = 0.f;
-    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
-      const float wgt = (m[sh] == -INFINITY) ? 0.f : exp2f(m[sh] - m_max);  // a share that saw nothing, or none
-      den += l[sh] * wgt;
-      sum += part[sh] * wgt;
-    }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
-    *reinterpret_cast<u32x2*>(out + ((size_t)(row0 + col) * heads + head) * D + d) =
-        Frag4{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
   }
+  float m_max = -INFINITY;
+#pragma unroll
+  for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) m_max = fmaxf(m_max, m[sh]);
+  float den = 0.f;
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int sh = 0; sh < PREFILL_MAX_SHARES; ++sh) {
+    const float wgt = (m[sh] == -INFINITY) ? 0.f : exp2f(m[sh] - m_max);  // a share that saw nothing, or none
+    den += l[sh] * wgt;
+    sum += part[sh] * wgt;
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  *reinterpret_cast<u32x2*>(out + ((size_t)(row0 + col) * heads + head) * D + d) =
+      Frag4{pack2(sum[0] * inv, sum[1] * inv), pack2(sum[2] * inv, sum[3] * inv)};
 }
 
 static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t* q, long q_stride,
@@ -1545,8 +1555,8 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
   }
   const int status = ts_launch_status();
   if (status != TS_OK || num_combine == 0) return status;
-  hipLaunchKernelGGL(prefill_combine_kernel, dim3(num_combine, heads), dim3(COMBINE_THREADS), 0, stream, out, partial_acc,
-                     partial_ml, combine, heads);
+  hipLaunchKernelGGL(prefill_combine_kernel, dim3(num_combine, heads, WIDE_ROWS / COMBINE_ROWS), dim3(COMBINE_THREADS), 0,
+                     stream, out, partial_acc, partial_ml, combine, heads);
   return ts_launch_status();
 }
 

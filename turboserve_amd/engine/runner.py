@@ -96,11 +96,13 @@ class ModelRunner:
     def dry_run(self, num_tokens: int) -> None:
         """One step of a made-up prompt of ``num_tokens`` tokens that writes nothing into the
         cache (every slot is the skip mark) and whose result is dropped: it makes every product
-        of the model run once at that size, for warming up or for timing the library's kernels."""
+        of the model run once at that size, for warming up or for timing the library's kernels
+        (the tokens differ from one another: products of equal rows draw less power and run
+        faster than those of a real prompt, and would be timed at clocks serving never sees)."""
         page = self.storage.page_size
         groups = len(self.layout.groups)
         entry = StepEntry(
-            request="dry-run", tokens=[0] * num_tokens, start=0,
+            request="dry-run", tokens=[(7919 * i + 13) % self.vocab_size for i in range(num_tokens)], start=0,
             tables=[[0] * (-(-num_tokens // page))] * groups, slots=[[-1] * num_tokens] * groups,
             state_slot=self.storage.pad_state_slot, want=[num_tokens - 1],
         )

@@ -157,7 +157,7 @@ class LLMEngine:
         sizes = {min(t, budget) for t in self.config.tune_gemm_tokens}
         if self.config.tune_gemm_step_sizes:
             ops = self.model.runtime.ops
-            ops.library_buckets = ops.bucket_sizes(budget)
+            ops.library_buckets = ops.bucket_sizes(budget)  # until close(): the model may outlive this engine
             sizes.update(size for size in ops.library_buckets if size > ops.skinny_max_rows)
         started = time.perf_counter()
         with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
@@ -455,6 +455,8 @@ class LLMEngine:
         self.storage = None
         if self.runner is not None and hasattr(self.runner, "release"):
             self.runner.release()
+        if self.config.tune_gemm_step_sizes and self.model is not None:
+            self.model.runtime.ops.library_buckets = ()
         if torch.cuda.is_available():
             torch.cuda.empty_cache()
 

@@ -246,6 +246,8 @@ class Ops:
         self.core = load_module("core")
         for module in modules:
             load_module(module)
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._tiled_plans: dict[tuple, tuple[int, int, int]] = {}  # (m, n, k, max_splits) -> grid of the tiled product
         #: Compute units of the device (256 on an MI355X): the launch plans below size their grids by it.
         self.compute_units = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
@@ -256,6 +258,9 @@ class Ops:
         self.skinny_resident_waves = 16 * self.compute_units
 
     def stream(self) -> int:
+        """The handle of torch's current stream on this device (what every launch goes to)."""
+        if self._raw_stream is not None:
+            return self._raw_stream(self._device_index)  # 0.06 us; the public way below takes 2 us, a step has 260 launches
         return torch.cuda.current_stream(self.device).cuda_stream
 
     # -- rows ---------------------------------------------------------------------------------

@@ -869,17 +869,30 @@ def test_truncation_helper_is_the_plain_rule():
 
 @pytest.mark.parametrize("vocab", [152064, 40001])
 def test_sampler_on_a_long_row_with_equal_logits(ops, vocab):
-    """A vocabulary of real size (rows that are and are not 16-byte aligned), smooth logits and
-    logits on a grid of 0.25 (thousands of equal values, keys whose low bits are zero): the token
-    lies in what the plain truncation keeps, and its cumulative interval holds the uniform number."""
+    """A vocabulary of real size (rows that are and are not 16-byte aligned), smooth logits,
+    logits on a grid of 0.25 (thousands of equal values, keys whose low bits are zero) and peaked
+    rows (the kernel's short way through a list of the likely tokens): the token lies in what the
+    plain truncation keeps, and its cumulative interval holds the uniform number."""
     from turboserve_amd.sampling.params import SamplingParams
 
     g = torch.Generator().manual_seed(vocab)
     settings = [dict(temperature=0.8), dict(temperature=0.8, top_k=50, top_p=0.9), dict(temperature=1.0, top_p=0.6),
                 dict(temperature=1.3, top_k=5), dict(temperature=0.7, top_k=2000, top_p=0.95), dict(temperature=1.0, top_p=0.05)]
-    rows = 2 * len(settings) * 2
+    group = 2 * len(settings)
+    rows = 5 * group
     logits = torch.randn(rows, vocab, generator=g) * 2.5
-    logits[rows // 2:] = torch.round(logits[rows // 2:] * 4) / 4
+    logits[group:2 * group] = torch.round(logits[group:2 * group] * 4) / 4
+    # Rows as a language model makes them, which the kernel's short way takes (few tokens far above
+    # the rest): thirty likely tokens all over the vocabulary; the same on a grid of 0.25 (equal
+    # logits among the likely ones); fifty likely tokens at the start of the vocabulary (one
+    # wavefront lists them all) with every logit negative.
+    for i in range(2 * group, 4 * group):
+        spots = torch.randperm(vocab, generator=g)[:30]
+        logits[i, spots] = torch.rand(30, generator=g) * 12 + 12
+    logits[3 * group:4 * group] = torch.round(logits[3 * group:4 * group] * 4) / 4
+    logits[4 * group:] = logits[4 * group:] - 40.0
+    logits[4 * group:, :50] += torch.rand(group, 50, generator=g) * 10 + 12
+    assert float(logits[4 * group:].max()) < 0
     params = [SamplingParams(**settings[i % len(settings)]) for i in range(rows)]
     seeds = [77 + i * 104729 for i in range(rows)]
     draws = [i for i in range(rows)]

@@ -228,12 +228,13 @@ extern "C" int ts_argmax_static(int* tokens, const float* logits, int rows, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// The sampling kernel proper.  A row of a large vocabulary is read a dozen times, so every
-// pass matters: rows are visited with 16-byte loads, several in flight per thread; the two
-// truncations pick their thresholds eight bits at a time from histograms in LDS (four passes
-// each instead of 32); the draw scans partial sums in parallel.  Everything is a function of
-// the row alone and is added up in a fixed order (histograms hold integers), so a row's token
-// does not depend on its neighbours or on the run.
+// The sampling kernel proper.  One workgroup works through a row of a large vocabulary, so every
+// walk over the row matters: rows are visited with 16-byte loads, several in flight per thread;
+// the two truncations pick their thresholds eight bits at a time from histograms in LDS, over
+// a list of the row's likely tokens where a truncation leaves few (four light walks over the
+// row), else over the row itself (four walks per truncation); the draw scans partial sums in
+// parallel.  Everything is a function of the row alone and is added up in a fixed order
+// (histograms hold integers), so a row's token does not depend on its neighbours or on the run.
 // ---------------------------------------------------------------------------------------------
 #define SAMPLE_WAVES (SAMPLE_THREADS / TS_WAVE)
 #define MASS_COPIES 4  // histograms of mass per workgroup (wavefront w adds to copy w % 4)

@@ -27,7 +27,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -101,6 +101,8 @@ def parse_args() -> argparse.Namespace:
                         "tokens, C of them live at a time; prints output tokens/s, time to first token and time between tokens")
     p.add_argument("--sampled", action="store_true",
                    help="with --closed-loop: temperature 0.7, top-p 0.8, top-k 20, repetition penalty 1.05 instead of greedy")
+    p.add_argument("--sample-kernel", type=int, default=0, metavar="ROWS",
+                   help="time the sampling kernel alone on ROWS rows of logits of the shape's vocabulary, and exit")
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
@@ -362,6 +364,47 @@ def run_attention_prefill(shape: dict, tokens: int, context: int, launches: int 
             "frac": round(flops / best / PEAK_FLOPS["bf16"], 4)}
 
 
+def run_sample_kernel(shape: dict, rows: int, launches: int = 20) -> dict:
+    """The sampling kernel alone on ``rows`` rows of logits of the shape's vocabulary, of a language
+    model's kind (N(0, 2.5) with thirty tokens at 12 to 24): microseconds a launch by device
+    events, the host's preparation of the launch included, for several settings."""
+    import torch
+
+    from turboserve_amd.kernels.ops import Ops
+    from turboserve_amd.sampling.params import SamplingParams
+    from turboserve_amd.sampling.sampler import Sampler
+
+    vocab = shape["vocab_size"]
+    sampler = Sampler(Ops("cuda:0"))
+    generator = torch.Generator(device="cuda").manual_seed(0)
+    logits = torch.randn(rows, vocab, device="cuda", generator=generator) * 2.5
+    spots = torch.randint(0, vocab, (rows, 30), device="cuda", generator=generator)
+    logits.scatter_(1, spots, torch.rand(rows, 30, device="cuda", generator=generator) * 12 + 12)
+    settings = {
+        "greedy": dict(temperature=0.0),
+        "temperature 0.8": dict(temperature=0.8),
+        "temperature 0.7, top-k 20, top-p 0.8": dict(temperature=0.7, top_k=20, top_p=0.8),
+        "the same with repetition penalty 1.05 over 800 tokens": dict(temperature=0.7, top_k=20, top_p=0.8, repetition_penalty=1.05),
+        "temperature 0.8, top-p 0.9": dict(temperature=0.8, top_p=0.9),
+        "temperature 0.8, top-k 50": dict(temperature=0.8, top_k=50),
+    }
+    histories = [list(range(100, 900)) for _ in range(rows)]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    result = {"kernel": "sampling", "rows": rows, "vocab": vocab, "us": {}}
+    for name, kwargs in settings.items():
+        params = [SamplingParams(**kwargs) for _ in range(rows)]
+        for _ in range(3):
+            sampler.launch(logits, params, list(range(rows)), [3] * rows, histories)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(launches):
+            sampler.launch(logits, params, list(range(rows)), [3] * rows, histories)
+        stop.record()
+        stop.synchronize()
+        result["us"][name] = round(start.elapsed_time(stop) / launches * 1e3, 1)
+    return result
+
+
 def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
     """Bytes a decode step has to read: every weight it uses once (all but the embedding
     table, of which it reads one row per request) and the cache of the live requests."""
@@ -389,6 +432,9 @@ def main() -> int:
         from turboserve_amd.profiling import format_shares, step_shares
 
         print(format_shares(step_shares(args.kernel_shares, steps=args.shares_steps)))
+        return 0
+    if args.sample_kernel:
+        print(json.dumps(run_sample_kernel(SHAPES[args.shape][1], args.sample_kernel)))
         return 0
     if args.attention_prefill:
         sizes = [int(v) for v in args.attention_prefill.split(",")]

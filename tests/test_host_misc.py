@@ -462,3 +462,33 @@ def test_prefill_work_list_shares_out_long_blocks():
     assert check([64, 64], [3000, 4000], 1024, 4, 256, min_windows=8)[1]
     check([5], [5], 0, 4, 256)
     check([], [], 0, 4, 256)
+
+
+def test_the_kept_token_array_follows_the_lists():
+    """``Sequence.token_array`` is ``token_ids`` at every moment: through appended tokens, places
+    taken for unread tokens and filled or dropped later, growth beyond what the array held, and a
+    reset for recomputation."""
+    import random
+
+    rng = random.Random(3)
+    seq = Sequence(seq_id=1, request_id="a", prompt_token_ids=[rng.randrange(1000) for _ in range(70)],
+                   sampling=SamplingParams(max_tokens=10_000))
+    assert seq.token_array().tolist() == seq.token_ids and seq.token_array().dtype == np.int32
+    pending = None
+    for turn in range(400):
+        action = rng.random()
+        if pending is not None and action < 0.6:
+            seq.set_unread_token(pending, rng.randrange(1000))
+            pending = None
+        elif pending is not None and action < 0.65:
+            seq.drop_unread_token(pending)
+            pending = None
+        elif pending is None and action < 0.8:
+            pending = seq.append_unread_token()
+        elif pending is None:
+            seq.append_token(rng.randrange(1000))
+        if turn % 3 == 0:  # not looked at every turn: several changes meet one call
+            assert seq.token_array().tolist() == seq.token_ids, turn
+        if turn == 250:
+            seq.reset_for_recompute()
+    assert seq.token_array().tolist() == seq.token_ids and seq.num_output_tokens > 100

@@ -110,11 +110,14 @@ class Sampler:
 
         want_logprobs = any(p.logprobs for p in params)
         history_start = [0]
-        flat_history: list[int] = []
+        pieces: list[np.ndarray] = []
         for i, p in enumerate(params):
+            held = history_start[-1]
             if p.repetition_penalty != 1.0 and histories is not None:
-                flat_history.extend(int(t) for t in histories[i])
-            history_start.append(len(flat_history))
+                pieces.append(np.asarray(histories[i], dtype=np.int32))  # no copy where it is an int32 array already
+                held += pieces[-1].shape[0]
+            history_start.append(held)
+        flat_history = np.concatenate(pieces) if pieces else np.empty(0, dtype=np.int32)
         floats = np.asarray(
             [[p.temperature for p in params], [p.top_p for p in params], [p.repetition_penalty for p in params]],
             dtype=np.float32,
@@ -128,7 +131,7 @@ class Sampler:
             np.asarray([int(d) & 0xFFFFFFFF for d in draw_indices], dtype=np.uint32).view(np.int32),
             np.asarray(history_start, dtype=np.int32),
             np.asarray(unread[1] if unread is not None else [-1] * rows, dtype=np.int32),
-            np.asarray(flat_history, dtype=np.int32),
+            flat_history,
         ])
         # One copy, from pinned memory and queued on the stream: a copy from pageable memory
         # would make the host wait for everything the stream holds, a step launched ahead included.
@@ -164,6 +167,6 @@ class Sampler:
             [seq.sampling for seq in sequences],
             [seq.sample_seed for seq in sequences],
             [seq.num_output_tokens for seq in sequences],
-            [seq.token_ids if seq.sampling.repetition_penalty != 1.0 else () for seq in sequences],
+            [seq.token_array() if seq.sampling.repetition_penalty != 1.0 else () for seq in sequences],
             unread,
         )

@@ -908,6 +908,37 @@ def test_sampler_on_a_long_row_with_equal_logits(ops, vocab):
         assert low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"row {i}: u={u} not in [{low}, {float(cdf[token])}]"
 
 
+def test_samplers_short_and_long_way_choose_alike(ops):
+    """The sampling kernel's short way (a list of the likely tokens) and its long way (the whole
+    row) use the same integer masses and comparisons: on thousands of peaked rows of every
+    truncation they choose the same token, but for a draw that falls within rounding of an
+    interval's end (the two add the same masses up in different orders)."""
+    from turboserve_amd.kernels.ops import Ops
+    from turboserve_amd.sampling.params import SamplingParams
+
+    long_way = Ops(DEV)
+    long_way.sample_max_listed = 0
+    g = torch.Generator().manual_seed(12)
+    settings = [dict(temperature=0.7, top_k=20, top_p=0.8), dict(temperature=1.0, top_k=50), dict(temperature=0.9, top_p=0.9),
+                dict(temperature=1.2, top_k=3, top_p=0.5), dict(temperature=0.8, top_k=400, top_p=0.95),
+                dict(temperature=0.6, top_p=0.3, repetition_penalty=1.3)]
+    differing = 0
+    for vocab, rows in ((5003, 3000), (152064, 96)):
+        logits = torch.randn(rows, vocab, generator=g) * 2.5
+        for i in range(rows):
+            spots = torch.randperm(vocab, generator=g)[:1 + i % 40]
+            logits[i, spots] = torch.rand(spots.numel(), generator=g) * 12 + 10
+        logits[::3] = torch.round(logits[::3] * 8) / 8  # equal logits among the likely ones
+        params = [SamplingParams(**settings[i % len(settings)]) for i in range(rows)]
+        seeds = [11 + 7919 * i for i in range(rows)]
+        draws = [i % 17 for i in range(rows)]
+        histories = [torch.randint(0, vocab, (30,), generator=g).tolist() for _ in range(rows)]
+        short = sample_rows(ops, logits, params, seeds, draws, histories).token_ids
+        long = sample_rows(long_way, logits, params, seeds, draws, histories).token_ids
+        differing += sum(a != b for a, b in zip(short, long))
+    assert differing <= 2, f"{differing} rows differ"
+
+
 def test_sampler_keeps_equal_logits_together(ops):
     """Five equal logits at the edge of top-k 3 are all kept (the plain rule: below the k-th
     largest is cut) and all drawn; a nucleus that ends inside a group of equal logits keeps the group."""

@@ -332,6 +332,8 @@ __device__ __forceinline__ void pick_digit_by_mass(const unsigned long long* tot
 // the host has not read yet (it was sampled by a launch still in flight) names that token's
 // place in `unread_tokens`, or -1; it counts as part of the row's history.
 // work [rows, vocab]: scratch for the penalised logits.  logprobs may be null.
+// max_listed: the most tokens the short way may list (at most SAMPLE_CANDIDATES; 0: every row
+// goes the long way).
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
               const float* __restrict__ logits, float* __restrict__ work, int vocab,
@@ -340,7 +342,7 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
               const uint32_t* __restrict__ seed_lo, const uint32_t* __restrict__ seed_hi,
               const uint32_t* __restrict__ draw_index, const int* __restrict__ history,
               const int* __restrict__ history_start, const int* __restrict__ unread_tokens,
-              const int* __restrict__ unread_row) {
+              const int* __restrict__ unread_row, int max_listed) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ unsigned long long lscratch[SAMPLE_WAVES];
@@ -502,9 +504,9 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
         __syncthreads();
         if (tid < 512) {
           if (use_k) {
-            if (above < (unsigned int)k && above + mine >= (unsigned int)k && above + mine <= SAMPLE_CANDIDATES)
+            if (above < (unsigned int)k && above + mine >= (unsigned int)k && above + mine <= (unsigned int)max_listed)
               picked[0] = (unsigned int)tid;  // one thread at most
-          } else if (above + mine <= SAMPLE_CANDIDATES) {
+          } else if (above + mine <= (unsigned int)max_listed) {
             atomicMin(&picked[0], (unsigned int)tid);
           }
         }
@@ -885,13 +887,14 @@ extern "C" int ts_sample(int* tokens, float* logprobs, const float* logits, floa
                          int vocab, const float* temperature, const int* top_k, const float* top_p,
                          const float* penalty, const uint32_t* seed_lo, const uint32_t* seed_hi,
                          const uint32_t* draw_index, const int* history, const int* history_start,
-                         const int* unread_tokens, const int* unread_row, hipStream_t stream) {
+                         const int* unread_tokens, const int* unread_row, int max_listed, hipStream_t stream) {
   if (rows == 0) return TS_OK;
   if (!tokens || !logits || !work || vocab < 1 || !temperature || !top_k || !top_p || !penalty ||
-      !seed_lo || !seed_hi || !draw_index || !history_start)
+      !seed_lo || !seed_hi || !draw_index || !history_start || max_listed < 0)
     return TS_ERR_ARG;
+  if (max_listed > SAMPLE_CANDIDATES) max_listed = SAMPLE_CANDIDATES;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, tokens, logprobs,
                      logits, work, vocab, temperature, top_k, top_p, penalty, seed_lo, seed_hi,
-                     draw_index, history, history_start, unread_tokens, unread_row);
+                     draw_index, history, history_start, unread_tokens, unread_row, max_listed);
   return ts_launch_status();
 }

@@ -59,7 +59,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                     c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     },
 }
 
@@ -943,6 +943,10 @@ class Ops:
                                    self.stream()), "ts_argmax")
         return tokens
 
+    #: Most tokens the sampling kernel lists for its short way through a truncated row (the kernel
+    #: holds 2,048); 0 sends every row the long way.
+    sample_max_listed = 2048
+
     def sample(
         self,
         logits: torch.Tensor,
@@ -988,5 +992,6 @@ class Ops:
         _check(self.core.ts_sample(_ptr(tokens), _ptr(logprobs), _ptr(logits), _ptr(work), rows, vocab,
                                    _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(penalty), _ptr(seed_lo),
                                    _ptr(seed_hi), _ptr(draw_index), _ptr(history), _ptr(history_start),
-                                   _ptr(unread_tokens), _ptr(unread_row), self.stream()), "ts_sample")
+                                   _ptr(unread_tokens), _ptr(unread_row), int(self.sample_max_listed), self.stream()),
+               "ts_sample")
         return tokens, logprobs

@@ -246,6 +246,12 @@ __device__ __forceinline__ unsigned long long mass_units(float x, float m, float
   return (unsigned long long)(expf((x - m) * inv_temp) * 4294967296.0f);
 }
 
+// A token's mass in the draw, e^x for x <= 0: the hardware's exponential (a few units in the last
+// place off, which moves a token's probability by a millionth of itself).  Every walk of a draw
+// uses this one function, so the sums a walk retraces come out the same.  (The thresholds' integer
+// masses above take the exact one: whether a token is kept must not hang on that millionth.)
+__device__ __forceinline__ float draw_mass(float x) { return __expf(x); }
+
 __device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* scratch) {
   const int lane = threadIdx.x & (TS_WAVE - 1);
   const int wave = threadIdx.x / TS_WAVE;
@@ -655,7 +661,7 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
           if (wave == 0) {
             auto lane_mass = [&](int slot) {
               const uint32_t key = listed_key(slot);
-              return (stands(slot) && key >= threshold) ? expf((key_value(key) - m) * inv_temp) : 0.f;
+              return (stands(slot) && key >= threshold) ? draw_mass((key_value(key) - m) * inv_temp) : 0.f;
             };
             auto inclusive = [&](float v) {
 #pragma unroll
@@ -795,7 +801,7 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
       for (int j = 0; j < 4; ++j) {
         const int i = at + j;
         const float v = i < vocab ? row[i] : -INFINITY;
-        e[j] = (i < vocab && ordered_key(v) >= threshold) ? expf((v - m) * inv_temp) : 0.f;
+        e[j] = (i < vocab && ordered_key(v) >= threshold) ? draw_mass((v - m) * inv_temp) : 0.f;
       }
     };
     auto wave_inclusive = [&](float v) {  // sum over lanes 0 .. lane, always by the same additions
@@ -812,7 +818,7 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
       float e[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        e[j] = (at + j < vocab && ordered_key(v[j]) >= threshold) ? expf((v[j] - m) * inv_temp) : 0.f;
+        e[j] = (at + j < vocab && ordered_key(v[j]) >= threshold) ? draw_mass((v[j] - m) * inv_temp) : 0.f;
       stretch += __shfl(wave_inclusive((e[0] + e[1]) + (e[2] + e[3])), TS_WAVE - 1, TS_WAVE);
     });
     if (lane == 0) wave_total[wave] = stretch;

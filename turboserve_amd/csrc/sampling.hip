@@ -466,7 +466,7 @@ sample_kernel(int* __restrict__ tokens, float* __restrict__ logprobs,
     // its largest logit; for a histogram, 16 bits of the key deep, of the tokens whose keys lie in
     // the largest logit's leading-digit class or the one below it (for positive logits: at least
     // a quarter of the largest), from which a bound L follows at or above which at least k and at
-    // most SAMPLE_CANDIDATES tokens lie; to count each wavefront's tokens at or above L; and to
+    // most max_listed tokens lie; to count each wavefront's tokens at or above L; and to
     // list them, in vocabulary order.  Thresholds, sums and the draw then walk that list in LDS.
     // The arithmetic is that of the long way below (the same integer masses and comparisons), so
     // both choose the same thresholds; where no such L exists or a nucleus reaches below it, the

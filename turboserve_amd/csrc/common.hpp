@@ -54,16 +54,35 @@ __device__ __forceinline__ float round_to(float v) {
   return to_float(from_float<T>(v));
 }
 
+// Sums and maxima over a wavefront by data-parallel moves between lanes (an instruction each;
+// the shuffles the compiler makes of __shfl_xor go through the LDS crossbar and cost six trips of
+// some hundred cycles).  Lanes meet in a fixed order: the four of a quad, the two quads of a
+// half row, the two halves of a row of 16, then the rows; every lane returns the result.
+template <int CONTROL, int ROW_MASK>
+__device__ __forceinline__ float lanes_moved(float keep, float v) {
+  // Lanes of rows outside ROW_MASK, and lanes whose source does not exist, get `keep`.
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v),
+                                                               CONTROL, ROW_MASK, 0xF, false));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = TS_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TS_WAVE);
-  return v;
+  v += lanes_moved<0xB1, 0xF>(0.f, v);   // quad_perm [1,0,3,2]
+  v += lanes_moved<0x4E, 0xF>(0.f, v);   // quad_perm [2,3,0,1]
+  v += lanes_moved<0x141, 0xF>(0.f, v);  // row_half_mirror
+  v += lanes_moved<0x140, 0xF>(0.f, v);  // row_mirror: every lane holds its row's sum
+  v += lanes_moved<0x142, 0xA>(0.f, v);  // row_bcast15 into rows 1 and 3
+  v += lanes_moved<0x143, 0xC>(0.f, v);  // row_bcast31 into rows 2 and 3: row 3 holds all
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), TS_WAVE - 1));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = TS_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, TS_WAVE));
-  return v;
+  v = fmaxf(v, lanes_moved<0xB1, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x4E, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x141, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x140, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x142, 0xA>(v, v));
+  v = fmaxf(v, lanes_moved<0x143, 0xC>(v, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), TS_WAVE - 1));
 }
 
 // Sum over a block of `blockDim.x` threads (a multiple of 64, at most 1024); `scratch` holds at

@@ -260,6 +260,50 @@ def test_random_configurations_replay_like_plain(trial, tmp_path, monkeypatch):
             check(got, expected, dtype_name, f"trial {trial} {config} page {page} {cut}")
 
 
+@pytest.mark.parametrize("trial", range(3))
+def test_long_requests_in_large_portions_replay_like_plain(trial, tmp_path, monkeypatch):
+    """Requests of hundreds to thousands of tokens in portions of up to 2,048 (and of two), on
+    narrow layers so that the plain implementation stays quick: the attention kernels' forms for
+    many keys (several blocks of rows per request, windows of a thousand keys, portions behind a
+    long context, decoding far into a request), which the tiny requests above never reach.  The
+    second trial shares out every block of four windows of keys or more."""
+    import random
+
+    from turboserve_amd.kernels.ops import Ops
+
+    rng = random.Random(7000 + trial)
+    if trial == 1:
+        monkeypatch.setattr(Ops, "prefill_share_min_windows", 4)
+        monkeypatch.setattr(Ops, "prefill_share_combine_cost", 0)
+    kv_heads, group = [(2, 7), (1, 8), (4, 5)][trial]
+    window = [None, 1025, 300][trial]
+    config = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": rng.choice([64, 96, 136]),
+        "num_hidden_layers": 2, "num_attention_heads": kv_heads * group, "num_key_value_heads": kv_heads,
+        "head_dim": [128, 64, 128][trial], "intermediate_size": rng.choice([64, 104]), "vocab_size": rng.choice([97, 256]),
+        "rope_theta": rng.choice([1e4, 1e6]), "rms_norm_eps": 1e-6, "tie_word_embeddings": trial == 1,
+        "use_sliding_window": window is not None, "max_position_embeddings": 8192,
+    }
+    if window is not None:
+        config["sliding_window"] = window
+        config["max_window_layers"] = trial - 1  # trial 2: one layer sees everything, one the window
+    page = [16, 32, 64][trial]
+    lengths = [[3300, 700, 150], [1900, 5000, 700], [150, 1900, 3300]][trial]
+    requests = {f"r{i}": tiny.random_tokens(config["vocab_size"], n, 500 + i) for i, n in enumerate(lengths)}
+    cuts = {
+        "portions": lambda reqs: th.portions(reqs, [512, 37, 1024, 2, 300, 2048]),
+        "mixed": lambda reqs: th.mixed(reqs, [256, 33, 700, 2, 1500], max_live=3, decode_tail=6),
+    }
+    for dtype_name, dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        folder = tiny.make_model_dir(tmp_path / dtype_name, config, trial, dtype, std=tiny.std_for(dtype, config["hidden_size"]))
+        raw, tensors = tiny.read_model_dir(folder)
+        expected = {rid: plain.forward_logits(raw, tensors, toks) for rid, toks in requests.items()}
+        for cut, make in cuts.items():
+            steps = make(requests)
+            got = th.collect(steps, run_trace(folder, dtype_name, page, steps), requests)
+            check(got, expected, dtype_name, f"long trial {trial} {config} page {page} {cut}")
+
+
 LAYER_SHAPES = {
     "7b": dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944, rms_norm_eps=1e-6),
     "14b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=13824, rms_norm_eps=1e-5),

@@ -111,6 +111,12 @@ def test_sliding_window_is_described_not_rejected():
     assert [every.layer_window(layer) for layer in range(2)] == [8, 8]
     with pytest.raises(UnsupportedModelError, match="sliding_window"):
         Qwen2Config.from_dict({**QWEN2_RAW, "use_sliding_window": True, "sliding_window": "wide"})
+    windowed = {**QWEN2_RAW, "use_sliding_window": True, "sliding_window": 8}
+    assert Qwen2Config.from_dict({**windowed, "max_window_layers": None}).max_window_layers == 0
+    with pytest.raises(UnsupportedModelError, match="max_window_layers.*non-negative"):
+        Qwen2Config.from_dict({**windowed, "max_window_layers": -1})
+    with pytest.raises(UnsupportedModelError, match="max_window_layers.*must be an int"):
+        Qwen2Config.from_dict({**windowed, "max_window_layers": "2"})
 
 
 def test_kv_bytes_and_round_trip(tmp_path):

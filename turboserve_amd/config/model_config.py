@@ -26,85 +26,146 @@ class UnsupportedModelError(ValueError):
     """
 
 
-#: Storage dtypes a checkpoint may declare (model_config.py:58-67).  Only bfloat16 and
+# ---------------------------------------------------------------------------------------------
+# The schema: which key of config.json fills which field, what kind of value it must be and
+# what stands in when the file has none.  ``from_dict`` and ``to_hf_dict`` both walk it.
+# ---------------------------------------------------------------------------------------------
+
+REQUIRED = object()  # a key without a default
+
+
+@dataclass(frozen=True)
+class Key:
+    """One plain key of ``config.json``.
+
+    ``kind``: ``"count"`` (an int of at least ``least``; a bool or a string is refused),
+    ``"flag"``, ``"real"``, ``"text"`` or ``"id"`` (an optional token id, kept as found).
+    ``default`` may name another key's field (a ``str`` starting with ``=``): the value read
+    for that field stands in."""
+
+    field: str
+    kind: str
+    default: Any = REQUIRED
+    least: int = 1
+
+    def read(self, data: Mapping[str, Any], so_far: Mapping[str, Any]) -> Any:
+        raw = data.get(self.field)
+        if raw is None or (self.kind == "count" and self.least == 0 and not raw):
+            if self.default is REQUIRED:
+                raise UnsupportedModelError(f"config.json is missing the required field {self.field!r}")
+            if isinstance(self.default, str) and self.default.startswith("="):
+                return so_far[self.default[1:]]
+            return self.default
+        if self.kind == "count":
+            if isinstance(raw, bool) or not isinstance(raw, int):
+                raise UnsupportedModelError(f"config.json field {self.field!r} must be an int, got {raw!r}")
+            if raw < self.least:
+                bound = "positive" if self.least == 1 else "a non-negative int"
+                raise UnsupportedModelError(f"config.json field {self.field!r} must be {bound}, got {raw}")
+            return raw
+        return {"flag": bool, "real": float, "text": str, "id": lambda v: v}[self.kind](raw)
+
+
+#: Read in this order (a default may point back at an earlier field).  Defaults and the
+#: messages of ``Key.read`` are the reference's (model_config.py:79-87, 278, 300-313).
+PLAIN_KEYS: tuple[Key, ...] = (
+    Key("model_type", "text", "qwen2"),
+    Key("hidden_size", "count"),
+    Key("num_hidden_layers", "count"),
+    Key("num_attention_heads", "count"),
+    Key("num_key_value_heads", "count", "=num_attention_heads"),
+    Key("intermediate_size", "count"),
+    Key("vocab_size", "count"),
+    Key("hidden_act", "text", "silu"),
+    Key("rms_norm_eps", "real", 1e-6),
+    Key("max_position_embeddings", "count", 2048),
+    Key("tie_word_embeddings", "flag", False),
+    Key("mlp_bias", "flag", False),
+    Key("max_window_layers", "count", 0, least=0),
+    Key("bos_token_id", "id", None),
+    Key("pad_token_id", "id", None),
+)
+
+#: Names a checkpoint may give its storage type (model_config.py:58-67).  Only bfloat16 and
 #: float32 can be *run*; the others are recognised so the error can say so.
 CHECKPOINT_DTYPES: dict[str, torch.dtype] = {
-    "float16": torch.float16,
-    "fp16": torch.float16,
-    "half": torch.float16,
-    "bfloat16": torch.bfloat16,
-    "bf16": torch.bfloat16,
-    "float32": torch.float32,
-    "fp32": torch.float32,
-    "float": torch.float32,
+    **dict.fromkeys(("float16", "fp16", "half"), torch.float16),
+    **dict.fromkeys(("bfloat16", "bf16"), torch.bfloat16),
+    **dict.fromkeys(("float32", "fp32", "float"), torch.float32),
 }
 
 ROPE_TYPES = ("default", "linear")
 
 
-def require_int(data: Mapping[str, Any], key: str, *, default: int | None = None) -> int:
-    """A positive int field; absent, non-int and non-positive each get their own message
-    (model_config.py:79-87)."""
-    value = data.get(key, default)
-    if value is None:
-        raise UnsupportedModelError(f"config.json is missing the required field {key!r}")
-    if isinstance(value, bool) or not isinstance(value, int):
-        raise UnsupportedModelError(f"config.json field {key!r} must be an int, got {value!r}")
-    if value < 1:
-        raise UnsupportedModelError(f"config.json field {key!r} must be positive, got {value}")
-    return value
+# Keys that need more than one lookup each get a function: config.json -> {field: value}.
 
 
-def rope_settings(data: Mapping[str, Any]) -> tuple[float, float]:
-    """``(theta, position divisor)`` from the flat (``rope_theta``/``rope_scaling``) or the
-    nested (``rope_parameters``) spelling (model_config.py:90-123)."""
-    block = data.get("rope_parameters")
-    if not isinstance(block, Mapping):
-        merged: dict[str, Any] = {}
+def _head_dim(data: Mapping[str, Any], so_far: Mapping[str, Any]) -> dict[str, Any]:
+    """``head_dim`` if the file has one, else ``hidden_size // heads`` (model_config.py:279-282)."""
+    given = data.get("head_dim")
+    head_dim = int(given) if given else so_far["hidden_size"] // so_far["num_attention_heads"]
+    if head_dim < 1:
+        raise UnsupportedModelError(f"head_dim resolved to {head_dim}")
+    return {"head_dim": head_dim}
+
+
+def _rope(data: Mapping[str, Any], so_far: Mapping[str, Any]) -> dict[str, Any]:
+    """Base and position divisor, from the nested spelling (``rope_parameters``) or the flat
+    one (``rope_theta`` beside ``rope_scaling``) (model_config.py:90-123)."""
+    nested = data.get("rope_parameters")
+    if isinstance(nested, Mapping):
+        settings = dict(nested)
+    else:
+        scaling = data.get("rope_scaling")
+        settings = dict(scaling) if isinstance(scaling, Mapping) else {}
         if "rope_theta" in data:
-            merged["rope_theta"] = data["rope_theta"]
-        if isinstance(data.get("rope_scaling"), Mapping):
-            merged.update(data["rope_scaling"])
-        block = merged
-    theta = float(block.get("rope_theta", 10000.0))
-    if theta <= 0:
-        raise UnsupportedModelError(f"rope_theta must be positive, got {theta}")
-    kind = str(block.get("rope_type") or block.get("type") or "default")
-    if kind not in ROPE_TYPES:
-        raise UnsupportedModelError(
-            f"rope_type {kind!r} is not implemented; supported: {list(ROPE_TYPES)}"
-        )
-    factor = float(block.get("factor", 1.0)) if kind == "linear" else 1.0
-    if factor <= 0:
-        raise UnsupportedModelError(f"rope scaling factor must be positive, got {factor}")
-    return theta, factor
+            settings["rope_theta"] = data["rope_theta"]
+    theta = float(settings.get("rope_theta", 10000.0))
+    kind = str(settings.get("rope_type") or settings.get("type") or "default")
+    factor = float(settings.get("factor", 1.0)) if kind == "linear" else 1.0
+    for ok, message in (
+        (theta > 0, f"rope_theta must be positive, got {theta}"),
+        (kind in ROPE_TYPES, f"rope_type {kind!r} is not implemented; supported: {list(ROPE_TYPES)}"),
+        (factor > 0, f"rope scaling factor must be positive, got {factor}"),
+    ):
+        if not ok:
+            raise UnsupportedModelError(message)
+    return {"rope_theta": theta, "rope_scaling_factor": factor}
 
 
-def checkpoint_dtype(data: Mapping[str, Any]) -> torch.dtype | None:
-    """``dtype`` (newer) or ``torch_dtype`` (older) of the checkpoint (model_config.py:126-137)."""
-    raw = data.get("dtype", data.get("torch_dtype"))
-    if raw is None:
-        return None
-    if isinstance(raw, torch.dtype):
-        return raw
-    name = str(raw).removeprefix("torch.")
-    if name not in CHECKPOINT_DTYPES:
-        raise UnsupportedModelError(f"unknown checkpoint dtype {raw!r}")
-    return CHECKPOINT_DTYPES[name]
+def _window(data: Mapping[str, Any], so_far: Mapping[str, Any]) -> dict[str, Any]:
+    """Sliding-window attention is on when the file says so *and* names a window."""
+    window = data.get("sliding_window")
+    if window is not None and (isinstance(window, bool) or not isinstance(window, int)):
+        raise UnsupportedModelError(f"config.json field 'sliding_window' must be an int, got {window!r}")
+    return {"use_sliding_window": bool(data.get("use_sliding_window", False)) and bool(window),
+            "sliding_window": window or None}
 
 
-def eos_ids(data: Mapping[str, Any]) -> tuple[int, ...]:
-    """``eos_token_id`` as a tuple, whether the file holds one id or a list (model_config.py:140-149)."""
-    raw = data.get("eos_token_id")
-    if raw is None:
-        return ()
-    if isinstance(raw, bool):
-        raise UnsupportedModelError(f"unsupported eos_token_id {raw!r}")
-    if isinstance(raw, int):
-        return (raw,)
-    if isinstance(raw, (list, tuple)):
-        return tuple(int(t) for t in raw)
-    raise UnsupportedModelError(f"unsupported eos_token_id {raw!r}")
+def _storage_dtype(data: Mapping[str, Any], so_far: Mapping[str, Any]) -> dict[str, Any]:
+    """``dtype`` (newer files) or ``torch_dtype`` (older) (model_config.py:126-137)."""
+    named = data.get("dtype", data.get("torch_dtype"))
+    if named is None or isinstance(named, torch.dtype):
+        return {"torch_dtype": named}
+    found = CHECKPOINT_DTYPES.get(str(named).removeprefix("torch."))
+    if found is None:
+        raise UnsupportedModelError(f"unknown checkpoint dtype {named!r}")
+    return {"torch_dtype": found}
+
+
+def _end_tokens(data: Mapping[str, Any], so_far: Mapping[str, Any]) -> dict[str, Any]:
+    """``eos_token_id`` holds one id or a list of them (model_config.py:140-149)."""
+    named = data.get("eos_token_id")
+    if named is None:
+        return {"eos_token_ids": ()}
+    if isinstance(named, int) and not isinstance(named, bool):
+        return {"eos_token_ids": (named,)}
+    if isinstance(named, (list, tuple)):
+        return {"eos_token_ids": tuple(int(t) for t in named)}
+    raise UnsupportedModelError(f"unsupported eos_token_id {named!r}")
+
+
+COMPOSITE_KEYS = (_head_dim, _rope, _window, _storage_dtype, _end_tokens)
 
 
 @dataclass(frozen=True)
@@ -205,95 +266,38 @@ class Qwen2Config:
 
     def to_hf_dict(self) -> dict[str, Any]:
         """A ``config.json`` mapping that parses back to this configuration."""
-        data: dict[str, Any] = {
-            "architectures": [self.architecture],
-            "model_type": self.model_type,
-            "hidden_size": self.hidden_size,
-            "num_hidden_layers": self.num_hidden_layers,
-            "num_attention_heads": self.num_attention_heads,
-            "num_key_value_heads": self.num_key_value_heads,
-            "head_dim": self.head_dim,
-            "intermediate_size": self.intermediate_size,
-            "vocab_size": self.vocab_size,
-            "hidden_act": self.hidden_act,
-            "rms_norm_eps": self.rms_norm_eps,
-            "rope_theta": self.rope_theta,
-            "max_position_embeddings": self.max_position_embeddings,
-            "tie_word_embeddings": self.tie_word_embeddings,
-            "use_sliding_window": self.use_sliding_window,
-            "sliding_window": self.sliding_window,
-            "max_window_layers": self.max_window_layers,
-        }
+        data: dict[str, Any] = {"architectures": [self.architecture]}
+        for key in PLAIN_KEYS:
+            value = getattr(self, key.field)
+            if value is not None and key.field != "mlp_bias":
+                data[key.field] = value
+        data.update(head_dim=self.head_dim, rope_theta=self.rope_theta, use_sliding_window=self.use_sliding_window,
+                    sliding_window=self.sliding_window)
         if self.rope_scaling_factor != 1.0:
             data["rope_scaling"] = {"rope_type": "linear", "factor": self.rope_scaling_factor}
         if self.torch_dtype is not None:
             data["torch_dtype"] = str(self.torch_dtype).removeprefix("torch.")
         if self.eos_token_ids:
             data["eos_token_id"] = list(self.eos_token_ids)
-        if self.bos_token_id is not None:
-            data["bos_token_id"] = self.bos_token_id
-        if self.pad_token_id is not None:
-            data["pad_token_id"] = self.pad_token_id
         return data
 
     # -- construction -----------------------------------------------------------------------
 
     @classmethod
     def from_dict(cls, data: Mapping[str, Any], *, name_or_path: str = "") -> "Qwen2Config":
-        """Parse a ``config.json`` mapping (model_config.py:254-314)."""
-        architectures = data.get("architectures") or []
-        architecture = str(architectures[0]) if architectures else ""
-        if architecture != cls.ARCHITECTURE:
-            raise UnsupportedModelError(
-                f"architecture {architecture or '<missing>'!r} is not a {cls.ARCHITECTURE}"
-            )
-        hidden_size = require_int(data, "hidden_size")
-        heads = require_int(data, "num_attention_heads")
-        kv_heads = require_int(data, "num_key_value_heads", default=heads)
-        raw_head_dim = data.get("head_dim")
-        head_dim = int(raw_head_dim) if raw_head_dim else hidden_size // heads
-        if head_dim < 1:
-            raise UnsupportedModelError(f"head_dim resolved to {head_dim}")
-        theta, factor = rope_settings(data)
-        use_window = bool(data.get("use_sliding_window", False)) and bool(data.get("sliding_window"))
-        window = data.get("sliding_window")
-        if window is not None and (isinstance(window, bool) or not isinstance(window, int)):
-            raise UnsupportedModelError(f"config.json field 'sliding_window' must be an int, got {window!r}")
-        max_window_layers = data.get("max_window_layers", 0) or 0
-        if isinstance(max_window_layers, bool) or not isinstance(max_window_layers, int) or max_window_layers < 0:
-            raise UnsupportedModelError(
-                f"config.json field 'max_window_layers' must be a non-negative int, got {max_window_layers!r}"
-            )
-        return cls(
-            architecture=architecture,
-            model_type=str(data.get("model_type") or "qwen2"),
-            hidden_size=hidden_size,
-            num_hidden_layers=require_int(data, "num_hidden_layers"),
-            num_attention_heads=heads,
-            num_key_value_heads=kv_heads,
-            head_dim=head_dim,
-            intermediate_size=require_int(data, "intermediate_size"),
-            vocab_size=require_int(data, "vocab_size"),
-            hidden_act=str(data.get("hidden_act", "silu")),
-            rms_norm_eps=float(data.get("rms_norm_eps", 1e-6)),
-            rope_theta=theta,
-            rope_scaling_factor=factor,
-            max_position_embeddings=require_int(data, "max_position_embeddings", default=2048),
-            tie_word_embeddings=bool(data.get("tie_word_embeddings", False)),
-            # Qwen2's q/k/v bias is part of the architecture; o_proj never has one
-            # (model_config.py:285-288).
-            qkv_bias=True,
-            o_proj_bias=False,
-            mlp_bias=bool(data.get("mlp_bias", False)),
-            use_sliding_window=use_window,
-            sliding_window=int(window) if window else None,
-            max_window_layers=int(max_window_layers),
-            torch_dtype=checkpoint_dtype(data),
-            eos_token_ids=eos_ids(data),
-            bos_token_id=data.get("bos_token_id"),
-            pad_token_id=data.get("pad_token_id"),
-            name_or_path=name_or_path,
-        )
+        """Parse a ``config.json`` mapping by the schema above (the reference's counterpart:
+        model_config.py:254-314)."""
+        named = data.get("architectures") or [""]
+        if str(named[0]) != cls.ARCHITECTURE:
+            raise UnsupportedModelError(f"architecture {str(named[0]) or '<missing>'!r} is not a {cls.ARCHITECTURE}")
+        values: dict[str, Any] = {}
+        for key in PLAIN_KEYS:
+            values[key.field] = key.read(data, values)
+        for composite in COMPOSITE_KEYS:
+            values.update(composite(data, values))
+        # Qwen2's q/k/v bias is part of the architecture, whatever ``attention_bias`` says; the
+        # output projection never has one (model_config.py:285-288).
+        return cls(architecture=cls.ARCHITECTURE, qkv_bias=True, o_proj_bias=False, name_or_path=name_or_path, **values)
 
     @classmethod
     def from_hf(cls, model_dir: str | Path) -> "Qwen2Config":

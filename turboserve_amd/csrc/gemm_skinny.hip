@@ -6,7 +6,7 @@
 // SwiGLU, or nobody when splits == 1) adds the splits up, so no rounding happens between the
 // product and its consumer.  (gemm_tiled.hip holds the product for up to 64 rows; this one
 // serves small matrices, whose product lasts a few microseconds and gains from many small
-// workgroups that start quickly, and the widest matrices at up to four rows.)
+// workgroups that start quickly, and the widest matrices at up to eight rows.)
 //
 // The product is bound by reading W once from HBM.  Layout of the work:
 //   * a workgroup of 4 or 8 wavefronts owns 64 or 128 consecutive weight rows (16 per

@@ -57,7 +57,9 @@ __device__ __forceinline__ float round_to(float v) {
 // Sums and maxima over a wavefront by data-parallel moves between lanes (an instruction each;
 // the shuffles the compiler makes of __shfl_xor go through the LDS crossbar and cost six trips of
 // some hundred cycles).  Lanes meet in a fixed order: the four of a quad, the two quads of a
-// half row, the two halves of a row of 16, then the rows; every lane returns the result.
+// half row, the two halves of a row of 16, then the rows; every lane returns the result.  All 64
+// lanes must be active at the call (a lane that is switched off contributes nothing, where a
+// shuffle would still read its register): call them from code the whole wavefront runs.
 template <int CONTROL, int ROW_MASK>
 __device__ __forceinline__ float lanes_moved(float keep, float v) {
   // Lanes of rows outside ROW_MASK, and lanes whose source does not exist, get `keep`.

@@ -86,7 +86,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--no-gemm-tuning", action="store_true",
                    help="leave the choice of the BLAS library's prefill kernels to its heuristic")
-    p.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling)")
+    p.add_argument("--only-prefill", nargs="?", type=int, const=PREFILL_TOKENS, default=None, metavar="TOKENS",
+                   help="run the prefill of one prompt alone (for profiling): 2,048 tokens, or TOKENS")
     p.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (the default run is 7b)")
     p.add_argument("--fill-hbm", action="store_true", help="size the cache pool to the free device memory")
     p.add_argument("--mixed-prefill", type=int, default=0, metavar="N",
@@ -470,8 +471,10 @@ def main() -> int:
         print(json.dumps(record))
         return 0
     if args.only_prefill:
-        seconds = run_prefill(model, config, PREFILL_TOKENS, tune=tune)
-        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}))
+        seconds = run_prefill(model, config, args.only_prefill, tune=tune)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": args.only_prefill, "layers": layers,
+                          "tokens_per_s": round(args.only_prefill / seconds, 1),
+                          "frac": round(prefill_flops(config, layers, args.only_prefill) / seconds / PEAK_FLOPS[dtype_key], 4)}))
         return 0
 
     main_run = run_decode(model, config, args.batch, args.context - 1, steps=args.steps, warmup=args.warmup,

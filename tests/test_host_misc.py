@@ -462,6 +462,19 @@ def test_prefill_work_list_shares_out_long_blocks():
     assert check([64, 64], [3000, 4000], 1024, 4, 256, min_windows=8)[1]
     check([5], [5], 0, 4, 256)
     check([], [], 0, 4, 256)
+    # the same invariants on seeded random steps: any mix of portions, contexts, windows, grids
+    import random
+
+    rng = random.Random(5)
+    shared_out = 0
+    for _ in range(400):
+        requests = rng.randint(1, 5)
+        query_lens = [rng.choice([1, 2, 31, 32, 33, 64, 100, 300, 700]) for _ in range(requests)]
+        context_lens = [q + rng.choice([0, 0, 5, 200, 3000, 20000]) for q in query_lens]
+        _, ranges, _ = check(query_lens, context_lens, rng.choice([0, 0, 33, 500, 4096]), rng.choice([1, 2, 4, 8, 16]),
+                             rng.choice([64, 256, 512]), min_windows=rng.choice([1, 4, 16]))
+        shared_out += bool(ranges)
+    assert shared_out > 40
 
 
 def test_the_kept_token_array_follows_the_lists():

@@ -7,7 +7,9 @@
 // The product is bound by reading W once from HBM, and what decides its rate is how the reading
 // is spread over the device, not how much of it is in flight:
 //   * a workgroup of four wavefronts (2 x 2) owns a tile of NT = 32 TN weight rows (TN = 2, 4
-//     or 5) by all activation rows (64 of them, or 128 when M > 64) and one range of K; the host
+//     or 5) by all activation rows (32 of them, 64 when M > 32, 128 when M > 64: rows beyond M
+//     are repeats that cost loads and LDS writes, so the tile is no larger than it must be) and
+//     one range of K; the host
 //     sizes tiles and ranges so that
 //     the grid is about one workgroup per compute unit (two for the smallest tile): every
 //     compute unit then streams one contiguous block of each of its rows, start to end;
@@ -19,7 +21,7 @@
 //     beyond the range repeat its last one), so the compiler can count the loads in flight and
 //     waits only for those it needs; pieces beyond K are cleared on their way into LDS;
 //   * a wavefront computes TN x MB tiles of v_mfma_f32_16x16x32_bf16 (A = 16 weight rows, B = 16
-//     activation rows; MB = 2, or 4 for M > 64): each weight fragment it reads from LDS serves MB
+//     activation rows; MB = 1, 2 or 4): each weight fragment it reads from LDS serves MB
 //     products, each activation fragment TN.
 #include "common.hpp"
 
@@ -221,6 +223,8 @@ int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x
 template <int TN>
 int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
                  const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+  if (m <= 32)
+    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
   if (m <= 64)
     return launch_tiled_rows<TN, 2>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
   return launch_tiled_rows<TN, 4>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);

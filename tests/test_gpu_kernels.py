@@ -154,7 +154,8 @@ def test_gemm_skinny(ops, m, n, k):
 
 
 @pytest.mark.parametrize("tile", [2, 4, 5])
-@pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (40, 64, 40), (128, 330, 520), (77, 1000, 264)])
+@pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (16, 200, 392), (17, 333, 264), (32, 96, 1096), (40, 64, 40),
+                                   (128, 330, 520), (77, 1000, 264)])
 def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
     """The tiled product with its grid given by hand: every tile size, ranges of K of one
     iteration and of several, a last range that is shorter, a last tile of rows that is partly
@@ -173,7 +174,8 @@ def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
 
 
 @pytest.mark.parametrize("tile", [2, 4, 5])
-@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (33, 1000, 40), (128, 250, 264), (90, 81, 128)])
+@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (16, 81, 392), (24, 250, 264), (33, 1000, 40), (128, 250, 264),
+                                       (90, 81, 128)])
 def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
     """A gate|up matrix with alternating rows through the tiled product with the activation in
     its epilogue gives, bit for bit, what the product's partial sums followed by the SwiGLU

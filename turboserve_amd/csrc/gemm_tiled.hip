@@ -7,7 +7,7 @@
 // The product is bound by reading W once from HBM, and what decides its rate is how the reading
 // is spread over the device, not how much of it is in flight:
 //   * a workgroup of four wavefronts (2 x 2) owns a tile of NT = 32 TN weight rows (TN = 2, 4
-//     or 5) by all activation rows (32 of them, 64 when M > 32, 128 when M > 64: rows beyond M
+//     or 5) by all activation rows (16 of them, 32 when M > 16, 64 when M > 32, 128 when M > 64: rows beyond M
 //     are repeats that cost loads and LDS writes, so the tile is no larger than it must be) and
 //     one range of K; the host
 //     sizes tiles and ranges so that
@@ -39,23 +39,27 @@ constexpr int ROW_PIECES = DEPTH / 8; // 16-byte pieces of a row of an iteration
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <int TN, int MB>
+// XROWS: activation rows of a workgroup's tile, 32 MB (each half of the wavefronts takes 16 MB of
+// them), or 16 with MB = 1: then both halves read the same 16 rows, the second half's products
+// are duplicates that nobody stores, and half as much is fetched and staged.
+template <int TN, int XROWS>
 struct TileRegs {
   static constexpr int W_PIECES = 32 * TN * ROW_PIECES / THREADS;  // 2 TN
-  static constexpr int X_PIECES = 32 * MB * ROW_PIECES / THREADS;  // 2 MB
+  static constexpr int X_PIECES = XROWS * ROW_PIECES / THREADS;    // XROWS / 16
   u32x4 w[W_PIECES];
   u32x4 x[X_PIECES];
 };
 
-template <int TN, int MB>
+template <int TN, int MB, int XROWS>
 __global__ void __launch_bounds__(THREADS)
 gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, const uint16_t* __restrict__ x,
                   long x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n,
                   int k, int iters_per_split) {
   constexpr int NT = 32 * TN;
-  constexpr int M_TILE = 32 * MB;
-  constexpr int STAGE = (NT + M_TILE) * LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
-  typedef TileRegs<TN, MB> Regs;
+  static_assert(XROWS == 32 * MB || (XROWS == 16 && MB == 1), "a tile of 32 MB activation rows, or of 16");
+  constexpr bool SHARED_ROWS = XROWS == 16;  // both halves of the wavefronts work on the same 16 rows
+  constexpr int STAGE = (NT + XROWS) * LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
+  typedef TileRegs<TN, XROWS> Regs;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [2][STAGE]
   const int tid = threadIdx.x;
   const int lane = tid & (TS_WAVE - 1);
@@ -126,7 +130,7 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
       u32x4 xf[MB];
 #pragma unroll
       for (int b = 0; b < MB; ++b)
-        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 16 * MB * wave_m + 16 * b) * LDS_ROW + 32 * step);
+        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + (SHARED_ROWS ? 0 : 16 * MB * wave_m) + 16 * b) * LDS_ROW + 32 * step);
 #pragma unroll
       for (int a = 0; a < TN; ++a) {
         const u32x4 wf = *reinterpret_cast<const u32x4*>(base + (wave_n * TN + a) * 16 * LDS_ROW + 32 * step);
@@ -154,7 +158,8 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
   }
 
   // acc[a][b][i] = sum for weight row n_base + 16 (wave_n TN + a) + 4 g + i and activation row
-  // 16 MB wave_m + 16 b + lane16.
+  // 16 MB wave_m + 16 b + lane16 (with shared rows: row lane16, stored by the first half only).
+  if (SHARED_ROWS && wave_m != 0) return;
 #pragma unroll
   for (int a = 0; a < TN; ++a) {
     const int nrow = n_base + (wave_n * TN + a) * 16 + 4 * group;
@@ -167,7 +172,7 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
     }
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      const int row = 16 * MB * wave_m + 16 * b + lane16;
+      const int row = (SHARED_ROWS ? 0 : 16 * MB * wave_m) + 16 * b + lane16;
       if (row >= m) continue;
       if (gated) {
         // The matrix is a gate|up projection with rows alternating gate, up (one range of K, no
@@ -198,24 +203,24 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
   }
 }
 
-template <int TN, int MB>
+template <int TN, int MB, int XROWS = 32 * MB>
 int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
                       const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits,
                       hipStream_t stream) {
   constexpr int NT = 32 * TN;
-  constexpr size_t lds_bytes = (size_t)2 * (NT + 32 * MB) * LDS_ROW * sizeof(uint16_t);
+  constexpr size_t lds_bytes = (size_t)2 * (NT + XROWS) * LDS_ROW * sizeof(uint16_t);
   static_assert(lds_bytes <= 160 * 1024, "two buffers must fit the LDS of a compute unit");
   if (lds_bytes > 48 * 1024) {
     static bool raised = false;  // per process; the attribute belongs to the kernel
     if (!raised) {
-      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN, MB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+      if (hipFuncSetAttribute((const void*)gemm_tiled_kernel<TN, MB, XROWS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)lds_bytes) != hipSuccess)
         return TS_ERR_LAUNCH;
       raised = true;
     }
   }
   dim3 grid((n + NT - 1) / NT, splits);
-  hipLaunchKernelGGL((gemm_tiled_kernel<TN, MB>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride,
+  hipLaunchKernelGGL((gemm_tiled_kernel<TN, MB, XROWS>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride,
                      w, bias, m, n, k, iters_per_split);
   return ts_launch_status();
 }
@@ -223,6 +228,8 @@ int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x
 template <int TN>
 int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
                  const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+  if (m <= 16)
+    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
   if (m <= 32)
     return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
   if (m <= 64)

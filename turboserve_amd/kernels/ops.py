@@ -251,9 +251,13 @@ class Ops:
         self._tiled_plans: dict[tuple, tuple[int, int, int]] = {}  # (m, n, k, max_splits) -> grid of the tiled product
         #: Compute units of the device (256 on an MI355X): the launch plans below size their grids by it.
         self.compute_units = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
-        #: Wavefronts a decode attention launch aims for: one per SIMD, four SIMDs a compute unit
-        #: (each keeps two windows of loads in flight).
-        self.decode_target_waves = 4 * self.compute_units
+        #: Wavefronts a decode attention launch aims for (each keeps two windows of loads in
+        #: flight): two per compute unit while the step has few requests x KV heads, one per SIMD
+        #: from half as many of those as there are compute units.  Measured through the engine at
+        #: the 7B shape (4 KV heads), context 8,192, two per unit against four: 3.78 against 3.83
+        #: ms a step with 4 requests, 4.11 against 4.15 with 8, 4.19 against 4.23 with 16 (context
+        #: 4,096), 6.27 against 6.28 with 32, 9.43 against 9.29 with 64.
+        self.decode_target_waves = (2 * self.compute_units, 4 * self.compute_units)
         #: Wavefronts (16 weight rows x one range of K each) the resident product aims for: 16 per compute unit.
         self.skinny_resident_waves = 16 * self.compute_units
 
@@ -524,7 +528,8 @@ class Ops:
         span = max_context if not window else min(max_context, window + 31)
         head_tiles = -(-(heads // kv_heads) // 16)
         pairs = requests * kv_heads * head_tiles
-        splits = max(1, min(-(-self.decode_target_waves // pairs), -(-span // self.decode_min_keys), 256))
+        waves = self.decode_target_waves[0 if 2 * pairs <= self.compute_units else 1]
+        splits = max(1, min(-(-waves // pairs), -(-span // self.decode_min_keys), 256))
         keys_per_split = -(-(-(-(span + 31) // splits)) // 32) * 32
         splits = -(-(span + 31) // keys_per_split)
         partial_acc = torch.empty((requests * heads * splits, head_dim), dtype=torch.float32, device=q.device)

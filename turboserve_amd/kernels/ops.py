@@ -701,12 +701,9 @@ class Ops:
     #: the resident-activation kernel, which is a little faster there; everything else up to 128
     #: rows runs the tiled kernel.
     resident_wide_rows = 8
-    #: Matrices smaller than this many bytes stay with the resident kernel up to eight rows: the
-    #: product lasts a few microseconds and the resident kernel's many small workgroups start
-    #: faster (7B shape, q|k|v and output projection, steps of 1 / 8 / 16 rows: 3.53 / 4.09 / 4.83 ms
-    #: against 3.56 / 4.10 / 4.81 with the tiled kernel and its tile of 16 activation rows).
+    #: Matrices smaller than this many bytes stay with the resident kernel up to 16 rows: the product
+    #: lasts a few microseconds and the resident kernel's many small workgroups start faster.
     resident_small_bytes = 64 << 20
-    resident_small_rows = 8
 
     def _tiled_plan(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int]:
         """(iterations of 128 per split, splits, tile) of the tiled product: the cheapest by
@@ -826,9 +823,9 @@ class Ops:
 
     def _resident_runs(self, m: int, n: int, k: int) -> bool:
         """Whether the resident kernel, not the tiled one, runs a decode-sized product: small
-        matrices and the widest ones, both up to eight rows (the head of the 7B shape at eight rows:
+        matrices up to 16 rows, the widest ones up to eight (the head of the 7B shape at eight rows:
         189 against 197 us)."""
-        if m <= self.resident_small_rows and 2 * n * k < self.resident_small_bytes:
+        if m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes:
             return True
         return m <= self.resident_wide_rows and -(-n // 160) >= 200
 

@@ -639,9 +639,8 @@ class Ops:
                   self.stream()),
                "ts_attention_prefill")
 
-    #: Fewest keys worth a wavefront of its own: one window (a step of one request at 640 tokens
-    #: of context, 7B shape: 3.45 ms against 3.50 with 128 and 3.54 with 256).
-    decode_min_keys = 32
+    #: Fewest keys worth a wavefront of its own.
+    decode_min_keys = 128
 
     # -- products -----------------------------------------------------------------------------
 

@@ -254,7 +254,7 @@ def test_recorded_steps_survive_the_growth_of_the_rotary_tables(tmp_path):
         assert torch.equal(results[False][step], results[True][step]), f"step {step}: recorded differs from eager"
 
 
-def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
+def test_timed_library_products_and_the_dry_step(model, tmp_path):
     """An engine asked to time the BLAS library's kernels at start-up: the choices are written
     to the given file, nothing is timed once the engine serves, products below the size worth
     timing keep the library's default kernel, and the dry step the timing runs in leaves every
@@ -290,16 +290,28 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path, monkeypatch):
     sequence = prompt + out.new_token_ids
     logits = plain.forward_logits(model["bf16_raw"], model["bf16_tensors"], sequence)
     check_logprobs(logits[len(prompt) - 1:], out)
-    # With the size limit lifted the same start-up times them and keeps its choices.
-    monkeypatch.setattr(Ops, "library_tuning_min_work", 0)
+    # A product of a size worth timing (and of a regular shape: the library's candidates for
+    # small odd shapes are not all sound) is timed inside the block, its choice is written to the
+    # file and stays in use afterwards.
+    from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
+
+    ops = Ops("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(256, 1024, generator=g).bfloat16().to("cuda:0")
+    w = (torch.randn(1024, 1024, generator=g) / 32).bfloat16().to("cuda:0")
+    assert x.shape[0] * w.shape[0] * w.shape[1] >= Ops.library_tuning_min_work
     results = tmp_path / "choices.csv"
-    engine = engine_with_tuning(results)
     try:
+        with LibraryGemmTuning(str(results), max_ms_per_candidate=5, max_iterations=5):
+            timed = ops.linear(x, w)
         assert results.exists() and "Gemm" in results.read_text()
-        assert not torch.cuda.tunable.tuning_is_enabled()
+        assert torch.cuda.tunable.is_enabled() and not torch.cuda.tunable.tuning_is_enabled()
+        again = ops.linear(x, w)
     finally:
-        engine.close()
         torch.cuda.tunable.enable(False)
+    want = x.float() @ w.float().t()
+    for got in (timed, again):
+        torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
 
 
 def test_library_products_at_timed_step_sizes(model, tmp_path):

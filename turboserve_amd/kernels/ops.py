@@ -875,9 +875,11 @@ class Ops:
         return x.as_strided((rows, x.shape[1]), (x.shape[1], 1))
 
     #: Products with fewer multiply-adds than this never use a timed choice of the BLAS library's
-    #: kernels, only its default: timing them is noise, and one of the library's candidates for
-    #: such a shape ([200, 64] x [256, 64]) returned garbage once in about eight processes.
-    library_tuning_min_work = 1 << 24
+    #: kernels, only its default: timing them is noise, and the library's candidates for small,
+    #: odd shapes are the ones that have misbehaved here (one for [200, 64] x [256, 64] returned
+    #: garbage once in about eight processes).  The smallest product an engine times for the 7B
+    #: shape, 160 rows of the output projection, has fifteen times as many.
+    library_tuning_min_work = 1 << 27
 
     def _library_product(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
                          out_dtype: torch.dtype | None) -> torch.Tensor:

@@ -3,6 +3,8 @@ whatever the token budget and however few pages there are; sampling follows the 
 
 from __future__ import annotations
 
+import itertools
+
 import pytest
 import torch
 
@@ -254,6 +256,9 @@ def test_recorded_steps_survive_the_growth_of_the_rotary_tables(tmp_path):
         assert torch.equal(results[False][step], results[True][step]), f"step {step}: recorded differs from eager"
 
 
+_TIMED_WIDTHS = itertools.count()
+
+
 def test_timed_library_products_and_the_dry_step(model, tmp_path):
     """An engine asked to time the BLAS library's kernels at start-up: the choices are written
     to the given file, nothing is timed once the engine serves, products below the size worth
@@ -297,8 +302,11 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
 
     ops = Ops("cuda:0")
     g = torch.Generator().manual_seed(3)
+    # A width of its own for every run of this test: a shape that was timed before in this process
+    # is not timed again, and nothing would be written.
+    width = 1024 + 128 * next(_TIMED_WIDTHS)
     x = torch.randn(256, 1024, generator=g).bfloat16().to("cuda:0")
-    w = (torch.randn(1024, 1024, generator=g) / 32).bfloat16().to("cuda:0")
+    w = (torch.randn(width, 1024, generator=g) / 32).bfloat16().to("cuda:0")
     assert x.shape[0] * w.shape[0] * w.shape[1] >= Ops.library_tuning_min_work
     results = tmp_path / "choices.csv"
     try:

@@ -1,0 +1,159 @@
+"""Host models of the addresses two kernels form, checked against their buffers' bounds.
+
+A wild address on the GPU can end more than the test that made it, so the index arithmetic of
+the two kernels whose launches the host plans most freely is restated here in Python and swept
+over shapes, plans and cache states on the CPU: the tiled product (``csrc/gemm_tiled.hip``:
+what a thread fetches, where it stages it in LDS, which fragments a wavefront reads, where the
+sums go) and the decode attention (``csrc/attention_mfma.hip``, ``decode_kernel``: which page and
+key every lane reads for every split, with pages given back below a window and table entries
+that are padding).  The models follow the kernels line by line and must be changed with them.
+"""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+DEPTH, LDS_ROW, THREADS, ROW_PIECES = 128, 136, 256, 16  # gemm_tiled.hip's constants
+
+
+def tiled_tile(m: int) -> tuple[int, int]:
+    """(MB, activation rows of the tile) that ``launch_tiled`` picks for ``m`` rows."""
+    if m <= 16:
+        return 1, 16
+    if m <= 32:
+        return 1, 32
+    return (2, 64) if m <= 64 else (4, 128)
+
+
+def check_tiled(m, n, k, tile, per_split, splits, gated, x_stride):
+    mb, xrows = tiled_tile(m)
+    nt = 32 * tile
+    stage = (nt + xrows) * LDS_ROW
+    w_pieces, x_pieces = nt * ROW_PIECES // THREADS, xrows * ROW_PIECES // THREADS
+    assert w_pieces * THREADS == nt * ROW_PIECES and x_pieces * THREADS == xrows * ROW_PIECES
+    x_size = (m - 1) * x_stride + k
+    total = -(-k // DEPTH)
+    shared = xrows == 16
+    blocks = -(-n // nt)
+    for bx in sorted({0, blocks // 2, blocks - 1}):
+        n_base = bx * nt
+        for split in sorted({0, splits - 1}):
+            first = split * per_split
+            last = min(first + per_split, total)
+            if first >= last:
+                continue
+            for tid in range(THREADS):
+                piece_k, piece_row = 8 * (tid % ROW_PIECES), tid // ROW_PIECES
+                for it in sorted({first, last - 1, last, last + 1}):  # the loop fetches two iterations past the range
+                    k0 = min(min(it, last - 1) * DEPTH + piece_k, k - 8)
+                    assert k0 >= 0
+                    for i in range(w_pieces):
+                        at = min(n_base + piece_row + 16 * i, n - 1) * k + k0
+                        assert 0 <= at and at + 8 <= n * k
+                    for i in range(x_pieces):
+                        at = min(piece_row + 16 * i, m - 1) * x_stride + k0
+                        assert 0 <= at and at + 8 <= x_size
+                dst = piece_row * LDS_ROW + piece_k
+                for buf in (0, 1):
+                    assert all(buf * stage + dst + (nt + 16 * i) * LDS_ROW + 8 <= (buf + 1) * stage for i in range(x_pieces))
+                    assert all(buf * stage + dst + 16 * i * LDS_ROW + 8 <= buf * stage + nt * LDS_ROW for i in range(w_pieces))
+                lane, wave = tid % 64, tid // 64
+                lane16, group, wave_n, wave_m = lane % 16, lane // 16, wave >> 1, wave & 1
+                base = lane16 * LDS_ROW + 8 * group
+                for step in range(DEPTH // 32):
+                    for b in range(mb):
+                        assert base + (nt + (0 if shared else 16 * mb * wave_m) + 16 * b) * LDS_ROW + 32 * step + 8 <= stage
+                    for a in range(tile):
+                        assert base + (wave_n * tile + a) * 16 * LDS_ROW + 32 * step + 8 <= nt * LDS_ROW
+                if shared and wave_m:
+                    continue
+                for a in range(tile):
+                    nrow = n_base + (wave_n * tile + a) * 16 + 4 * group
+                    if nrow >= n:
+                        continue
+                    for b in range(mb):
+                        row = (0 if shared else 16 * mb * wave_m) + 16 * b + lane16
+                        if row >= m:
+                            continue
+                        if gated:
+                            width = 2 if nrow + 3 < n else (1 if nrow + 1 < n else 0)
+                            assert row * (n // 2) + nrow // 2 + width <= m * (n // 2)
+                        else:
+                            width = 4 if (nrow + 3 < n and n % 4 == 0) else min(4, n - nrow)
+                            assert (split * m + row) * n + nrow + width <= splits * m * n
+
+
+@pytest.mark.parametrize("m", [1, 9, 16, 17, 32, 33, 64, 65, 128])
+def test_tiled_product_stays_inside_its_buffers(m):
+    rng = random.Random(m)
+    for n, k in ((97, 72), (5003, 200), (160, 48), (48, 40), (64, 264), (161, 128), (256, 1096), (6, 16)):
+        iters = -(-k // DEPTH)
+        for tile in (2, 4, 5):
+            for want in sorted({1, 2, iters}):
+                per_split = -(-iters // min(want, iters))
+                splits = -(-iters // per_split)
+                check_tiled(m, n, k, tile, per_split, splits, False, k + 8 * rng.randint(0, 3))
+                if splits == 1 and n % 2 == 0:
+                    check_tiled(m, n, k, tile, per_split, splits, True, k)
+
+
+WINDOW_KEYS = 32  # attention_mfma.hip
+
+
+def check_decode(ctx, window, shift, table, splits, keys_per_split, device_context=None):
+    """Every page a lane of ``decode_kernel`` selects is a live one, and the splits cover the
+    keys lo..ctx-1 exactly."""
+    if device_context is not None:  # a recorded launch sizes the splits on the device
+        span = device_context
+        if window and span > window + WINDOW_KEYS - 1:
+            span = window + WINDOW_KEYS - 1
+        per = (span + WINDOW_KEYS - 1 + splits - 1) // splits
+        keys_per_split = -(-per // WINDOW_KEYS) * WINDOW_KEYS
+    p = ctx - 1
+    lo = max(0, p - window + 1) if window else 0
+    covered = set()
+    for split in range(splits):
+        begin = (lo & ~31) + split * keys_per_split
+        end = min(begin + keys_per_split, ctx)
+        for w in range(begin, end, WINDOW_KEYS):
+            first = w >> shift
+            pages = [table[min(first + i, len(table) - 1)] for i in range(4)]
+            for lane16 in range(16):
+                for t in range(2):
+                    key = w + 8 * (lane16 >> 2) + 4 * t + (lane16 & 3)
+                    live = min(max(key, max(w, lo)), min(w + 31, p))
+                    assert pages[(live - w) >> shift] >= 0, (ctx, window, 1 << shift, split, w, key)
+                    if lo <= key <= p:
+                        assert key not in covered
+                        covered.add(key)
+            for group in range(4):
+                chunk = w + 8 * group
+                live = chunk + 7 >= lo and chunk <= p
+                key = chunk if live else (min(max(chunk, max(w, lo)), min(w + 31, p)) & ~7)
+                assert pages[(key - w) >> shift] >= 0, (ctx, window, 1 << shift, split, w, chunk)
+    assert covered == set(range(lo, ctx)), (ctx, window, splits, keys_per_split)
+
+
+def test_decode_attention_reads_live_pages_only():
+    rng = random.Random(2)
+    for _ in range(3000):
+        shift = rng.choice([3, 4, 5, 6])
+        page = 1 << shift
+        ctx = rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 100, 257, 600, 1000, rng.randint(1, 5000)])
+        window = rng.choice([0, 0, 1, 12, 16, 33, 70, 300, 1025])
+        needed = -(-ctx // page)
+        width = needed + rng.choice([0, 1, 5])
+        table = [rng.randint(0, 500) for _ in range(needed)] + [-1] * (width - needed)
+        if window:  # pages wholly below the window's lower bound were given back
+            for i in range(max(0, ctx - window) // page):
+                table[i] = -1
+        bound = rng.choice([ctx, min(ctx + 50, width * page), width * page])  # what the host knows of the longest context
+        span = bound if not window else min(bound, window + 31)
+        for splits_wanted in (1, 2, rng.randint(1, 64), 256):
+            splits = max(1, min(splits_wanted, -(-span // 32)))
+            keys_per_split = -(-(-(-(span + 31) // splits)) // 32) * 32
+            splits = -(-(span + 31) // keys_per_split)
+            check_decode(ctx, window, shift, table, splits, keys_per_split)
+            check_decode(ctx, window, shift, table, splits, keys_per_split, device_context=ctx)

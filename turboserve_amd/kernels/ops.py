@@ -257,7 +257,8 @@ class Ops:
         #: the 7B shape (4 KV heads), context 8,192, two per unit against four: 3.78 against 3.83
         #: ms a step with 4 requests, 4.11 against 4.15 with 8, 4.19 against 4.23 with 16 (context
         #: 4,096), 6.27 against 6.28 with 32, 9.43 against 9.29 with 64.
-        self.decode_target_waves = (2 * self.compute_units, 4 * self.compute_units)
+        self.decode_waves_few_pairs = 2 * self.compute_units
+        self.decode_waves_many_pairs = 4 * self.compute_units
         #: Wavefronts (16 weight rows x one range of K each) the resident product aims for: 16 per compute unit.
         self.skinny_resident_waves = 16 * self.compute_units
 
@@ -528,7 +529,7 @@ class Ops:
         span = max_context if not window else min(max_context, window + 31)
         head_tiles = -(-(heads // kv_heads) // 16)
         pairs = requests * kv_heads * head_tiles
-        waves = self.decode_target_waves[0 if 2 * pairs <= self.compute_units else 1]
+        waves = self.decode_waves_few_pairs if 2 * pairs <= self.compute_units else self.decode_waves_many_pairs
         splits = max(1, min(-(-waves // pairs), -(-span // self.decode_min_keys), 256))
         keys_per_split = -(-(-(-(span + 31) // splits)) // 32) * 32
         splits = -(-(span + 31) // keys_per_split)

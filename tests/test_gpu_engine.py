@@ -25,12 +25,12 @@ def make_engine(folder, dtype, page, *, num_blocks, budget=2048, max_num_seqs=8,
     ))
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def model(request, tmp_path_factory):
     config, seed, page = tiny.TINY[request.param]
     folder = tiny.make_model_dir(tmp_path_factory.mktemp(f"engine{request.param}"), config, seed, torch.float32)
     raw, tensors = tiny.read_model_dir(folder)
-    lengths = [5, 17, 33] if request.param == "A" else [1, 9, 24, 40]
+    lengths = {"A": [5, 17, 33], "B": [1, 9, 24, 40], "C": [20, 50, 97], "D": [2, 31, 52, 20]}[request.param]
     prompts = [tiny.random_tokens(config["vocab_size"], n, 50 + n) for n in lengths]
     # The same architecture with a wider spread of weights, for the 32-bit token-for-token tests:
     # its greedy continuations do not settle on one token, so every step's logits matter.
@@ -68,7 +68,7 @@ def test_greedy_generation_equals_plain(model):
     new = 8 if model["name"] == "A" else 12
     want = [plain.greedy_generate(model["wide_raw"], model["wide_tensors"], p, new) for p in model["prompts"]]
     assert all(len(set(tokens)) > 2 for tokens in want), "the continuations should not repeat one token"
-    for budget, blocks in ((2048, 64), (16, 64), (7 if model["page"] <= 7 else model["page"], 64)):
+    for budget, blocks in ((2048, 64), (max(16, model["page"]), 64), (7 if model["page"] <= 7 else model["page"], 64)):
         with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=blocks, budget=budget) as engine:
             outputs = engine.generate(model["prompts"], SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
             assert [o.new_token_ids for o in outputs] == want, f"budget {budget}"
@@ -108,7 +108,7 @@ def test_temperature_sampling_follows_the_rule(model):
     new = 12
     params = [SamplingParams(max_tokens=new, temperature=0.8, seed=1000 + i, ignore_eos=True, logprobs=True)
               for i in range(len(model["prompts"]))]
-    with make_engine(model["folder"], "float32", model["page"], num_blocks=64, budget=7 if model["page"] <= 7 else 16) as engine:
+    with make_engine(model["folder"], "float32", model["page"], num_blocks=64, budget=7 if model["page"] <= 7 else max(16, model["page"])) as engine:
         outputs = engine.generate(model["prompts"], params)
     for i, (prompt, output) in enumerate(zip(model["prompts"], outputs)):
         tokens = list(prompt)
@@ -449,6 +449,54 @@ def test_truncated_and_penalised_sampling_through_the_engine(model):
                 low = float(cdf[token - 1]) if token > 0 else 0.0
                 assert cdf.numel() and low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"request {i} draw {draw}: {token} != {want}"
             tokens.append(token)
+
+
+def test_a_penalised_request_that_stops_while_a_step_is_in_flight(model):
+    """Steps launched ahead with a repetition penalty: the sampler counts the token that only the
+    device knows yet into the history, and a request that hits a stop token while the next step
+    is already in flight drops that step's result.  Tokens equal those of the loop that reads
+    every step before it schedules the next, and the plain sampler's."""
+    from turboserve_amd.sampling.params import SamplingParams
+
+    new = 14
+    prompts = model["prompts"]
+
+    def params(stops):
+        return [SamplingParams(max_tokens=new, temperature=0.0 if i % 2 else 0.9, seed=400 + i, ignore_eos=True,
+                               repetition_penalty=1.6, stop_token_ids=stops.get(i, ()))
+                for i in range(len(prompts))]
+
+    with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=64) as engine:
+        free = [o.new_token_ids for o in engine.generate(prompts, params({}))]
+    for i, (prompt, produced) in enumerate(zip(prompts, free)):  # the plain sampler's tokens, with the history
+        tokens = list(prompt)
+        for draw, token in enumerate(produced):
+            logits = plain.forward_logits(model["wide_raw"], model["wide_tensors"], tokens)[-1]
+            want, cdf = plain.sample_token(logits, temperature=0.0 if i % 2 else 0.9, seed=400 + i, draw_index=draw,
+                                           penalty=1.6, history=tokens)
+            if token != want:
+                u = plain.philox_uniform(400 + i, draw)
+                low = float(cdf[token - 1]) if token > 0 else 0.0
+                assert cdf.numel() and low - 1e-5 <= u <= float(cdf[token]) + 1e-5, f"request {i} draw {draw}: {token} != {want}"
+            tokens.append(token)
+    # request 0 stops at its 6th token, the last request at its 9th: each while later steps are in flight
+    stops = {0: (free[0][5],), len(prompts) - 1: (free[-1][8],)}
+    results = []
+    for ahead in (False, True):
+        with make_engine(model["wide_folder"], "float32", model["page"], num_blocks=64, run_ahead=ahead) as engine:
+            outputs = engine.generate(prompts, params(stops))
+            results.append([(o.new_token_ids, o.finish_reason) for o in outputs])
+            if ahead:
+                assert engine.runner.graphs.num_replays > 0
+            engine.scheduler.check_invariants()
+            assert all(pool.num_in_use == 0 for pool in engine.scheduler.cache.pools)
+    assert results[0] == results[1]
+    for i, (tokens, reason) in enumerate(results[1]):
+        if i in stops:
+            cut = free[i].index(stops[i][0]) + 1
+            assert tokens == free[i][:cut] and reason == "stop"
+        else:
+            assert tokens == free[i] and reason == "length"
 
 
 def test_prompts_are_not_cut_when_chunking_is_off(model):

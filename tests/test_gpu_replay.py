@@ -34,13 +34,19 @@ ATOL_F32_CUTS = 1e-5
 #: one layer's cache exceeds these bounds more than tenfold.  Measured on these models: up to
 #: 1.6% (``tiny.BF16_STD`` has the figures, also for the reference's own formulas in bfloat16).
 RTOL_BF16 = 2e-2
+#: The same for steps of more than 128 rows, whose projections the BLAS library computes: it
+#: rounds the q|k|v and gate|up projections to bfloat16 where this engine's own products hand
+#: 32-bit sums to their consumers, so such a step carries more rounding: 140 short requests as
+#: one step are off by up to 2.3% where each alone is off by up to 1.7% (mean 0.6%), and the
+#: reference's own formulas in bfloat16 by up to 2.8%.  A fault moves the logits by 24% or more.
+RTOL_BF16_LIBRARY = 3e-2
 
 
 def lengths_for(name: str) -> list[int]:
-    return {"A": [5, 17, 33, 70, 50], "B": [1, 9, 24, 40, 75, 66], "C": [3, 45, 97, 130, 64]}[name]
+    return {"A": [5, 17, 33, 70, 50], "B": [1, 9, 24, 40, 75, 66], "C": [3, 45, 97, 130, 64], "D": [2, 31, 80, 49, 112]}[name]
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def case(request, tmp_path_factory):
     name = request.param
     config, seed, page = tiny.TINY[name]
@@ -69,19 +75,20 @@ def run_trace(folder: Path, dtype: str, page: int, steps: list[dict], max_tokens
     return outputs
 
 
-def excess(got: torch.Tensor, want: torch.Tensor, dtype: str) -> torch.Tensor:
+def excess(got: torch.Tensor, want: torch.Tensor, dtype: str, rtol_bf16: float = RTOL_BF16) -> torch.Tensor:
     """Per position: the largest |difference| of its logits divided by the bound for that
     position (above 1: out of bounds).  32-bit: ``ATOL_F32`` times the size of the logits where
-    that is above 1; bfloat16: ``RTOL_BF16`` times the position's largest |logit|."""
+    that is above 1; bfloat16: ``rtol_bf16`` times the position's largest |logit|."""
     diff = (got - want).abs().max(dim=1).values
     scale = want.abs().max(dim=1).values
-    bound = ATOL_F32 * scale.clamp(min=1.0) if dtype == "float32" else RTOL_BF16 * scale
+    bound = ATOL_F32 * scale.clamp(min=1.0) if dtype == "float32" else rtol_bf16 * scale
     return diff / bound
 
 
-def check(got: dict[str, torch.Tensor], expected: dict[str, torch.Tensor], dtype: str, what: str) -> None:
+def check(got: dict[str, torch.Tensor], expected: dict[str, torch.Tensor], dtype: str, what: str,
+          rtol_bf16: float = RTOL_BF16) -> None:
     for rid, want in expected.items():
-        ratio = excess(got[rid], want, dtype)
+        ratio = excess(got[rid], want, dtype, rtol_bf16)
         if float(ratio.max()) > 1.0:
             row = int(ratio.argmax())
             first = int((ratio > 1.0).nonzero()[0])
@@ -185,6 +192,51 @@ def test_a_fault_in_the_last_layers_cache_is_seen(case, dtype):
     assert worst["swapped"] > 5.0, f"swapped values in the last layer move the logits by only {worst['swapped']:.2f} times the bound"
     if replayer.storage.layout.groups[group].window is None:
         assert worst["swapped with keys"] <= 1.0, "the order of a request's pages should not matter when keys and values move together"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_portions_beside_more_single_tokens_than_a_recorded_step_takes(case, dtype):
+    """Steps that hold 140 single tokens and portions of two prompts: a two-token portion, one
+    that ends just past a page's edge, one that starts just before one.  More rows than a
+    recorded step or the decode products take, so the decode attention runs without the
+    device-side longest context beside the prefill attention, and the bfloat16 projections are
+    the library's."""
+    page = case["page"]
+    vocab = tiny.TINY[case["name"]][0]["vocab_size"]
+    many = {f"d{i}": tiny.random_tokens(vocab, 4 + i % 9, 6000 + i) for i in range(140)}
+    long = {"p": tiny.random_tokens(vocab, 2 * page + 9, 6500), "q": tiny.random_tokens(vocab, page + 6, 6501)}
+    requests = {**many, **long}
+    steps: list[dict] = []
+    names = list(many)
+    for first in range(0, len(names), 35):  # the prompts of the many, 35 requests a step, all but their last two tokens
+        steps.append({"step": len(steps), "end": [], "entries": [
+            {"id": rid, "tokens": many[rid][:-2], "want": list(range(len(many[rid]) - 2))} for rid in names[first:first + 35]]})
+    cuts = {"p": [(0, 2), (2, page + 1), (page + 1, 2 * page + 9)], "q": [(0, page + 3), (page + 3, page + 5), (page + 5, page + 6)]}
+    for k in range(3):
+        entries = []
+        if k < 2:
+            entries += [{"id": rid, "tokens": [many[rid][len(many[rid]) - 2 + k]], "want": [0]} for rid in names]
+        for rid in ("q", "p") if k % 2 else ("p", "q"):
+            lo, hi = cuts[rid][k]
+            entries.insert(len(entries) // 2, {"id": rid, "tokens": long[rid][lo:hi], "want": list(range(hi - lo))})
+        steps.append({"step": len(steps), "entries": entries, "end": names if k == 1 else (["p", "q"] if k == 2 else [])})
+    from turboserve_amd.engine.replay import TraceReplayer
+
+    replayer = TraceReplayer(case["folders"][dtype], dtype=dtype, max_tokens=th.peak_tokens(steps, rounding=max(64, page)),
+                             page_size=page, max_live=len(requests))
+    outputs = {}
+    for record in steps:
+        outputs[record["step"]] = replayer.run_step(record).float().cpu()
+    if replayer.runner.graphs is not None:
+        assert replayer.runner.graphs.num_replays == 0
+    replayer.manager.check_invariants()
+    raw, tensors = tiny.read_model_dir(case["folders"][dtype])
+    expected = {rid: plain.forward_logits(raw, tensors, tokens) for rid, tokens in requests.items()}
+    got = th.collect(steps, outputs, requests)
+    check(got, expected, dtype, f"tiny {case['name']} portions beside 140 single tokens", RTOL_BF16_LIBRARY)
+    # ... and all but a few positions inside the bound of the engine's own products
+    ratios = torch.cat([excess(got[rid], want, dtype) for rid, want in expected.items()])
+    assert float((ratios > 1.0).float().mean()) <= 0.005, f"{int((ratios > 1.0).sum())} of {ratios.numel()} positions"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -109,7 +109,7 @@ def test_one_packer_fills_exact_and_padded_shapes():
     entries[1].state_slot = 2
     layout = StepLayout.make(4, 4, 4, (4,))
     data = np.full(layout.total, 77, dtype=np.int32)
-    pack_step(data, layout, entries, range(4), pad_state_slot=9, token_sources={1: 0})
+    pack_step(data, layout, entries, range(4), pad_state_slot=9, token_sources={1: 0}, recorded=True)
     field = lambda name: layout.view(data, name).tolist()
     assert field("token_ids") == [9, 8, 3, 0] and field("positions") == [6, 2, 0, 0]
     assert field("token_seq") == [0, 1, 2, 3] and field("query_start_loc") == [0, 1, 2, 3, 4]
@@ -119,6 +119,18 @@ def test_one_packer_fills_exact_and_padded_shapes():
     assert field("slot_mapping0") == [6, 30, 16, -1]
     assert layout.view(data, "block_table0").reshape(4, 4).tolist() == [[5, 1, 0, 0], [7, 0, 0, 0], [4, 0, 0, 0], [0, 0, 0, 0]]
     check_packed(data, layout, entries, 4, StepLimits(num_pages=[8], windows=[None], vocab_size=10, num_state_slots=9))
+    # the fill of unused table entries follows the kind of step, not whether every row is a request
+    exact = StepLayout.make(3, 3, 3, (4,))
+    filled = np.zeros(exact.total, dtype=np.int32)
+    pack_step(filled, exact, entries, range(3), recorded=True)
+    assert exact.view(filled, "block_table0").reshape(3, 4).tolist() == [[5, 1, 0, 0], [7, 0, 0, 0], [4, 0, 0, 0]]
+    pack_step(filled, exact, entries, range(3))
+    assert exact.view(filled, "block_table0").reshape(3, 4).tolist() == [[5, 1, -1, -1], [7, -1, -1, -1], [4, -1, -1, -1]]
+    # a request whose own table is too short for its context is refused whatever the fill
+    short = [entry("x", [9], 6, [5, 1]), entry("y", [8], 4, [7])]
+    pack_step(filled, exact, [*short, entries[2]], range(3), recorded=True)
+    with pytest.raises(ValueError, match="'y': its block table of group 0 holds 1 pages, 5 tokens need 2"):
+        check_packed(filled, exact, [*short, entries[2]], 4, StepLimits(num_pages=[8], windows=[None]))
     with pytest.raises(ValueError, match="'y': token id 8"):  # a token taken from the device is not known: only 'y' is checked here
         pack_step(data, layout, entries, range(4), pad_state_slot=9, token_sources={0: 0})
         check_packed(data, layout, entries, 4, StepLimits(num_pages=[8], windows=[None], vocab_size=8))
@@ -505,3 +517,27 @@ def test_the_kept_token_array_follows_the_lists():
         if turn == 250:
             seq.reset_for_recompute()
     assert seq.token_array().tolist() == seq.token_ids and seq.num_output_tokens > 100
+
+
+def test_an_attention_geometry_no_kernel_takes_is_refused_when_the_model_is_put_together():
+    """A head size above what the attention kernels take, or an odd one, is refused when the part
+    is built (from the configuration alone, on the host), not at the first step after the weights
+    have been read."""
+    import tiny
+    from turboserve_amd.kernels.ops import ATTENTION_MAX_HEAD_DIM, attention_geometry_error
+    from turboserve_amd.parts.attention import GroupedQueryAttention
+    from turboserve_amd.parts.base import Runtime
+    from turboserve_amd.weights.random_init import describe_model
+
+    describe_model({**tiny.CONFIG_A, "head_dim": ATTENTION_MAX_HEAD_DIM})
+    with pytest.raises(ValueError, match="model.layers.0.self_attn: a head size of 520 is above"):
+        describe_model({**tiny.CONFIG_A, "head_dim": ATTENTION_MAX_HEAD_DIM + 8})
+    assert attention_geometry_error(28, 4, 128) is None and attention_geometry_error(5, 1, 20) is None
+    assert "not a multiple" in attention_geometry_error(6, 4, 64)
+    assert "not even" in attention_geometry_error(4, 2, 33)
+    runtime = Runtime(device=torch.device("cpu"), dtype=torch.float32, ops=None)
+    common = dict(hidden_size=64, scale=1.0, qkv_bias=False, out_bias=False, window=None, position=PartSpec("none"))
+    with pytest.raises(ValueError, match="not even"):
+        GroupedQueryAttention("m", runtime, num_heads=4, num_kv_heads=2, head_dim=7, **common)
+    with pytest.raises(ValueError, match="not a multiple"):
+        GroupedQueryAttention("m", runtime, num_heads=5, num_kv_heads=2, head_dim=8, **common)

@@ -1,12 +1,15 @@
-"""Host models of the addresses two kernels form, checked against their buffers' bounds.
+"""Host models of the addresses three kernels form, checked against their buffers' bounds.
 
 A wild address on the GPU can end more than the test that made it, so the index arithmetic of
-the two kernels whose launches the host plans most freely is restated here in Python and swept
+the kernels whose launches the host plans most freely is restated here in Python and swept
 over shapes, plans and cache states on the CPU: the tiled product (``csrc/gemm_tiled.hip``:
 what a thread fetches, where it stages it in LDS, which fragments a wavefront reads, where the
-sums go) and the decode attention (``csrc/attention_mfma.hip``, ``decode_kernel``: which page and
+sums go), the decode attention (``csrc/attention_mfma.hip``, ``decode_kernel``: which page and
 key every lane reads for every split, with pages given back below a window and table entries
-that are padding).  The models follow the kernels line by line and must be changed with them.
+that are padding) and the 32-row prefill attention (``prefill_wide_kernel``: the block-table
+look-ups of its pipeline, five windows ahead, self-fed and fed, whole blocks and shares of a
+block, and the slots the shares' partial sums go to).  The models follow the kernels line by
+line and must be changed with them.
 """
 
 from __future__ import annotations
@@ -157,3 +160,121 @@ def test_decode_attention_reads_live_pages_only():
             splits = -(-(span + 31) // keys_per_split)
             check_decode(ctx, window, shift, table, splits, keys_per_split)
             check_decode(ctx, window, shift, table, splits, keys_per_split, device_context=ctx)
+
+
+def check_prefill_wide(pos0, cols, window, shift, table, fed, share=None):
+    """``prefill_wide_kernel``'s block-table look-ups for one block of ``cols`` rows whose first
+    row is at ``pos0``: every index lies inside the row, every page a load is formed from is a
+    live one, and a window whose scores are used is fetched from its own pages.  ``share``:
+    (first window, windows) of a block whose keys are shared out."""
+    width = len(table)
+    p_last = pos0 + cols - 1
+    lo_first = max(0, pos0 - window + 1) if window else 0
+    lo_last = max(0, p_last - window + 1) if window else 0
+    begin, end = lo_first & ~31, p_last + 1
+    if share is not None and share[1] > 0:
+        begin += share[0] * WINDOW_KEYS
+        end = min(end, begin + share[1] * WINDOW_KEYS)
+    if begin >= end:
+        return 0
+    rounds = (end - begin + WINDOW_KEYS - 1) // WINDOW_KEYS
+    last_window = (end - 1) & ~31
+    steady_from = (lo_last - begin + WINDOW_KEYS - 1) // WINDOW_KEYS
+    steady_to = min((pos0 + 1 - begin) // WINDOW_KEYS - 6, rounds - 1) if cols == 32 else -1
+    if fed:
+        assert shift >= 4, "the fed form wants pages of 16 keys or more"
+    pieces = [0, 2] if fed else [0, 1, 2, 3]  # the pieces whose page a wavefront looks up (fed: one per half window)
+
+    def window_at(i):
+        return min(begin + i * WINDOW_KEYS, last_window)
+
+    def page_of_chunk(w, piece):
+        index = min((w + 8 * piece) >> shift, width - 1)
+        assert 0 <= index < width
+        return table[index]
+
+    def fetch(w, pages, inside, used):
+        """Keys or values of window ``w`` with the page ids looked up earlier (per looked-up piece)."""
+        if inside or (w >= lo_first and w + 31 <= p_last):
+            for piece, page in zip(pieces, pages):
+                assert page >= 0, (pos0, cols, window, 1 << shift, share, w, piece)
+                if used:
+                    assert page == table[(w + 8 * piece) >> shift]
+                    if fed:  # the half window's other piece lies on the same page
+                        assert (w + 8 * piece + 8) >> shift == (w + 8 * piece) >> shift
+        else:  # a window at the edge looks its pages up per lane
+            for key in range(w, w + 32):
+                live = min(max(key, max(w, lo_first)), min(w + 31, p_last))
+                assert 0 <= live >> shift < width and table[live >> shift] >= 0, (pos0, cols, window, 1 << shift, share, w, key)
+
+    page = [[page_of_chunk(window_at(k), piece) for piece in pieces] for k in range(5)]
+    fetch(window_at(0), page[0], False, True)
+    fetch(window_at(1), page[1], False, rounds > 1)
+    fetch(window_at(2), page[2], False, rounds > 2)
+    page = page[1:]  # page1 .. page4
+    order = []
+    i = 0
+    while i < rounds and i < steady_from:
+        order.append((i, False))
+        if i + 1 < rounds:
+            order.append((i + 1, False))
+        i += 2
+    while i + 1 <= steady_to:
+        order += [(i, True), (i + 1, True)]
+        i += 2
+    while i < rounds:
+        order.append((i, False))
+        if i + 1 < rounds:
+            order.append((i + 1, False))
+        i += 2
+    assert [r for r, _ in order] == list(range(rounds))
+    for i, steady in order:
+        w = begin + i * WINDOW_KEYS
+
+        def at(k, w=w, i=i, steady=steady):
+            return w + k * WINDOW_KEYS if steady else window_at(i + k)
+
+        if steady:  # nothing is tested or clamped: the windows must lie inside what every column sees
+            assert w >= lo_last and at(5) + 31 <= pos0
+        fetch(at(3), page[2], steady, i + 3 < rounds)
+        fetch(at(1), page[0], steady, i + 1 < rounds)
+        page = page[1:] + [[page_of_chunk(at(5), piece) for piece in pieces]]
+    return rounds
+
+
+def test_prefill_attention_looks_up_live_pages_only():
+    """Blocks of the 32-row prefill attention kernel over random contexts, windows, page sizes and
+    shares: whole prompts, portions at the end of long contexts, blocks of fewer than 32 rows,
+    tables with padding behind a request's pages and pages given back below a window."""
+    from turboserve_amd.kernels.ops import prefill_block_windows, prefill_share_list
+
+    rng = random.Random(5)
+    for _ in range(1500):
+        shift = rng.choice([3, 4, 5, 6])
+        page = 1 << shift
+        window = rng.choice([0, 0, 0, 1, 12, 33, 70, 300])
+        count = rng.choice([2, 5, 31, 32, 33, 64, 100, 257, rng.randint(2, 700)])
+        before = rng.choice([0, 0, 7, 32, 45, 1000, rng.randint(0, 3000)])
+        context = before + count
+        needed = -(-context // page)
+        table = [rng.randint(0, 500) for _ in range(needed)] + [-1] * rng.choice([0, 0, 1, 3])
+        if window:  # pages wholly below the lowest key the portion's first row sees were given back
+            for i in range(max(0, before - window + 1) // page):
+                table[i] = -1
+        fed = shift >= 4 and rng.random() < 0.5
+        for offset in range(0, count, 32):
+            check_prefill_wide(before + offset, min(32, count - offset), window, shift, table, fed)
+        # the same blocks with their keys shared out, as the planner would for an idle device
+        blocks, ranges, combine = prefill_share_list([count], [context], 32, window, 1, 4096, rng.choice([1, 2, 16]), combine_cost=0)
+        slots = sum(entry[3] for entry in combine)
+        seen = set()
+        for (_, row), (first, windows, slot) in zip(blocks, ranges):
+            cols = min(32, count - row)
+            assert windows == 0 or first + windows <= prefill_block_windows(before + row, cols, window)
+            check_prefill_wide(before + row, cols, window, shift, table, fed, (first, windows))
+            if slot >= 0:
+                assert slot < slots and slot not in seen  # every share writes a partial slot of its own
+                seen.add(slot)
+        for row, rows, first_slot, shares in combine:
+            assert 0 <= row and row + rows <= count and 0 <= first_slot and first_slot + shares <= slots
+            assert set(range(first_slot, first_slot + shares)) <= seen

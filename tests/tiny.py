@@ -73,7 +73,29 @@ CONFIG_C = {
 }
 PAGE_C = 32
 
-TINY = {"A": (CONFIG_A, 0, PAGE_A), "B": (CONFIG_B, 1, PAGE_B), "C": (CONFIG_C, 2, PAGE_C)}
+#: D: sizes that 16-byte accesses do not divide: a width of 100, a feed-forward of 172 and five
+#: heads of 20 on one KV head (every product's K is 4 more than a multiple of 8, the head size is
+#: no multiple of 8 or 16), an odd vocabulary, tied head, a window of 24 in the second layer.
+CONFIG_D = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 100,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 5,
+    "num_key_value_heads": 1,
+    "intermediate_size": 172,
+    "vocab_size": 333,
+    "rope_theta": 50000.0,
+    "rms_norm_eps": 2e-5,
+    "tie_word_embeddings": True,
+    "use_sliding_window": True,
+    "sliding_window": 24,
+    "max_window_layers": 1,
+    "max_position_embeddings": 192,
+}
+PAGE_D = 16
+
+TINY = {"A": (CONFIG_A, 0, PAGE_A), "B": (CONFIG_B, 1, PAGE_B), "C": (CONFIG_C, 2, PAGE_C), "D": (CONFIG_D, 3, PAGE_D)}
 
 
 #: A wider spread of the weights for 32-bit comparisons.  With the usual 0.02 a model this small

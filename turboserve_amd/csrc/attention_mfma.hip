@@ -925,7 +925,9 @@ struct StagedValues {
 // earlier so that nothing waits for it here; a window at the edge of lo..last looks its pages up
 // per lane instead.
 __device__ __forceinline__ int page_of_chunk(const PageGeometry& g, int w, int wave) {
-  return g.table[__builtin_amdgcn_readfirstlane(w + KEYS_PER_WAVE * wave) >> g.block_shift];
+  // Clamped to the row: in a block's last window the chunk may lie past the last page (such a
+  // window looks its pages up per lane, so the value is dropped, but the load stays inside).
+  return g.table[min(__builtin_amdgcn_readfirstlane(w + KEYS_PER_WAVE * wave) >> g.block_shift, g.table_width - 1)];
 }
 
 // A lane's 32-bit offset as the compiler must see it for a load to take a scalar base and this

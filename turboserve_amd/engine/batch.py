@@ -127,12 +127,15 @@ def pack_step(
     *,
     pad_state_slot: int = 0,
     token_sources: dict[int, int] | None = None,
+    recorded: bool = False,
 ) -> None:
     """Write a step into ``data`` (int32, ``layout.total`` long).  ``entries`` are in row order.
     Where the layout is larger than the step (a recorded shape: more requests, all of one
     token), the rest is padding: position 0, context 1, no cache write, the padding state
-    slot, page 0.  ``token_sources[i] = j``: entry ``i``'s single token is element ``j`` of a
-    device tensor and is patched in on the device."""
+    slot.  ``recorded``: the layout is a recorded step's (a bucket's shape, replayed with any
+    data), and block-table entries no request uses are page 0, not ``PAD_PAGE``.
+    ``token_sources[i] = j``: entry ``i``'s single token is element ``j`` of a device tensor and
+    is patched in on the device."""
     live = len(entries)
     seqs, tokens = layout.num_seqs, layout.num_tokens
     query_lens = [len(e.tokens) for e in entries]
@@ -177,10 +180,10 @@ def pack_step(
     for group, width in enumerate(layout.widths):
         put(f"slot_mapping{group}", _flat([e.slots[group] for e in entries]), -1)  # padding writes nothing
         table = layout.view(data, f"block_table{group}").reshape(seqs, width)
-        # Unused entries: PAD_PAGE in an exact-shape step (as the reference pads, types.py:213-234);
-        # page 0 in a padded shape, whose kernels may form addresses from a whole row (never read
-        # past the context).
-        table[:] = PAD_PAGE if live == seqs else 0
+        # Unused entries: PAD_PAGE in an eager step (as the reference pads, types.py:213-234);
+        # page 0 in a recorded shape (its rows of padding included), whose kernels may form
+        # addresses from a whole row (never read past the context).
+        table[:] = 0 if recorded else PAD_PAGE
         for i, e in enumerate(entries):
             row = table_array(e.tables[group])
             table[i, : row.size] = row
@@ -229,6 +232,13 @@ def check_packed(data: np.ndarray, layout: StepLayout, entries: Sequence[StepEnt
             row, col = (int(v) for v in beyond[0])
             raise ValueError(f"request {name_of(row)}: page id {int(table[row, col])} at index {col} of its block "
                              f"table of group {group} is outside the pool of {pool} pages")
+        # Each request's own table against the pages its context needs (whatever the unused
+        # entries of the packed row were filled with).
+        for row, entry in enumerate(entries):
+            if len(entry.tables[group]) * page_size < int(contexts[row]):
+                raise ValueError(f"request {name_of(row)}: its block table of group {group} holds "
+                                 f"{len(entry.tables[group])} pages, {int(contexts[row])} tokens need "
+                                 f"{-(-int(contexts[row]) // page_size)}")
         lowest_key = np.zeros(seqs, dtype=np.int64) if window is None else np.maximum(0, first_position - window + 1)
         columns = np.arange(width, dtype=np.int64)[None, :]
         read = (columns >= (lowest_key // page_size)[:, None]) & (columns < (-(-contexts // page_size))[:, None])

@@ -9,8 +9,11 @@ shape's layout), copies it to the device and launches the graph.
 Shapes are bucketed so that few graphs serve every batch: the number of requests is rounded up
 to a power of two (the extra rows are padding: position 0, context 1, no cache write, results
 dropped) and each cache group's block-table width to a power of two.  The kernels read the
-true context lengths from the device, so one graph serves every length up to its width.  The
-graphs hold only this engine's own kernels (no library call, no memset node).
+true context lengths from the device, so one graph serves every length up to its width.  What
+the engine's own parts launch in such a step are this engine's kernels only (no BLAS call, no
+memset node): products of up to 128 rows are the weight-streaming kernels, or, where K is no
+multiple of 8, the plain fused-multiply-add kernel.  A part from elsewhere may record torch
+operations; it answers for them with ``Part.capturable``.
 
 The reference has no counterpart: it launches eager torch ops every step
 (src/turboserve/engine/runtime/worker.py:221-233).
@@ -126,7 +129,8 @@ class DecodeGraphs:
         shape.turn ^= 1
         host = shape.host_ints[shape.turn]
         data = host.numpy()
-        pack_step(data, shape.layout, entries, range(shape.batch), pad_state_slot=self.pad_state_slot, token_sources=patch)
+        pack_step(data, shape.layout, entries, range(shape.batch), pad_state_slot=self.pad_state_slot, token_sources=patch,
+                  recorded=True)
         if check and self.limits is not None:
             check_packed(data, shape.layout, entries, self.page_size, self.limits)
         return host

@@ -135,6 +135,24 @@ def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtyp
           "value pages must be [NB, Hkv, D, BS] for key pages [NB, Hkv, BS, D]")
 
 
+#: Largest head size an attention kernel takes (the generic kernel's; the matrix-core kernels stop at 256).
+ATTENTION_MAX_HEAD_DIM = 512
+
+
+def attention_geometry_error(num_heads: int, num_kv_heads: int, head_dim: int) -> str | None:
+    """Why no attention kernel of this library takes a geometry, or ``None`` if one does.  A pure
+    function of the sizes, so a part can refuse at construction, before any weight is read."""
+    if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads != 0:
+        return f"{num_heads} query heads are not a multiple of {num_kv_heads} KV heads"
+    if num_heads > 65535:
+        return f"{num_heads} query heads are more than a launch's 65,535"
+    if head_dim < 2 or head_dim % 2 != 0:
+        return f"a head size of {head_dim} is not even (keys and values are written in pairs)"
+    if head_dim > ATTENTION_MAX_HEAD_DIM:
+        return f"a head size of {head_dim} is above the {ATTENTION_MAX_HEAD_DIM} the attention kernels take"
+    return None
+
+
 def prefill_block_list(query_lens, context_lens, rows: int) -> list[list[int]]:
     """``[request index, first row]`` of every block of ``rows`` consecutive rows of requests that
     bring ``query_lens`` tokens and hold ``context_lens`` afterwards, rows numbered through the
@@ -470,9 +488,9 @@ class Ops:
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows")
         _need(block_table.dim() == 2 and token_seq.numel() == tokens, "block_table [S, MB], token_seq [T]")
-        _need(heads % kv_heads == 0, "query heads must be a multiple of KV heads")
-        _need(head_dim <= 512, "head_dim above 512 is not supported by the attention kernel")
-        out = torch.empty((tokens, heads * head_dim), dtype=q.dtype, device=q.device)
+        _need(attention_geometry_error(heads, kv_heads, head_dim) is None,
+              attention_geometry_error(heads, kv_heads, head_dim) or "")
+        out = self.rows_buffer(tokens, heads * head_dim, q.dtype, q.device)
         _check(self.core.ts_paged_attention_generic(
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim,
@@ -917,17 +935,31 @@ class Ops:
                 return self.gemm_tiled(x, weight, plan=plan, gated=True)
         return self.swiglu(self.linear(x, weight), x.dtype, paired=True)
 
-    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
+               for_residual: bool = False) -> torch.Tensor:
         """The projection of the serving path.  32-bit runs use :meth:`gemm_plain` (no reduced
-        matrix mode).  bfloat16 runs with decode-sized batches use :meth:`gemm_skinny` and
-        return ``[S, M, N]`` 32-bit partial sums for the consumer to add up; larger batches use
-        the BLAS library behind torch, as the reference does for every linear layer
-        (src/turboserve/engine/model/layers.py:142)."""
+        matrix mode).  bfloat16 runs with decode-sized batches (up to ``skinny_max_rows`` rows) use
+        :meth:`gemm_skinny` and return ``[S, M, N]`` 32-bit partial sums for the consumer to add
+        up, or, where K is no multiple of 8 (the matrix-core kernels load 16 bytes at a time),
+        :meth:`gemm_plain` on bfloat16 operands: slower, but a kernel of this engine, so a
+        recorded step never holds a library call.  Larger batches use the BLAS library behind
+        torch, as the reference does for every linear layer
+        (src/turboserve/engine/model/layers.py:142).  ``for_residual``: the result is what a
+        norm adds to the 32-bit residual stream, so the library leaves it in 32-bit too (as
+        ``[1, M, N]``, one partial sum): the stream then gets the same unrounded addend from a
+        prompt's step as from a decode step's partial sums."""
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight, bias)
         _gpu(x, weight, bias)
-        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
-            return self.gemm_skinny(x, weight, bias)
+        if x.shape[0] <= self.skinny_max_rows:
+            if self.skinny_supported(x, weight):
+                return self.gemm_skinny(x, weight, bias)
+            return self.gemm_plain(x, weight, bias)  # a K that 16-byte loads do not divide
+        if for_residual:
+            out = self._library_product(x, weight, None, torch.float32)
+            if bias is not None:
+                out += bias
+            return out.unsqueeze(0)
         return self._library_product(x, weight, bias, None)
 
     def linear_float32_out(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -936,8 +968,10 @@ class Ops:
         if x.dtype == torch.float32:
             return self.gemm_plain(x, weight)
         _gpu(x, weight)
-        if self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
-            return self.gemm_skinny(x, weight, max_splits=1)[0]
+        if x.shape[0] <= self.skinny_max_rows:
+            if self.skinny_supported(x, weight):
+                return self.gemm_skinny(x, weight, max_splits=1)[0]
+            return self.gemm_plain(x, weight, out_float32=True)
         return self._library_product(x, weight, None, torch.float32)
 
     # -- sampling -----------------------------------------------------------------------------

@@ -7,6 +7,7 @@ from collections.abc import Mapping
 
 import torch
 
+from turboserve_amd.kernels.ops import attention_geometry_error
 from turboserve_amd.parts.base import CacheNeed, Mixer, PagedKV, PagedKVView, PartSpec, Runtime, TensorSpec
 from turboserve_amd.parts.registry import build_part, register_mixer
 
@@ -37,8 +38,11 @@ class GroupedQueryAttention(Mixer):
         position: PartSpec,
     ) -> None:
         super().__init__(prefix, runtime)
-        if num_heads % num_kv_heads != 0:
-            raise ValueError(f"{num_heads} query heads is not a multiple of {num_kv_heads} KV heads")
+        # Refused here, when the model is put together, not at the first step after the weights
+        # have been read: a geometry that no attention kernel takes.
+        refusal = attention_geometry_error(int(num_heads), int(num_kv_heads), int(head_dim))
+        if refusal is not None:
+            raise ValueError(f"{prefix or 'attention'}: {refusal}")
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)
@@ -62,8 +66,9 @@ class GroupedQueryAttention(Mixer):
         return self.capturable and self.position.is_capturable()
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        """The fused projection, the attention output and the output projection of a step."""
-        return tokens * (self.q_size + 2 * self.kv_size + self.q_size + self.hidden_size) * itemsize
+        """The fused projection, the attention output and the output projection (32-bit: it is
+        added to the residual stream) of a step."""
+        return tokens * ((self.q_size + 2 * self.kv_size + self.q_size) * itemsize + self.hidden_size * 4)
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs = {
@@ -101,7 +106,7 @@ class GroupedQueryAttention(Mixer):
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache
         )
         attended = self.attend(q, q_stride, ctx, cache)
-        return ops.linear(attended, self.o_weight, self.o_bias_tensor)
+        return ops.linear(attended, self.o_weight, self.o_bias_tensor, for_residual=True)
 
     def attend(self, qkv: torch.Tensor, q_stride: int, ctx, cache: PagedKVView) -> torch.Tensor:
         """``[T, Hq D]`` attention output for the step's encoded queries: the first ``Hq D``

@@ -32,8 +32,9 @@ class SwiGLU(FeedForward):
         }
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
-        """The gate|up projection, the activated product and the down projection of a step."""
-        return tokens * (3 * self.intermediate_size + self.hidden_size) * itemsize
+        """The gate|up projection, the activated product and the down projection (32-bit: it is
+        added to the residual stream) of a step."""
+        return tokens * (3 * self.intermediate_size * itemsize + self.hidden_size * 4)
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         gate, up = tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]
@@ -42,4 +43,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
-        return ops.linear(ops.linear_swiglu(x, self.gate_up_weight), self.down_weight)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up_weight), self.down_weight, for_residual=True)

@@ -6,11 +6,13 @@ from __future__ import annotations
 import random
 
 import pytest
+import torch
 
 from turboserve_amd.cache.allocator import InvalidPageError, OutOfPagesError, PageAllocator
 from turboserve_amd.cache.layout import CacheLayout
 from turboserve_amd.cache.manager import PAD_PAGE, CacheManager
 from turboserve_amd.cache.sizing import MemoryProfileError, size_cache, window_pages_needed
+from turboserve_amd.cache.storage import CacheStorage
 from turboserve_amd.cache.state_slots import OutOfStateSlotsError, StateSlotPool
 from turboserve_amd.config.engine_config import SchedulerConfig
 from turboserve_amd.parts.base import FixedState, PagedKV
@@ -195,6 +197,40 @@ def test_layout_groups_layers_by_their_needs():
     # tests/unit/test_kv_cache_storage.py:267-305: 2 layers, pages of 4, 2 heads of 8, 32-bit: 1024 bytes a page.
     two = CacheLayout.from_needs([full, full], [None, None])
     assert two.bytes_per_page(4, 4) == [1024] and two.bytes_per_token(4) == 256
+
+
+def test_a_layer_may_keep_pages_and_state_and_values_of_another_width():
+    """One schedule entry with several needs gets one unit for each, in order; keys and values
+    of different widths (or no values at all) are a group of their own and are sized apart."""
+    pages, wide, latent, state = PagedKV(2, 8), PagedKV(2, 8, None, 24), PagedKV(1, 16, None, 0), FixedState((3,))
+    layout = CacheLayout.from_needs([(pages, state), wide, (state, None, pages), latent, None, (pages, state)],
+                                    [None, None, None, None, 0, None])
+    assert layout.entry_units == ((("pages", 0, 0), ("state", 0)), ("pages", 1, 0), (("state", 1), None, ("pages", 0, 1)),
+                                  ("pages", 2, 0), ("reads", 0), (("pages", 0, 2), ("state", 2)))
+    assert [(g.head_dim, g.value_width, g.entries) for g in layout.groups] == [(8, 8, (0, 2, 5)), (8, 24, (1,)), (16, 0, (3,))]
+    assert [entry for entry, _ in layout.state_entries] == [0, 2, 5]
+    assert layout.bytes_per_page(4, 2) == [3 * 2 * 16 * 4 * 2, 2 * 32 * 4 * 2, 16 * 4 * 2]
+    # a value width said explicitly and equal to the keys' is the same group as one left out
+    same = CacheLayout.from_needs([PagedKV(2, 8, None, 8), PagedKV(2, 8)], [None, None])
+    assert len(same.groups) == 1 and same.groups[0].value_dim is None
+    with pytest.raises(TypeError, match="unknown cache need"):
+        CacheLayout.from_needs([(pages, "rows")], [None])
+
+    storage = CacheStorage(layout, [5, 6, 7], 4, 2, torch.float32, "cpu")
+    first, second = storage.view_of(0)
+    assert tuple(first.k.shape) == (5, 2, 4, 8) and tuple(first.v.shape) == (5, 2, 8, 4) and first.group == 0
+    assert tuple(second.state.shape) == (3, 3)
+    own = storage.view_of(1)
+    assert tuple(own.k.shape) == (6, 2, 4, 8) and tuple(own.v.shape) == (6, 2, 24, 4) and own.group == 1
+    slot, nothing, again = storage.view_of(2)
+    assert nothing is None and tuple(again.k.shape) == (5, 2, 4, 8) and again.k.data_ptr() != first.k.data_ptr()
+    assert slot.state.data_ptr() != second.state.data_ptr()
+    only_keys = storage.view_of(3)
+    assert tuple(only_keys.k.shape) == (7, 1, 4, 16) and only_keys.v.numel() == 0
+    borrowed = storage.view_of(4)  # reads entry 0's units, all read-only
+    assert not borrowed[0].writable and not borrowed[1].writable and borrowed[0].k.data_ptr() == first.k.data_ptr()
+    assert len(storage.views()) == 6
+    assert storage.num_bytes() == sum(c * b for c, b in zip([5, 6, 7], layout.bytes_per_page(4, 4))) + 3 * 3 * 3 * 4
 
 
 def test_sizing():

@@ -285,9 +285,9 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
     try:
         assert torch.cuda.tunable.is_enabled() and not torch.cuda.tunable.tuning_is_enabled()
         assert not untouched.exists() or "Gemm" not in untouched.read_text()
-        before = [t.clone() for t in engine.storage.pages]
+        before = [t.clone() for t in engine.storage.tensors()]
         engine.runner.dry_run(150)
-        assert all(torch.equal(a, b) for a, b in zip(before, engine.storage.pages))
+        assert all(torch.equal(a, b) for a, b in zip(before, engine.storage.tensors()))
         out = engine.generate([prompt], SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True, logprobs=True))[0]
     finally:
         engine.close()

@@ -132,6 +132,20 @@ def test_attention_and_feed_forward_and_block_parts(dtype, window):
 # -- a toy mixer with state of its own, and a toy architecture ---------------------------------------
 
 
+def _position_buckets(entries):
+    return [(entry.start + i) // 5 for entry in entries for i in range(len(entry.tokens))]
+
+
+def _make_position_bucket_field():
+    from turboserve_amd.engine.batch import StepField
+
+    return StepField("position_bucket", lambda tokens, requests, wanted: tokens, _position_buckets, pad=0)
+
+
+#: The step field of the toy mixer below: defined once, so that every layer of the kind names the same one.
+POSITION_BUCKET = _make_position_bucket_field()
+
+
 def register_toy_architecture():
     """Everything a new mixer and a new architecture need, using only the public registries."""
     from turboserve_amd.config import registry as arch_registry
@@ -173,6 +187,76 @@ def register_toy_architecture():
                     cache.state.index_copy_(0, slot, torch.cat((sums[-1], counts[-1:]))[None])
                     row += count
                 return out
+
+    if "sink_attention" not in part_registry.MIXERS:
+        from turboserve_amd.parts.base import PagedKV
+
+        @part_registry.register_mixer("sink_attention")
+        class SinkAttention(Mixer):
+            """One-head attention whose cached values are wider than its keys, plus the running
+            mean of its inputs: a layer that keeps pages AND fixed-size state, and that asks the
+            step for a field of its own (the bucket of five positions a token lies in, looked up
+            in a learned table and added to the query).  Plain torch operations on the pages, no
+            kernel of the engine: everything is indexed on the device, so it records."""
+
+            def __init__(self, prefix, runtime, *, hidden_size, key_dim, value_dim, buckets):
+                super().__init__(prefix, runtime)
+                self.hidden, self.key_dim, self.value_dim, self.buckets = hidden_size, key_dim, value_dim, buckets
+                self.w = {}
+
+            def cache_need(self):
+                return (PagedKV(1, self.key_dim, None, self.value_dim), FixedState((self.hidden + 1,), torch.float32))
+
+            def step_fields(self):
+                return (POSITION_BUCKET,)
+
+            def tensor_specs(self):
+                h, dk, dv = self.hidden, self.key_dim, self.value_dim
+                shapes = {"q.weight": (dk, h), "k.weight": (dk, h), "v.weight": (dv, h), "o.weight": (h, dv),
+                          "sink.weight": (h, h), "bucket_table": (self.buckets, dk)}
+                return {self.name(key): TensorSpec(shape) for key, shape in shapes.items()}
+
+            def load(self, tensors):
+                self.w = {key: tensors[self.name(key)].float() for key in
+                          ("q.weight", "k.weight", "v.weight", "o.weight", "sink.weight", "bucket_table")}
+
+            def forward(self, x, ctx, cache):
+                pages, state = cache
+                assert tuple(pages.v.shape[1:]) == (1, self.value_dim, pages.block_size) and pages.k.shape[-1] == self.key_dim
+                xf = x.float()
+                bucket = ctx.extras["position_bucket"].long().clamp(max=self.buckets - 1)
+                q = xf @ self.w["q.weight"].t() + self.w["bucket_table"].index_select(0, bucket)
+                k, v = xf @ self.w["k.weight"].t(), xf @ self.w["v.weight"].t()
+                num_pages, size = pages.k.shape[0], pages.block_size
+                # write: slot -> row of the pages seen as [pages x size, width] (a padded row's slot is -1 and matches nothing)
+                slots = ctx.slot_mapping[pages.group].long()
+                hit = (slots[:, None] == torch.arange(num_pages * size, device=x.device)[None, :]).float()  # [T, slots]
+                written = hit.sum(dim=0) > 0
+                flat_k = pages.k.view(num_pages * size, self.key_dim)
+                flat_k.copy_(torch.where(written[:, None], (hit.t() @ k).to(flat_k.dtype), flat_k))
+                flat_v = pages.v.permute(0, 1, 3, 2).reshape(num_pages * size, self.value_dim)
+                flat_v = torch.where(written[:, None], (hit.t() @ v).to(flat_v.dtype), flat_v)
+                pages.v.copy_(flat_v.view(num_pages, 1, size, self.value_dim).permute(0, 1, 3, 2))
+                # read: every token over the keys 0 .. its position of its request, through the block table
+                table = ctx.block_tables[pages.group].index_select(0, ctx.token_seq.long()).long()  # [T, width]
+                places = torch.arange(table.shape[1] * size, device=x.device)
+                where = table.clamp(min=0)[:, places // size] * size + (places % size)[None, :]  # [T, L]
+                keys = flat_k.float()[where]
+                values = flat_v.float()[where]
+                scores = (q[:, None, :] * keys).sum(dim=-1) * self.key_dim ** -0.5
+                scores = scores.masked_fill(places[None, :] > ctx.positions[:, None], float("-inf"))
+                attended = (torch.softmax(scores, dim=-1)[:, :, None] * values).sum(dim=1) @ self.w["o.weight"].t()
+                # the running mean, per request, continued from the request's state slot
+                rows_of = ctx.token_seq.long()
+                slot_of = ctx.state_slots.long().index_select(0, rows_of)
+                before = state.state.index_select(0, slot_of)  # [T, H + 1]
+                same = (rows_of[:, None] == rows_of[None, :]) & (ctx.positions[None, :] <= ctx.positions[:, None])
+                sums = before[:, : self.hidden] + same.float() @ xf
+                counts = before[:, self.hidden] + same.float().sum(dim=1)
+                mean = sums / counts[:, None]
+                last = ctx.query_start_loc[1:].long() - 1  # each request's last row of this step
+                state.state.index_copy_(0, ctx.state_slots.long(), torch.cat((sums, counts[:, None]), dim=1).index_select(0, last))
+                return (attended + mean @ self.w["sink.weight"].t()).to(x.dtype)
 
     if "top1_experts" not in part_registry.FEED_FORWARDS:
 
@@ -322,7 +406,10 @@ def register_toy_architecture():
             toy = PartSpec("running_mean", {"hidden_size": hidden})
             routed = PartSpec("top1_experts", {"hidden_size": hidden, "intermediate_size": cfg["intermediate_size"],
                                                "num_experts": cfg["experts"]})
-            mixers = {"attention": attention, "attention_learned": learned, "attention_biased": biased, "state": toy}
+            sink = PartSpec("sink_attention", {"hidden_size": hidden, "key_dim": cfg["sink_key_dim"],
+                                               "value_dim": cfg["sink_value_dim"], "buckets": cfg["sink_buckets"]})
+            mixers = {"attention": attention, "attention_learned": learned, "attention_biased": biased, "state": toy,
+                      "sink": sink}
             layers = []
             for index, kind in enumerate(cfg["mixers"]):  # mixer and feed-forward are chosen layer by layer
                 block = PartSpec("prenorm", {"mixer": mixers[kind],
@@ -379,6 +466,15 @@ def toy_plain_logits(cfg, tensors, tokens):
             else:
                 mixed = plain.attention(q, k, v, plain.attention_mask(pos, len(tokens), None), dim ** -0.5)
             mixed = mixed.reshape(len(tokens), -1) @ tensors[f"{p}.self_attn.o_proj.weight"].T
+        elif cfg["mixers"][layer] == "sink":
+            a = f"{p}.self_attn"
+            q = x @ tensors[f"{a}.q.weight"].T + tensors[f"{a}.bucket_table"][pos // 5]
+            k, v = x @ tensors[f"{a}.k.weight"].T, x @ tensors[f"{a}.v.weight"].T
+            mask = plain.attention_mask(pos, len(tokens), None)
+            scores = (q @ k.T) * cfg["sink_key_dim"] ** -0.5  # written out: the plain attention has one width for keys and values
+            mixed = torch.softmax(scores.masked_fill(~mask, float("-inf")), dim=-1) @ v
+            mean = torch.cumsum(x, dim=0) / torch.arange(1, len(tokens) + 1)[:, None]
+            mixed = mixed @ tensors[f"{a}.o.weight"].T + mean @ tensors[f"{a}.sink.weight"].T
         else:
             mean = torch.cumsum(x, dim=0) / torch.arange(1, len(tokens) + 1)[:, None]
             mixed = mean @ tensors[f"{p}.self_attn.mix.weight"].T
@@ -400,13 +496,15 @@ TOY_CONFIG = {
     "architectures": ["ToyForCausalLM"], "hidden_size": 40, "intermediate_size": 56, "vocab_size": 97, "heads": 5,
     "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "experts": 3,
     "embedding_multiplier": 1.5, "logit_scale": 0.5, "slopes": [0.5, 0.25, 0.125, 0.0625, 0.03125],
-    "mixers": ["attention", "state", "attention", "attention_learned", "attention_biased"],
-    "feed_forwards": ["swiglu", "routed", "swiglu", "routed", "swiglu"],
+    "sink_key_dim": 8, "sink_value_dim": 24, "sink_buckets": 64,
+    "mixers": ["attention", "state", "attention", "attention_learned", "attention_biased", "sink"],
+    "feed_forwards": ["swiglu", "routed", "swiglu", "routed", "swiglu", "swiglu"],
     # layer 0, the stateful layer (with a routed feed-forward), layer 0 AGAIN (weights reused, a
     # cache of its own), layer 2 reading the cache of the first call instead of keeping one, then
     # a layer whose attention takes learned positions instead of rotation, then one whose position
-    # encoding is a bias on the scores.
-    "schedule": [[0, None], [1, None], [0, None], [2, 0], [3, None], [4, None]],
+    # encoding is a bias on the scores, then a layer that keeps pages (values three times as wide
+    # as its keys) and state, and reads a step field of its own.
+    "schedule": [[0, None], [1, None], [0, None], [2, 0], [3, None], [4, None], [5, None]],
 }
 
 
@@ -424,8 +522,13 @@ def test_toy_model_is_data(toy_folder):
 
     _, model = describe_model(TOY_CONFIG)
     layout = CacheLayout.from_model(model)
-    assert [u and u[0] for u in layout.entry_units] == ["pages", "state", "pages", "reads", "pages", "pages"]
-    assert len(layout.groups) == 1 and layout.groups[0].entries == (0, 2, 4, 5) and layout.state_entries[0][0] == 1
+    assert [u and u[0] for u in layout.entry_units[:6]] == ["pages", "state", "pages", "reads", "pages", "pages"]
+    assert layout.entry_units[6] == (("pages", 1, 0), ("state", 1)), "the last layer keeps pages and state"
+    assert len(layout.groups) == 2 and layout.groups[0].entries == (0, 2, 4, 5) and layout.groups[1].entries == (6,)
+    assert (layout.groups[1].head_dim, layout.groups[1].value_width) == (8, 24)
+    assert [entry for entry, _ in layout.state_entries] == [1, 6]
+    assert [one.name for one in model.step_fields()] == ["position_bucket"]
+    assert "model.layers.5.self_attn.bucket_table" in model.tensor_specs()
     names = list(model.tensor_specs())
     assert "model.layers.1.self_attn.mix.weight" in names and "model.layers.2.self_attn.q_proj.weight" in names
     assert "model.layers.1.mlp.experts.2.down_proj.weight" in names and "model.layers.1.mlp.router.weight" in names
@@ -470,7 +573,7 @@ def test_toy_architecture_generates_through_the_engine_and_the_command_line(toy_
     if dtype == "bfloat16":
         # Without the routed feed-forward: a router's near-tie may fall to another expert in
         # bfloat16, which is a different function, not a rounding error.
-        dense = {**TOY_CONFIG, "feed_forwards": ["swiglu"] * 5}
+        dense = {**TOY_CONFIG, "feed_forwards": ["swiglu"] * 6}
         folder = write_random_model(dense, tmp_path / "toy_bf16", seed=5, dtype=torch.bfloat16, std=0.1)
     raw, tensors = tiny.read_model_dir(folder)
     prompts = [tiny.random_tokens(97, n, 40 + n) for n in (3, 12, 29)]
@@ -489,7 +592,7 @@ def test_toy_architecture_generates_through_the_engine_and_the_command_line(toy_
         max_num_seqs=4, max_num_batched_tokens=16, block_size=8))
     with LLMEngine(config) as engine:
         assert engine.sizing is not None and engine.sizing.reason == "max_model_len cap"
-        assert engine.sizing.num_blocks == [32] and engine.sizing.activation_bytes > 0
+        assert engine.sizing.num_blocks == [32, 32] and engine.sizing.activation_bytes > 0
         outputs = engine.generate(prompts, SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
         for prompt, output in zip(prompts, outputs):
             check_tokens(prompt, output.new_token_ids)
@@ -505,7 +608,7 @@ def test_toy_architecture_generates_through_the_engine_and_the_command_line(toy_
     assert cli.main(["engine", "kv-size", "--model", str(folder), "--dtype", dtype, "--max-model-len", "64", "--block-size", "8"]) == 0
     sizing = capsys.readouterr().out
     sizing = json.loads(sizing[sizing.index("{"):])
-    assert sizing["reason"] == "max_model_len cap" and sizing["num_blocks"] == [8 * 64] and sizing["activation_bytes"] > 0
+    assert sizing["reason"] == "max_model_len cap" and sizing["num_blocks"] == [8 * 64, 8 * 64] and sizing["activation_bytes"] > 0
 
 
 def test_a_part_can_keep_the_model_out_of_graphs(toy_folder):

@@ -177,14 +177,15 @@ def test_a_fault_in_the_last_layers_cache_is_seen(case, dtype):
         table = replayer.manager.get("r").tables[group]
         a, b = table[64 // case["page"] - 2], table[64 // case["page"] - 1]
         assert a >= 0 and b >= 0 and a != b
-        pages = replayer.storage.pages[group][member]  # [2 (keys, values), pages, kv heads, page x head size]
+        keys = replayer.storage.key_pages[group][member]  # [pages, kv heads, page x head size]
+        values = replayer.storage.value_pages[group][member]
         if fault == "lost":
-            pages[1, b] = 0
+            values[b] = 0
         elif fault.startswith("swapped"):
-            which = slice(0, 2) if fault.endswith("keys") else slice(1, 2)
-            kept = pages[which, a].clone()
-            pages[which, a] = pages[which, b]
-            pages[which, b] = kept
+            for pages in (keys, values) if fault.endswith("keys") else (values,):
+                kept = pages[a].clone()
+                pages[a] = pages[b]
+                pages[b] = kept
         rows = [replayer.run_step({"entries": [{"id": "r", "tokens": [t], "want": [0]}]}).float().cpu() for t in tokens[64:]]
         worst[fault] = float(excess(torch.cat(rows), want, dtype).max())
     assert worst["none"] <= 1.0, f"the undisturbed run is off by {worst['none']:.2f} times its bound"

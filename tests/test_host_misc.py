@@ -541,3 +541,36 @@ def test_an_attention_geometry_no_kernel_takes_is_refused_when_the_model_is_put_
         GroupedQueryAttention("m", runtime, num_heads=4, num_kv_heads=2, head_dim=7, **common)
     with pytest.raises(ValueError, match="not a multiple"):
         GroupedQueryAttention("m", runtime, num_heads=5, num_kv_heads=2, head_dim=8, **common)
+
+
+def test_a_parts_own_step_field_travels_in_the_packed_buffer():
+    """A field a part asks for (``Part.step_fields``) lies behind the engine's own in the packed
+    buffer, is filled from the entries in row order, padded in a recorded shape, and reaches the
+    part as ``ctx.extras[name]``."""
+    from turboserve_amd.engine.batch import StepField, merge_step_fields
+
+    age = StepField("request_start", lambda t, s, n: s, lambda entries: [e.start for e in entries], pad=-7)
+    parity = StepField("token_parity", lambda t, s, n: t, lambda entries: [tok % 2 for e in entries for tok in e.tokens])
+    fields = merge_step_fields([age, parity, age])
+    assert fields == (age, parity)
+    with pytest.raises(ValueError, match="different step fields named 'request_start'"):
+        merge_step_fields([age, StepField("request_start", age.length, age.fill, pad=0)])
+    for taken in ("positions", "block_table0", "slot_mapping12"):
+        with pytest.raises(ValueError, match="one of the engine's own"):
+            merge_step_fields([StepField(taken, age.length, age.fill)])
+    entries = [entry("x", [9], 6, [5, 1]), entry("p", [1, 2, 3], 4, [2, 6]), entry("z", [3], 0, [4], want=[0])]
+    ctx = build_context(entries, num_groups=1, page_size=4, device="cpu", extra_fields=fields)
+    assert ctx.extras["request_start"].tolist() == [4, 6, 0]  # the portion first, then the single tokens as given
+    assert ctx.extras["token_parity"].tolist() == [1, 0, 1, 1, 1]
+    assert ctx.token_ids.tolist() == [1, 2, 3, 9, 3] and ctx.logit_rows.tolist() == [4]
+    # the same fields in a recorded shape of four rows: padding behind the three entries
+    single = [entry("x", [9], 6, [5, 1]), entry("y", [8], 2, [7]), entry("z", [3], 0, [4])]
+    layout = StepLayout.make(4, 4, 4, (2,), fields)
+    data = np.full(layout.total, 77, dtype=np.int32)
+    pack_step(data, layout, single, range(4), recorded=True)
+    assert layout.view(data, "request_start").tolist() == [6, 2, 0, -7]
+    assert layout.view(data, "token_parity").tolist() == [1, 0, 1, 0]
+    assert all(start % 4 == 0 for start, _ in layout.offsets.values())
+    with pytest.raises(ValueError, match="'request_start': 5 values for a field of 4"):
+        pack_step(data, StepLayout.make(4, 4, 4, (2,), [StepField("request_start", age.length, lambda entries: [0] * 5)]),
+                  single, range(4))

@@ -1,10 +1,11 @@
 """Device side of the cache: the page tensors of every group and the state tensors.
 
-Per group one tensor ``[members, 2, num_pages, kv_heads, page_size * head_dim]`` (keys at index
-0, values at 1).  A key page of one head is ``[page_size, head_dim]``; a value page is stored
-transposed, ``[head_dim, page_size]``, so that the attention kernels load eight consecutive
-keys' values of one head dimension at once.  The reference keeps
-``[num_blocks, block_size, kv_heads, head_dim]`` per layer
+Per group one tensor of keys ``[members, num_pages, kv_heads, page_size * head_dim]`` and one of
+values ``[members, num_pages, kv_heads, value_dim * page_size]`` (``value_dim`` is ``head_dim``
+unless the group's mixers asked for another width, or for none).  A key page of one head is
+``[page_size, head_dim]``; a value page is stored transposed, ``[value_dim, page_size]``, so
+that the attention kernels load eight consecutive keys' values of one head dimension at once.
+The reference keeps ``[num_blocks, block_size, kv_heads, head_dim]`` per layer
 (src/turboserve/engine/core/kv_cache.py:372-400); the slot contract (``page * page_size +
 offset``) is the same.
 """
@@ -37,12 +38,12 @@ class CacheStorage:
         self.page_size = page_size
         self.num_pages = list(num_pages)
         self.dtype = dtype
-        self.pages = [
-            torch.zeros(
-                (len(group.entries), 2, count, group.num_kv_heads, page_size * group.head_dim),
-                dtype=dtype,
-                device=device,
-            )
+        self.key_pages = [
+            torch.zeros((len(group.entries), count, group.num_kv_heads, page_size * group.head_dim), dtype=dtype, device=device)
+            for group, count in zip(layout.groups, num_pages)
+        ]
+        self.value_pages = [
+            torch.zeros((len(group.entries), count, group.num_kv_heads, group.value_width * page_size), dtype=dtype, device=device)
             for group, count in zip(layout.groups, num_pages)
         ]
         # One row more than there are slots: the row padded batch entries point at.
@@ -54,24 +55,33 @@ class CacheStorage:
         ]
 
     def num_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in (*self.pages, *self.states))
+        return sum(t.numel() * t.element_size() for t in self.tensors())
+
+    def tensors(self) -> list[torch.Tensor]:
+        """Every device tensor of the cache (keys, values, states)."""
+        return [*self.key_pages, *self.value_pages, *self.states]
 
     def view_of(self, entry: int, *, writable: bool = True) -> CacheView:
+        """What schedule entry ``entry`` is handed: the view of its unit, a tuple of views for an
+        entry with several units, the (read-only) views of the entry it reads, or ``None``."""
         unit = self.layout.entry_units[entry]
+        if unit is not None and len(unit) > 0 and unit[0] == "reads":
+            return self.view_of(unit[1], writable=False)
+        if unit is not None and (len(unit) == 0 or not isinstance(unit[0], str)):
+            return tuple(self._unit_view(one, writable) for one in unit)
+        return self._unit_view(unit, writable)
+
+    def _unit_view(self, unit: tuple | None, writable: bool) -> CacheView:
         if unit is None:
             return None
-        if unit[0] == "reads":
-            return self.view_of(unit[1], writable=False)
         if unit[0] == "pages":
             _, group, member = unit
-            tensor = self.pages[group][member]
             spec = self.layout.groups[group]
-            pages = tensor.shape[1]
+            pages = self.num_pages[group]
             return PagedKVView(
-                k=tensor[0].view(pages, spec.num_kv_heads, self.page_size, spec.head_dim),
-                v=tensor[1].view(pages, spec.num_kv_heads, spec.head_dim, self.page_size),
-                group=group, block_size=self.page_size,
-                window=self.layout.groups[group].window, writable=writable,
+                k=self.key_pages[group][member].view(pages, spec.num_kv_heads, self.page_size, spec.head_dim),
+                v=self.value_pages[group][member].view(pages, spec.num_kv_heads, spec.value_width, self.page_size),
+                group=group, block_size=self.page_size, window=spec.window, writable=writable,
             )
         return FixedStateView(state=self.states[unit[1]], writable=writable)
 

@@ -7,8 +7,9 @@ Python lists by four ``torch.tensor`` calls (src/turboserve/engine/runtime/worke
 here all integer inputs travel in one int32 buffer and the context keeps the host's copies of
 the lengths, so nothing is read back.
 
-There is one description of that buffer (``STEP_FIELDS`` / ``GROUP_FIELDS``), one function that
-fills it (``pack_step``) and one that checks what it holds (``check_packed``).  An eager step
+There is one description of that buffer (``STEP_FIELDS`` / ``GROUP_FIELDS``, and behind them the
+fields a model's parts ask for: ``StepField``), one function that fills it (``pack_step``) and
+one that checks what it holds (``check_packed``).  An eager step
 packs into a fresh buffer of exactly its shape; a recorded step (``decode_graph``) packs into a
 pinned buffer of its bucket's shape, the rows beyond the entries being padding.  A field added
 to the tables below therefore reaches both.
@@ -76,6 +77,36 @@ GROUP_FIELDS: tuple[tuple[str, Callable[[int, int, int], int]], ...] = (
 
 
 @dataclass(frozen=True)
+class StepField:
+    """One more integer field of a step, asked for by a part (``Part.step_fields``): it travels
+    in the packed buffer like the engine's own, in eager and in recorded steps, and the part
+    finds it as ``ctx.extras[name]``.  ``length(T, S, n)`` is its length in a step of ``T``
+    tokens, ``S`` requests and ``n`` wanted rows; ``fill(entries)`` gives its values for the
+    step's entries (in row order: multi-token entries first), as many as the entries account
+    for; what lies beyond them (the padding rows of a recorded shape) is ``pad``."""
+
+    name: str
+    length: Callable[[int, int, int], int]
+    fill: Callable[[Sequence["StepEntry"]], Sequence[int]]
+    pad: int = 0
+
+
+def merge_step_fields(fields: Sequence[StepField]) -> tuple[StepField, ...]:
+    """The distinct fields of a model's parts, in first-seen order.  Every layer's part of a kind
+    asks for the same field, so a kind defines its field once (a module-level object that all
+    its instances return); different fields under one name are refused."""
+    taken = {name for name, _ in STEP_FIELDS} | {name for name, _ in GROUP_FIELDS}
+    merged: dict[str, StepField] = {}
+    for one in fields:
+        if one.name in taken or any(one.name.startswith(name) and one.name[len(name):].isdigit() for name, _ in GROUP_FIELDS):
+            raise ValueError(f"step field {one.name!r} is one of the engine's own")
+        if one.name in merged and merged[one.name] != one:
+            raise ValueError(f"two parts ask for different step fields named {one.name!r}")
+        merged.setdefault(one.name, one)
+    return tuple(merged.values())
+
+
+@dataclass(frozen=True)
 class StepLayout:
     """Where each field lies in the packed int32 buffer of a step of one shape."""
 
@@ -85,9 +116,11 @@ class StepLayout:
     widths: tuple[int, ...]
     offsets: dict[str, tuple[int, int]]  # name (group fields: name + group index) -> (start, length)
     total: int
+    extra: tuple[StepField, ...] = ()  # the parts' own fields, behind the engine's
 
     @classmethod
-    def make(cls, num_tokens: int, num_seqs: int, num_logit_rows: int, widths: Sequence[int]) -> "StepLayout":
+    def make(cls, num_tokens: int, num_seqs: int, num_logit_rows: int, widths: Sequence[int],
+             extra: Sequence[StepField] = ()) -> "StepLayout":
         offsets: dict[str, tuple[int, int]] = {}
         cursor = 0
 
@@ -101,7 +134,9 @@ class StepLayout:
         for group, width in enumerate(widths):
             for name, length in GROUP_FIELDS:
                 take(f"{name}{group}", length(num_tokens, num_seqs, width))
-        return cls(num_tokens, num_seqs, num_logit_rows, tuple(widths), offsets, cursor)
+        for one in extra:
+            take(one.name, one.length(num_tokens, num_seqs, num_logit_rows))
+        return cls(num_tokens, num_seqs, num_logit_rows, tuple(widths), offsets, cursor, tuple(extra))
 
     def view(self, buffer: Any, name: str) -> Any:
         """The field's slice of ``buffer`` (a numpy array or a tensor of ``total`` int32)."""
@@ -187,6 +222,11 @@ def pack_step(
         for i, e in enumerate(entries):
             row = table_array(e.tables[group])
             table[i, : row.size] = row
+    for one in layout.extra:
+        values = np.asarray(one.fill(entries), dtype=np.int32).reshape(-1)
+        if values.size > layout.offsets[one.name][1]:
+            raise ValueError(f"step field {one.name!r}: {values.size} values for a field of {layout.offsets[one.name][1]}")
+        put(one.name, values, one.pad)
 
 
 def check_packed(data: np.ndarray, layout: StepLayout, entries: Sequence[StepEntry], page_size: int,
@@ -297,6 +337,8 @@ class StepContext:
     #: A recorded step: replayed with other data than it was recorded with, so a part may use
     #: nothing about the step but its shape, the fields above and what ``derive`` refuses there.
     recorded: bool = False
+    #: The fields the model's parts asked for (``Part.step_fields``), by name: int32 device views.
+    extras: dict = field(default_factory=dict)
     _derived: dict = field(default_factory=dict, repr=False)
 
     def derive(self, key: Hashable, make: Callable[["StepContext"], Any]) -> Any:
@@ -327,6 +369,7 @@ def context_views(layout: StepLayout, device_ints: torch.Tensor) -> dict[str, An
         max_decode_context_dev=layout.view(device_ints, "max_decode_context"),
         slot_mapping=[layout.view(device_ints, f"slot_mapping{g}") for g in groups],
         block_tables=[layout.view(device_ints, f"block_table{g}").view(seqs, layout.widths[g]) for g in groups],
+        extras={one.name: layout.view(device_ints, one.name) for one in layout.extra},
     )
 
 
@@ -368,6 +411,7 @@ def build_context(
     device: torch.device | str,
     check: bool = True,
     limits: StepLimits | None = None,
+    extra_fields: Sequence[StepField] = (),
 ) -> StepContext:
     """Pack a step's entries into device tensors with one copy.
 
@@ -391,7 +435,7 @@ def build_context(
         first_row += n
     logit_rows = [row_of[id(e)] + place for e in given for place in e.want]
     widths = [max((len(e.tables[g]) for e in entries), default=1) or 1 for g in range(num_groups)]
-    layout = StepLayout.make(num_tokens, num_seqs, len(logit_rows), widths)
+    layout = StepLayout.make(num_tokens, num_seqs, len(logit_rows), widths, extra_fields)
     data = np.empty(layout.total, dtype=np.int32)
     pack_step(data, layout, entries, logit_rows)
     if check and limits is not None:

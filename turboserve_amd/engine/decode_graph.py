@@ -35,10 +35,10 @@ def next_power_of_two(n: int) -> int:
 class _Graph:
     """One recorded shape: its static input buffer, context, output and the graph."""
 
-    def __init__(self, batch: int, widths: tuple[int, ...]) -> None:
+    def __init__(self, batch: int, widths: tuple[int, ...], extra_fields=()) -> None:
         self.batch = batch
         self.widths = widths
-        self.layout = StepLayout.make(batch, batch, batch, widths)
+        self.layout = StepLayout.make(batch, batch, batch, widths, extra_fields)
         self.graph: torch.cuda.CUDAGraph | None = None
         self.device_ints: torch.Tensor | None = None
         self.host_ints: list[torch.Tensor] = []
@@ -49,7 +49,7 @@ class _Graph:
 
 class DecodeGraphs:
     def __init__(self, model, views, *, page_size: int, num_groups: int, pad_state_slot: int,
-                 max_batch: int = 128, limits: StepLimits | None = None) -> None:
+                 max_batch: int = 128, limits: StepLimits | None = None, extra_fields=()) -> None:
         self.model = model
         self.views = views
         self.page_size = page_size
@@ -58,6 +58,8 @@ class DecodeGraphs:
         self.max_batch = max_batch
         #: What every replayed step's page ids, slots and token ids are checked against.
         self.limits = limits
+        #: Fields the model's parts add to the packed buffer (``Part.step_fields``).
+        self.extra_fields = tuple(extra_fields)
         self.device = model.runtime.device
         self._graphs: dict[tuple, _Graph] = {}
         self._pool = None
@@ -79,7 +81,7 @@ class DecodeGraphs:
 
     def _build(self, key: tuple) -> _Graph:
         batch, widths = key
-        shape = _Graph(batch, widths)
+        shape = _Graph(batch, widths, self.extra_fields)
         total = shape.layout.total
         shape.device_ints = torch.zeros(total, dtype=torch.int32, device=self.device)
         shape.host_ints = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]

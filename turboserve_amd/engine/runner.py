@@ -39,10 +39,13 @@ class ModelRunner:
         #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``), unless a part
         #: of the model says it cannot be recorded (``Part.capturable``).
         self.graphs: DecodeGraphs | None = None
+        #: Fields the model's parts add to every step's packed buffer.
+        self.extra_fields = model.step_fields()
         if use_graphs and model.is_capturable():
             self.graphs = DecodeGraphs(
                 model, self.views, page_size=storage.page_size, num_groups=len(self.layout.groups),
                 pad_state_slot=storage.pad_state_slot, max_batch=max_graph_batch, limits=self.limits,
+                extra_fields=self.extra_fields,
             )
 
     def release(self) -> None:
@@ -64,6 +67,7 @@ class ModelRunner:
             device=self.model.runtime.device,
             check=self.check,
             limits=self.limits,
+            extra_fields=self.extra_fields,
         )
 
     @torch.inference_mode()
@@ -106,7 +110,8 @@ class ModelRunner:
             tables=[[0] * (-(-num_tokens // page))] * groups, slots=[[-1] * num_tokens] * groups,
             state_slot=self.storage.pad_state_slot, want=[num_tokens - 1],
         )
-        ctx = build_context([entry], num_groups=groups, page_size=page, device=self.model.runtime.device, check=False)
+        ctx = build_context([entry], num_groups=groups, page_size=page, device=self.model.runtime.device, check=False,
+                            extra_fields=self.extra_fields)
         stream = self.model.forward(ctx.token_ids, ctx, self.views)
         self.model.logits(stream, ctx.logit_rows)
         torch.cuda.synchronize(self.model.runtime.device)

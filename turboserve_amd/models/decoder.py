@@ -138,6 +138,17 @@ class DecoderModel:
         return (all(block.is_capturable() for block in self.blocks) and self.embedding.is_capturable()
                 and self.head.is_capturable())
 
+    def step_fields(self) -> tuple:
+        """The integer fields the model's parts want in every step's packed buffer beside the
+        engine's own (``Part.step_fields``), each name once."""
+        from turboserve_amd.engine.batch import merge_step_fields
+
+        asked = [*self.embedding.step_fields()]
+        for block in self.blocks:
+            asked.extend(block.step_fields())
+        asked.extend(self.head.step_fields())
+        return merge_step_fields(asked)
+
     def cache_needs(self) -> list[CacheNeed]:
         """What each schedule entry needs a cache for (``None``: nothing, or it reads another's)."""
         needs: list[CacheNeed] = []

@@ -65,6 +65,9 @@ class GroupedQueryAttention(Mixer):
     def is_capturable(self) -> bool:
         return self.capturable and self.position.is_capturable()
 
+    def step_fields(self) -> tuple:
+        return self.position.step_fields()
+
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """The fused projection, the attention output and the output projection (32-bit: it is
         added to the residual stream) of a step."""

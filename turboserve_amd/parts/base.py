@@ -52,12 +52,19 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class PagedKV:
-    """A mixer's need for per-token cache pages: ``num_kv_heads x head_dim`` keys and values
-    per token; ``window`` keys are ever read again (``None``: all of them)."""
+    """A mixer's need for per-token cache pages: per token ``num_kv_heads`` keys of ``head_dim``
+    elements and as many values of ``value_dim`` (``None``: as wide as the keys; 0: the mixer
+    caches one vector per token and head, and the value pages have no room at all);
+    ``window`` keys are ever read again (``None``: all of them)."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -69,14 +76,17 @@ class FixedState:
     dtype: torch.dtype = torch.float32
 
 
-CacheNeed = PagedKV | FixedState | None
+#: What a mixer asks of the cache: nothing, pages, fixed-size state, or several of these (a
+#: layer that keeps pages and a state of its own gets one view for each, in the order asked).
+CacheNeed = PagedKV | FixedState | None | tuple
 
 
 @dataclass
 class PagedKVView:
     """One cache unit's pages: ``k`` is ``[num_blocks, kv_heads, block_size, head_dim]``, ``v`` is
-    stored transposed, ``[num_blocks, kv_heads, head_dim, block_size]``; ``group`` indexes the step's per-group block tables and slot mappings;
-    ``writable`` is false when the layer reads another layer's cache."""
+    stored transposed, ``[num_blocks, kv_heads, value_dim, block_size]`` (``value_dim`` is
+    ``head_dim`` unless the mixer asked otherwise); ``group`` indexes the step's per-group block
+    tables and slot mappings; ``writable`` is false when the layer reads another layer's cache."""
 
     k: torch.Tensor
     v: torch.Tensor
@@ -95,7 +105,8 @@ class FixedStateView:
     writable: bool = True
 
 
-CacheView = PagedKVView | FixedStateView | None
+#: What a layer call is handed: the view of its one need, or a tuple of views, one per need.
+CacheView = PagedKVView | FixedStateView | None | tuple
 
 
 @dataclass
@@ -157,6 +168,14 @@ class Part:
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:  # pragma: no cover - default
         return None
+
+    def step_fields(self) -> tuple:
+        """Integer fields this part wants in every step's packed buffer beside the engine's own
+        (``engine.batch.StepField``: a name, a length rule, a function that fills it from the
+        step's entries, a padding value): per-token, per-request or per-step numbers that the
+        host knows and the part's kernels need on the device, in eager and in recorded steps
+        alike.  The part finds them as ``ctx.extras[name]``."""
+        return ()
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """Bytes of the transient tensors this part holds at once in a step of ``tokens`` rows
@@ -232,6 +251,8 @@ class Mixer(Part):
     """Mixes information between the tokens of a request (attention, or anything with state)."""
 
     def cache_need(self) -> CacheNeed:
+        """``None``, one :class:`PagedKV` or :class:`FixedState`, or a tuple of them; ``forward``
+        gets the matching view, or a tuple of views in the same order."""
         return None
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: CacheView) -> torch.Tensor:
@@ -259,6 +280,9 @@ class Block(Part):
 
     def is_capturable(self) -> bool:
         return self.capturable and all(part.is_capturable() for part in self.parts())
+
+    def step_fields(self) -> tuple:
+        return tuple(one for part in self.parts() for one in part.step_fields())
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """The largest of its parts' needs: they run one after the other."""

@@ -72,7 +72,7 @@ PAGE = 16
 WORKLOAD_PROMPT, WORKLOAD_NEW = 512, 256
 
 
-def parse_args() -> argparse.Namespace:
+def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     p = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=64)
@@ -107,7 +107,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
-    return p.parse_args()
+    return p.parse_args(argv)
 
 
 def tuning_file() -> str:
@@ -427,8 +427,8 @@ def prefill_flops(config, layers: int, tokens: int) -> float:
     return 2.0 * tokens * linear + attention + 2.0 * config.vocab_size * h
 
 
-def main() -> int:
-    args = parse_args()
+def main(argv: list[str] | None = None) -> int:
+    args = parse_args(argv)
     if args.kernel_shares:
         from turboserve_amd.profiling import format_shares, step_shares
 
@@ -447,7 +447,7 @@ def main() -> int:
     import torch
 
     from turboserve_amd.engine.loading import build_model, make_runtime, resolve_run_dtype
-    from turboserve_amd.hwinfo import collect
+    from turboserve_amd.hwinfo import brief
     from turboserve_amd.weights.random_init import random_tensors_on_device
 
     shape_name, shape = SHAPES[args.shape]
@@ -569,9 +569,7 @@ def main() -> int:
             }
         result["points"] = points
         result["workload"] = workload
-    info = collect()
-    result["hw"] = {"gpu": info["gpu_name"], "torch": info["torch"]["version"], "hip": info["torch"]["hip_version"],
-                    "git": (info["git"]["sha"] or "")[:12]}
+    result["hw"] = brief()
     print(json.dumps(result))
     return 0
 

@@ -9,7 +9,7 @@ import torch
 
 from turboserve_amd.cli import build_parser
 from turboserve_amd.engine.batch import StepEntry, StepLayout, StepLimits, build_context, check_packed, pack_step, validate_entries
-from turboserve_amd.engine.detokenizer import IncrementalDetokenizer, StopStringMatcher, StreamingDecoder
+from turboserve_amd.engine.detokenizer import StopAutomaton, TextStream
 from turboserve_amd.engine.sequence import Sequence
 from turboserve_amd.models.decoder import LayerCall, LayerSpec, ModelPlan
 from turboserve_amd.parts.base import PartSpec
@@ -187,34 +187,85 @@ class FakeTokenizer:
         return out
 
 
-def test_incremental_detokenizer_holds_back_half_characters():
-    """src/turboserve/engine/runtime/streaming.py:142-171."""
-    detok = IncrementalDetokenizer(FakeTokenizer())
-    assert detok.append([0, 1]) == "ab"
-    assert detok.append([99]) == ""  # incomplete character: nothing yet
-    assert detok.append([100]) == "é"
-    assert detok.append([2] * 20) == "c" * 20
-    assert detok.text == "abé" + "c" * 20
-    detok.append([99])
-    assert detok.flush() == "�"  # at the end what is left is emitted
+class PlainText:
+    """A stand-in tokenizer whose tokens are characters."""
+
+    def decode(self, ids, skip_special_tokens=True):
+        return "".join(ids)
+
+
+def test_text_is_released_when_certain_and_half_characters_are_held_back():
+    """src/turboserve/engine/runtime/streaming.py:142-171: the behaviour, not the method."""
+    stream = TextStream(FakeTokenizer())
+    assert stream.push([0, 1]).text == "ab"
+    assert stream.push([99]).text == ""  # incomplete character: nothing yet
+    assert stream.push([100]).text == "é"
+    assert stream.push([2] * 20).text == "c" * 20
+    assert stream.text == "abé" + "c" * 20
+    for token in range(60):  # far past the point where the early tokens stop being decoded again
+        assert stream.push([token]).text == chr(ord("a") + token % 26)
+    assert len(stream._tail) <= TextStream.RESEAL_TOKENS + 1
+    assert stream.push([99]).text == ""
+    assert stream.close() == "\ufffd"  # at the end what is left is emitted
+    assert stream.text == "abé" + "c" * 20 + "".join(chr(ord("a") + t % 26) for t in range(60)) + "\ufffd"
+    # a half character that is completed across a reseal
+    stream = TextStream(FakeTokenizer())
+    stream.push(list(range(TextStream.RESEAL_TOKENS)))
+    assert stream.push([3, 99]).text == "d" and stream.push([100, 4]).text == "ée"
+    # the same text whatever the pieces
+    ids = [5, 99, 100, 7, 99, 100, 99, 100, 1, 2] * 9
+    whole = TextStream(FakeTokenizer())
+    whole.push(ids)
+    pieces = TextStream(FakeTokenizer())
+    for i in range(0, len(ids), 3):
+        pieces.push(ids[i:i + 3])
+    assert whole.text + whole.close() == pieces.text + pieces.close() == FakeTokenizer().decode(ids)
 
 
 def test_stop_strings():
-    """src/turboserve/engine/runtime/streaming.py:193-262."""
-    matcher = StopStringMatcher(["</s>", "END"])
-    assert matcher.feed("hello <").text == "hello "  # "<" could still grow into a stop string
-    assert matcher.feed("b").text == "<b"
-    assert matcher.feed("x</").text == "x"
-    delta = matcher.feed("s>tail")
-    assert delta.stop == "</s>" and delta.text == "" and delta.stopped
-    assert StopStringMatcher([]).feed("anything").text == "anything"
-    decoder = StreamingDecoder(FakeTokenizer(), ["cd"])
-    assert decoder.feed([0, 1]).text == "ab"
-    assert decoder.feed([2]).text == ""
-    delta = decoder.feed([3])
+    """src/turboserve/engine/runtime/streaming.py:193-262: text that may still become a stop
+    string is held back, a completed one ends the request and is cut."""
+    stream = TextStream(PlainText(), ["</s>", "END"])
+    assert stream.push("hello <").text == "hello "  # "<" could still grow into a stop string
+    assert stream.push("b").text == "<b"
+    assert stream.push("x</").text == "x"
+    delta = stream.push("s>tail")
+    assert delta.stop == "</s>" and delta.text == "" and delta.stopped and stream.stopped_by == "</s>"
+    assert stream.push("more").text == "" and stream.close() == "" and stream.text == "hello <bx"
+    assert TextStream(PlainText(), []).push("anything").text == "anything"
+    # held text is released when the request ends otherwise
+    stream = TextStream(PlainText(), ["END"])
+    assert stream.push("the EN").text == "the " and stream.close() == "EN" and stream.text == "the EN"
+    # one stop string inside another, overlapping beginnings, and the same result however the text arrives
+    for text in ("xxabcdyy", "ababcab", "aENENDb", "abcabcabd", "no stop here ab"):
+        results = set()
+        for size in (1, 2, 3, 100):
+            stream = TextStream(PlainText(), ["abcd", "bc", "END", "abd"])
+            for i in range(0, len(text), size):
+                stream.push(text[i:i + size])
+            results.add((stream.text + stream.close(), stream.stopped_by))
+        assert len(results) == 1, (text, results)
+        out, stop = results.pop()
+        firsts = [(text.find(s) + len(s), -len(s), s) for s in ("abcd", "bc", "END", "abd") if s in text]
+        if firsts:  # the stop string that is complete first (the longest of those that end there)
+            end, _, which = min(firsts)
+            assert stop == which and out == text[:end - len(which)]
+        else:
+            assert stop is None and out == text
+    automaton = StopAutomaton(["</s>", "END", ""])
+    assert automaton.stops == ("</s>", "END")
+    state = 0
+    for char, held in zip("a</</s", (0, 1, 2, 1, 2, 3)):
+        state = automaton.step(state, char)
+        assert automaton.held(state) == held and automaton.ended(state) is None
+    assert automaton.ended(automaton.step(state, ">")) == "</s>"
+    decoder = TextStream(FakeTokenizer(), ["cd"])
+    assert decoder.push([0, 1]).text == "ab"
+    assert decoder.push([2]).text == ""
+    delta = decoder.push([3])
     assert delta.stopped and decoder.text == "ab"
-    silent = StreamingDecoder(None, ["x"])
-    assert silent.feed([1, 2]).text == "" and silent.finish() == ""
+    silent = TextStream(None, ["x"])
+    assert silent.push([1, 2]).text == "" and silent.close() == ""
 
 
 def test_command_line_options_are_the_references():
@@ -574,3 +625,28 @@ def test_a_parts_own_step_field_travels_in_the_packed_buffer():
     with pytest.raises(ValueError, match="'request_start': 5 values for a field of 4"):
         pack_step(data, StepLayout.make(4, 4, 4, (2,), [StepField("request_start", age.length, lambda entries: [0] * 5)]),
                   single, range(4))
+
+
+def test_replay_and_bench_are_commands_of_the_one_command_line(capsys):
+    """``turboserve engine replay`` and ``turboserve engine bench`` hand their arguments to the
+    trace replay program and to ``bench.py``; every other command still refuses what it does not
+    know.  The measurement's record names the code by a digest of the sources where there is no
+    git checkout."""
+    from turboserve_amd import cli
+    from turboserve_amd.hwinfo import brief, git_info, source_digest
+
+    assert cli.main(["engine", "bench", "--gpus", "2"]) == 2
+    assert "measures one GPU" in capsys.readouterr().out
+    with pytest.raises(SystemExit) as stop:
+        cli.main(["engine", "replay", "--help"])
+    assert stop.value.code == 0 and "--max-tokens" in capsys.readouterr().out
+    with pytest.raises(SystemExit) as stop:
+        cli.main(["engine", "replay", "--model", "nowhere"])  # trace_run's own parser: the other arguments are required
+    assert stop.value.code == 2
+    capsys.readouterr()
+    with pytest.raises(SystemExit):
+        cli.main(["engine", "kv-size", "--bogus"])
+    assert "unrecognized arguments: --bogus" in capsys.readouterr().err
+    facts = brief()
+    assert set(facts) == {"gpu", "arch", "torch", "hip", "rocm", "git", "source"}
+    assert len(facts["source"]) == 12 and facts["source"] == source_digest()[:12] == git_info()["source_digest"][:12]

@@ -4,12 +4,16 @@ src/turboserve/engine/runtime/engine.py:515-641)::
     turboserve [--log-level L] engine generate PROMPT... --model DIR [options]
     turboserve engine kv-size --model DIR [options]
     turboserve engine random-model --config FILE --out DIR --seed N
+    turboserve engine replay --model DIR --dtype D --out DIR --max-tokens N    (bin/trace_run's arguments)
+    turboserve engine bench [bench.py's arguments]
     turboserve version | hwinfo [--indent N]
 
 Option names, defaults and meanings are the reference's where it has them (``--max-tokens 64``,
 ``--temperature 0`` = greedy, ``--max-num-seqs 8`` for ``generate`` and 64 for ``kv-size``,
 ...).  Added here: ``--prompt-ids`` (prompts as comma-separated token ids, so no tokenizer is
-needed), ``--top-k``, ``--repetition-penalty`` and the ``random-model`` command.  The
+needed), ``--top-k``, ``--repetition-penalty`` and the ``random-model``, ``replay`` and ``bench``
+commands (the last two hand their arguments to the trace replay program and to ``bench.py`` in
+the checkout, which stay programs of their own as well).  The
 reference's ``--offline`` and ``--no-prefix-caching`` are accepted and change nothing (there is
 no download and no prefix cache); ``--prefix-caching`` is refused with that reason.
 """
@@ -83,6 +87,12 @@ def build_parser() -> argparse.ArgumentParser:
     rnd.add_argument("--out", required=True)
     rnd.add_argument("--seed", type=int, default=0)
     rnd.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+
+    replay = engine.add_parser("replay", add_help=False,
+                               help="feed given token ids through a model step by step and write logits (bin/trace_run)")
+    replay.set_defaults(passes_on=True)  # everything behind the command's name goes to that program's own parser
+    bench = engine.add_parser("bench", add_help=False, help="the measurements of bench.py in the checkout")
+    bench.set_defaults(passes_on=True)
     return parser
 
 
@@ -171,8 +181,26 @@ def _random_model(args: argparse.Namespace) -> int:
     return 0
 
 
+def _bench(rest: list[str]) -> int:
+    """``bench.py`` of the checkout this package lies in, with the given arguments."""
+    import importlib.util
+    from pathlib import Path
+
+    path = Path(__file__).resolve().parent.parent / "bench.py"
+    if not path.is_file():
+        print(f"no bench.py beside the package ({path}): the measurements live in the checkout", file=sys.stderr)
+        return 2
+    spec = importlib.util.spec_from_file_location("turboserve_bench", path)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return int(module.main(rest) or 0)
+
+
 def main(argv: list[str] | None = None) -> int:
-    args = build_parser().parse_args(argv)
+    parser = build_parser()
+    args, rest = parser.parse_known_args(argv)
+    if rest and not getattr(args, "passes_on", False):
+        parser.error("unrecognized arguments: " + " ".join(rest))
     logging.basicConfig(level=getattr(logging, str(args.log_level).upper(), logging.INFO),
                         format="%(asctime)s %(levelname)s %(name)s: %(message)s")
     if args.command == "version":
@@ -189,6 +217,12 @@ def main(argv: list[str] | None = None) -> int:
         return _generate(args)
     if args.engine_command == "kv-size":
         return _kv_size(args)
+    if args.engine_command == "replay":
+        from turboserve_amd.engine.replay import main as replay_main
+
+        return replay_main(rest)
+    if args.engine_command == "bench":
+        return _bench(rest)
     return _random_model(args)
 
 

@@ -1,4 +1,13 @@
-"""Incremental detokenisation and stop strings (src/turboserve/engine/runtime/streaming.py:91-351).
+"""Text out of token ids, piece by piece, and stop strings.
+
+The behaviour is the reference's (src/turboserve/engine/runtime/streaming.py:91-351): text is
+passed on as soon as it is certain, a character whose bytes have not all arrived is held back,
+text that could still grow into a stop string is held back, a completed stop string ends the
+request and is cut from its text, and whatever is held when the request ends otherwise is
+passed on.  The design is this engine's: one object per request (:class:`TextStream`) that
+re-decodes only a short tail of the tokens and finds stop strings with one automaton over all
+of them, a character at a time, so that the result does not depend on how the text arrived in
+pieces.
 
 A tokenizer is needed only for text: prompts and outputs as token ids work without one.
 """
@@ -10,12 +19,15 @@ from dataclasses import dataclass
 from pathlib import Path
 from typing import Any
 
-REPLACEMENT_CHAR = "�"
-WINDOW_TOKENS = 8
+#: What a decoder puts where bytes do not (yet) make a character.
+UNDECIDED = "\ufffd"
 
 
 @dataclass
-class DecodedDelta:
+class TextDelta:
+    """What a push of tokens released: ``text`` to pass on, and the stop string that ended the
+    request, if one did."""
+
     text: str = ""
     stop: str | None = None
 
@@ -62,111 +74,141 @@ def get_tokenizer(path: str | Path | None) -> TokenizerFile | None:
     return TokenizerFile(candidate) if candidate.is_file() else None
 
 
-class IncrementalDetokenizer:
-    """Windowed re-decoding: text is the difference between decoding ``tokens[prefix:]`` and
-    ``tokens[prefix:read]``; a window that ends inside a character (U+FFFD) emits nothing yet
-    (streaming.py:91-190)."""
+class StopAutomaton:
+    """All stop strings as one trie with fall-back links (Aho-Corasick): fed a character at a
+    time, its state is the longest end of the text so far that begins a stop string, which is
+    exactly the text that has to be held back; a state that ends a stop string means the
+    request stops.  Where several stop strings end at the same character, the longest counts
+    (it begins earliest)."""
 
-    def __init__(self, tokenizer: Any, *, skip_special_tokens: bool = True) -> None:
+    def __init__(self, stops: Iterable[str]) -> None:
+        self.stops = tuple(dict.fromkeys(s for s in stops if s))
+        self._next: list[dict[str, int]] = [{}]
+        self._depth = [0]
+        self._ends: list[str | None] = [None]  # the longest stop string that ends in this state
+        for stop in self.stops:
+            node = 0
+            for char in stop:
+                if char not in self._next[node]:
+                    self._next[node][char] = len(self._next)
+                    self._next.append({})
+                    self._depth.append(self._depth[node] + 1)
+                    self._ends.append(None)
+                node = self._next[node][char]
+            self._ends[node] = stop
+        # Fall-back links, breadth first: the longest proper end of a state's string that is itself
+        # a beginning of a stop string; a state inherits a stop string that ends in its fall-back.
+        self._back = [0] * len(self._next)
+        queue = list(self._next[0].values())
+        for node in queue:
+            for char, child in self._next[node].items():
+                back = self._back[node]
+                while back and char not in self._next[back]:
+                    back = self._back[back]
+                self._back[child] = self._next[back].get(char, 0)
+                if self._ends[child] is None:
+                    self._ends[child] = self._ends[self._back[child]]
+                queue.append(child)
+
+    def step(self, state: int, char: str) -> int:
+        while state and char not in self._next[state]:
+            state = self._back[state]
+        return self._next[state].get(char, 0)
+
+    def held(self, state: int) -> int:
+        """Characters at the end of the text that may still become a stop string."""
+        return self._depth[state]
+
+    def ended(self, state: int) -> str | None:
+        return self._ends[state]
+
+
+class TextStream:
+    """One request's text.  ``push(token_ids)`` returns what those tokens release; ``close()``
+    what is still held when the request ends for another reason than a stop string.
+
+    Decoding: only a tail of the tokens is ever decoded again.  The tail is re-decoded whole at
+    every push, because a tokenizer joins tokens by rules of its own (a space before a word, a
+    character spread over several tokens); of its text, what was passed on before is skipped
+    and the rest is new, except for the characters at the very end that are still undecided
+    (the decoder's U+FFFD for bytes that do not make a character yet).  When the tail has grown
+    past ``RESEAL_TOKENS`` and ends on a whole character, all but its last ``CONTEXT_TOKENS``
+    tokens are sealed: they are never decoded again, and the kept ones (whose text has been
+    passed on) stay as the context the next tokens are joined to.  Should a tail's text ever
+    not continue what it spelled before (a decoder that rewrites earlier characters), text
+    that is out stays out and the new text goes on from where the two part.
+
+    Without a tokenizer nothing is decoded, no text is released and no stop string is found.
+    """
+
+    RESEAL_TOKENS = 24
+    CONTEXT_TOKENS = 6
+
+    def __init__(self, tokenizer: Any | None, stop: Iterable[str] = (), *, skip_special_tokens: bool = True) -> None:
         self._tokenizer = tokenizer
         self._skip = skip_special_tokens
-        self._tokens: list[int] = []
-        self._prefix = 0
-        self._read = 0
-        self.text = ""
+        self._automaton = StopAutomaton(stop) if tokenizer is not None else StopAutomaton(())
+        self._state = 0
+        self._tail: list[int] = []   # the tokens decoded at every push
+        self._spelled = ""           # the part of the tail's text that has gone to the stop automaton
+        self._held = ""              # text gone to the automaton that it holds back
+        self.stopped_by: str | None = None
+        self.text = ""               # everything released so far
 
-    def _decode(self, ids: list[int]) -> str:
-        return self._tokenizer.decode(list(ids), skip_special_tokens=self._skip)
+    # -- decoding ------------------------------------------------------------------------------
 
-    def append(self, token_ids: Iterable[int]) -> str:
-        new = list(token_ids)
-        if not new:
-            return ""
-        self._tokens.extend(new)
-        before = self._decode(self._tokens[self._prefix:self._read])
-        window = self._decode(self._tokens[self._prefix:])
-        if window.endswith(REPLACEMENT_CHAR):
-            return ""
-        if window.startswith(before):
-            delta = window[len(before):]
-        else:
-            full = self._decode(self._tokens)
-            delta = full[len(self.text):] if full.startswith(self.text) else full
-        self._prefix = self._read
-        self._read = len(self._tokens)
-        if len(self._tokens) - self._prefix > WINDOW_TOKENS:
-            self._prefix = len(self._tokens) - WINDOW_TOKENS
-        self.text += delta
-        return delta
+    def _spell(self) -> str:
+        return self._tokenizer.decode(list(self._tail), skip_special_tokens=self._skip)
 
-    def flush(self) -> str:
-        if self._read >= len(self._tokens):
-            return ""
-        before = self._decode(self._tokens[self._prefix:self._read])
-        window = self._decode(self._tokens[self._prefix:])
-        delta = window[len(before):] if window.startswith(before) else ""
-        self._prefix = self._read
-        self._read = len(self._tokens)
-        self.text += delta
-        return delta
+    def _certain(self, token_ids: Iterable[int]) -> str:
+        """The text that the new tokens make certain."""
+        self._tail.extend(token_ids)
+        spelled = self._spell()
+        decided = len(spelled.rstrip(UNDECIDED))
+        if spelled.startswith(self._spelled):
+            start = len(self._spelled)
+        else:  # the decoder rewrote what it had spelled: go on from where the two texts part
+            start = next((i for i, (a, b) in enumerate(zip(spelled, self._spelled)) if a != b), min(len(spelled), len(self._spelled)))
+        fresh = spelled[start:decided] if decided > start else ""
+        self._spelled = spelled[:max(decided, start)]
+        if len(self._tail) > self.RESEAL_TOKENS and decided == len(spelled):
+            self._tail = self._tail[-self.CONTEXT_TOKENS:]
+            self._spelled = self._spell()
+        return fresh
 
+    # -- stop strings --------------------------------------------------------------------------
 
-class StopStringMatcher:
-    """Holds back the shortest suffix that could still grow into a stop string and cuts the
-    text before a completed one (streaming.py:193-262)."""
+    def _screen(self, fresh: str) -> TextDelta:
+        """Pass ``fresh`` through the stop automaton: what it lets go, and a stop if one ended."""
+        if not self._automaton.stops:
+            return TextDelta(fresh)
+        pending = self._held + fresh
+        for offset, char in enumerate(fresh):
+            self._state = self._automaton.step(self._state, char)
+            ended = self._automaton.ended(self._state)
+            if ended is not None:
+                upto = len(self._held) + offset + 1 - len(ended)
+                self._held, self.stopped_by = "", ended
+                return TextDelta(pending[:upto], ended)
+        keep = self._automaton.held(self._state)
+        self._held = pending[len(pending) - keep:] if keep else ""
+        return TextDelta(pending[:len(pending) - keep])
 
-    def __init__(self, stop: Iterable[str] = ()) -> None:
-        self._stop = tuple(s for s in stop if s)
-        self._max_len = max((len(s) for s in self._stop), default=0)
-        self._buffer = ""
+    # -- the request's side --------------------------------------------------------------------
 
-    @property
-    def is_active(self) -> bool:
-        return bool(self._stop)
-
-    def feed(self, text: str) -> DecodedDelta:
-        if not self._stop:
-            return DecodedDelta(text=text)
-        self._buffer += text
-        hits = [(self._buffer.find(s), s) for s in self._stop if s in self._buffer]
-        if hits:
-            index, matched = min(hits)
-            emit, self._buffer = self._buffer[:index], ""
-            return DecodedDelta(text=emit, stop=matched)
-        keep = 0
-        for length in range(min(len(self._buffer), self._max_len - 1), 0, -1):
-            if any(s.startswith(self._buffer[-length:]) for s in self._stop):
-                keep = length
-                break
-        emit = self._buffer[:len(self._buffer) - keep]
-        self._buffer = self._buffer[len(self._buffer) - keep:]
-        return DecodedDelta(text=emit)
-
-    def flush(self) -> str:
-        pending, self._buffer = self._buffer, ""
-        return pending
-
-
-class StreamingDecoder:
-    """Per-request text state: detokeniser plus stop-string matcher (streaming.py:265-327).
-    Without a tokenizer it emits no text and never stops on a string."""
-
-    def __init__(self, tokenizer: Any | None, stop: Iterable[str] = ()) -> None:
-        self.detokenizer = IncrementalDetokenizer(tokenizer) if tokenizer is not None else None
-        self.matcher = StopStringMatcher(stop if tokenizer is not None else ())
-        self.text = ""
-
-    def feed(self, token_ids: Iterable[int]) -> DecodedDelta:
-        if self.detokenizer is None:
-            return DecodedDelta()
-        delta = self.matcher.feed(self.detokenizer.append(token_ids))
+    def push(self, token_ids: Iterable[int]) -> TextDelta:
+        if self._tokenizer is None or self.stopped_by is not None:
+            return TextDelta()
+        delta = self._screen(self._certain(token_ids))
         self.text += delta.text
         return delta
 
-    def finish(self) -> str:
-        if self.detokenizer is None:
+    def close(self) -> str:
+        """The request ended (length, an end token, an abort): everything still held is text."""
+        if self._tokenizer is None or self.stopped_by is not None:
             return ""
-        tail = self.detokenizer.flush()
-        pending = self.matcher.flush() + tail if self.matcher.is_active else tail
-        self.text += pending
-        return pending
+        spelled = self._spell() if self._tail else ""
+        undecided = spelled[len(self._spelled):] if spelled.startswith(self._spelled) else ""
+        rest, self._held, self._tail, self._spelled = self._held + undecided, "", [], ""
+        self.text += rest
+        return rest

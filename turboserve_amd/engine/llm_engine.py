@@ -20,7 +20,7 @@ import torch
 from turboserve_amd.cache.manager import CacheManager
 from turboserve_amd.cache.sizing import CacheSizing, activation_headroom_bytes, size_cache
 from turboserve_amd.config.engine_config import EngineConfig
-from turboserve_amd.engine.detokenizer import StreamingDecoder, get_tokenizer
+from turboserve_amd.engine.detokenizer import TextStream, get_tokenizer
 from turboserve_amd.engine.outputs import RequestOutput
 from turboserve_amd.engine.scheduler import Scheduler, SchedulerOutput
 from turboserve_amd.engine.sequence import Sequence
@@ -131,7 +131,7 @@ class LLMEngine:
         self.sampler = sampler if sampler is not None else Sampler(model.runtime.ops)
         if (config.tune_gemm_tokens or config.tune_gemm_step_sizes) and runner is None:
             self._tune_library_products()
-        self._decoders: dict[str, StreamingDecoder] = {}
+        self._decoders: dict[str, TextStream] = {}
         self._seed = config.seed if config.seed is not None else time.time_ns() & 0xFFFFFFFF
         self._num_generated_tokens = 0
         self._num_prompt_tokens = 0
@@ -219,7 +219,7 @@ class LLMEngine:
             request_id, token_ids, sampling, priority=priority, arrival=arrival,
             sample_seed=self._request_seed(sampling, self.scheduler._next_seq_id),
         )
-        self._decoders[request_id] = StreamingDecoder(self.tokenizer, sampling.stop)
+        self._decoders[request_id] = TextStream(self.tokenizer, sampling.stop)
         self._num_prompt_tokens += len(token_ids)
         return seq
 
@@ -349,14 +349,14 @@ class LLMEngine:
     def _emit(self, seq: Sequence, token: int, reason, logprob, *, now: float) -> RequestOutput:
         decoder = self._decoders.get(seq.request_id)
         if decoder is None:
-            decoder = self._decoders[seq.request_id] = StreamingDecoder(self.tokenizer, seq.sampling.stop)
-        delta = decoder.feed((token,))
+            decoder = self._decoders[seq.request_id] = TextStream(self.tokenizer, seq.sampling.stop)
+        delta = decoder.push((token,))
         text = delta.text
         if delta.stopped and reason is None:
             self.scheduler.finish(seq, FinishReason.STOP, now=now)
             reason = FinishReason.STOP
         elif reason is not None and not delta.stopped:
-            text += decoder.finish()
+            text += decoder.close()
         if reason is not None:
             self._decoders.pop(seq.request_id, None)
         return RequestOutput(

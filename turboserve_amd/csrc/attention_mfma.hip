@@ -203,9 +203,13 @@ struct ValueFrags {
 };
 struct WindowFrags : KeyFrags, ValueFrags {};
 
-// Issue the loads of window `w` (keys outside lo..last: see live_key).
+// Issue the loads of window `w` (keys outside lo..last: see live_key).  ONCE: the keys and
+// values are read by this wavefront alone (a decode step reads every cached key once), so the
+// loads are marked non-temporal.
+template <bool ONCE = false>
 __device__ __forceinline__ void load_window(WindowFrags& f, const PageGeometry& g, int w, int lo, int last,
                                             int lane16, int group) {
+  auto load8 = [](const uint16_t* p) -> Frag8 { return ONCE ? load_once16(p) : *reinterpret_cast<const u32x4*>(p); };
   const WindowPages wp = window_pages(g, w);
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -387,15 +391,15 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
     QueryFrags qf;
     load_query(qf, head_valid ? q + (size_t)token * q_stride + (size_t)head * D : nullptr, group);
     WindowFrags fa, fb;
-    load_window(fa, geo, begin, lo, p, lane16, group);
+    load_window<true>(fa, geo, begin, lo, p, lane16, group);
     int w = begin;
     while (true) {
-      if (w + WINDOW_KEYS < end) load_window(fb, geo, w + WINDOW_KEYS, lo, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window<true>(fb, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fa, w, lo, p, group);
       attend_window<true>(st, fa, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;
       if (w >= end) break;
-      if (w + WINDOW_KEYS < end) load_window(fa, geo, w + WINDOW_KEYS, lo, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window<true>(fa, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fb, w, lo, p, group);
       attend_window<true>(st, fb, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;

@@ -41,12 +41,12 @@ __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row
   const int base = k0 + 8 * group;
   if (k0 + CHUNK <= k_limit) {
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) w.piece[j] = *reinterpret_cast<const u32x4*>(row + base + 32 * j);
+    for (int j = 0; j < STEPS; ++j) w.piece[j] = load_once16(row + base + 32 * j);
   } else {
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
       const int k = base + 32 * j;
-      w.piece[j] = (k < k_limit) ? *reinterpret_cast<const u32x4*>(row + k) : u32x4{0u, 0u, 0u, 0u};
+      w.piece[j] = (k < k_limit) ? load_once16(row + k) : u32x4{0u, 0u, 0u, 0u};
     }
   }
 }

@@ -96,7 +96,7 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
 #pragma unroll
     for (int i = 0; i < Regs::X_PIECES; ++i) r.x[i] = *reinterpret_cast<const u32x4*>(xsrc[i] + k0);
 #pragma unroll
-    for (int i = 0; i < Regs::W_PIECES; ++i) r.w[i] = *reinterpret_cast<const u32x4*>(wsrc[i] + k0);
+    for (int i = 0; i < Regs::W_PIECES; ++i) r.w[i] = load_once16(wsrc[i] + k0);
   };
   auto stage = [&](const Regs& r, int buf, int it) {
     uint16_t* base = lds + buf * STAGE + dst;

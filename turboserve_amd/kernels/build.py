@@ -38,6 +38,7 @@ MODULES: dict[str, tuple[str, ...]] = {
         "gemm_skinny.hip",
         "gemm_tiled.hip",
         "sampling.hip",
+        "probe.hip",
     ),
 }
 

@@ -203,13 +203,20 @@ struct ValueFrags {
 };
 struct WindowFrags : KeyFrags, ValueFrags {};
 
-// Issue the loads of window `w` (keys outside lo..last: see live_key).  ONCE: the keys and
-// values are read by this wavefront alone (a decode step reads every cached key once), so the
-// loads are marked non-temporal.
-template <bool ONCE = false>
+// Issue the loads of window `w` (keys outside lo..last: see live_key).  ONCE: bit 0, the keys,
+// bit 1, the values are read with non-temporal loads (by this wavefront alone: a decode step
+// reads every cached key once).  A decode step wants that for the values only (DECODE_ONCE): an
+// instruction of theirs reads runs of 512 bytes, one of the keys' 64 bytes of each of 16 rows, so
+// two instructions share every 128-byte line, and marking those costs more than it gains
+// (7B heads, attention and combine, plain / keys / values / both: 8 requests at 8,192 tokens
+// 30.7 / 30.5 / 29.3 / 29.5 us, 64 at 8,192 188 / 177 / 172 / 171, 64 at 640 22.8 / 23.4 / 21.8 /
+// 23.4).
+constexpr int DECODE_ONCE = 2;
+template <int ONCE = 0>
 __device__ __forceinline__ void load_window(WindowFrags& f, const PageGeometry& g, int w, int lo, int last,
                                             int lane16, int group) {
-  auto load8 = [](const uint16_t* p) -> Frag8 { return ONCE ? load_once16(p) : *reinterpret_cast<const u32x4*>(p); };
+  auto load8 = [](const uint16_t* p) -> Frag8 { return (ONCE & 1) ? load_once16(p) : *reinterpret_cast<const u32x4*>(p); };
+  auto load8v = [](const uint16_t* p) -> Frag8 { return (ONCE & 2) ? load_once16(p) : *reinterpret_cast<const u32x4*>(p); };
   const WindowPages wp = window_pages(g, w);
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -224,7 +231,7 @@ __device__ __forceinline__ void load_window(WindowFrags& f, const PageGeometry& 
   const uint16_t* vp = value_chunk(g, wp, w, live ? chunk : (live_key(chunk, w, lo, last) & ~7));
 #pragma unroll
   for (int n = 0; n < NT; ++n)
-    f.v[n] = load8(vp + ((long long)(16 * n + lane16) << g.block_shift));
+    f.v[n] = load8v(vp + ((long long)(16 * n + lane16) << g.block_shift));
 }
 
 // Values of keys beyond `last` are whatever an earlier owner of the page left: clear them, so
@@ -349,6 +356,7 @@ __device__ __forceinline__ float column_sum(float l) { return groups_sum(l); }
 // decode: grid (splits, kv_heads * head_tiles, requests); one wavefront each.
 // partial_acc [requests, heads, splits, D] float; partial_ml [requests, heads, splits, 2] float.
 // ---------------------------------------------------------------------------------------------
+template <int ONCE>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(TS_WAVES_PER_SIMD, TS_WAVES_PER_SIMD)))
 decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
               const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
@@ -391,15 +399,15 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
     QueryFrags qf;
     load_query(qf, head_valid ? q + (size_t)token * q_stride + (size_t)head * D : nullptr, group);
     WindowFrags fa, fb;
-    load_window<true>(fa, geo, begin, lo, p, lane16, group);
+    load_window<ONCE>(fa, geo, begin, lo, p, lane16, group);
     int w = begin;
     while (true) {
-      if (w + WINDOW_KEYS < end) load_window<true>(fb, geo, w + WINDOW_KEYS, lo, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window<ONCE>(fb, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fa, w, lo, p, group);
       attend_window<true>(st, fa, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;
       if (w >= end) break;
-      if (w + WINDOW_KEYS < end) load_window<true>(fa, geo, w + WINDOW_KEYS, lo, p, lane16, group);
+      if (w + WINDOW_KEYS < end) load_window<ONCE>(fa, geo, w + WINDOW_KEYS, lo, p, lane16, group);
       if (w < lo || w + WINDOW_KEYS > ctx) clear_stale_values(fb, w, lo, p, group);
       attend_window<true>(st, fb, qf, w, group, lo, p, scale_log2);
       w += WINDOW_KEYS;
@@ -1605,7 +1613,8 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
   const int head_tiles = (heads / kv_heads + 15) / 16;
   if (kv_heads * head_tiles > 65535) return TS_ERR_SHAPE;
   dim3 grid(splits, kv_heads * head_tiles, requests);
-  hipLaunchKernelGGL(decode_kernel, grid, dim3(64), 0, stream, (float*)partial_acc, (float*)partial_ml,
+  // The values are read with non-temporal loads, the keys with plain ones (DECODE_ONCE).
+  hipLaunchKernelGGL(decode_kernel<DECODE_ONCE>, grid, dim3(64), 0, stream, (float*)partial_acc, (float*)partial_ml,
                      (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages,
                      block_table, table_width, query_start_loc, context_lens, seq_begin, heads, kv_heads,
                      shift, scale * LOG2E, window, keys_per_split, splits, max_context);

@@ -37,16 +37,18 @@ struct WeightChunk {
 
 // `row` points at the lane's weight row; k_limit = K: pieces at or beyond it read as zero
 // (K is a multiple of 8, so a piece is wholly inside or wholly outside).
+template <bool ONCE>
 __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row, int k0, int group, int k_limit) {
+  auto load = [](const uint16_t* p) -> u32x4 { return ONCE ? load_once16(p) : *reinterpret_cast<const u32x4*>(p); };
   const int base = k0 + 8 * group;
   if (k0 + CHUNK <= k_limit) {
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) w.piece[j] = load_once16(row + base + 32 * j);
+    for (int j = 0; j < STEPS; ++j) w.piece[j] = load(row + base + 32 * j);
   } else {
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
       const int k = base + 32 * j;
-      w.piece[j] = (k < k_limit) ? load_once16(row + k) : u32x4{0u, 0u, 0u, 0u};
+      w.piece[j] = (k < k_limit) ? load(row + k) : u32x4{0u, 0u, 0u, 0u};
     }
   }
 }
@@ -56,7 +58,7 @@ __device__ __forceinline__ void load_weights(WeightChunk& w, const uint16_t* row
 // the range is longer than LDS should hold) and its wavefronts then stream their weight rows
 // without meeting at a barrier again, two chunks of loads in flight each.  mpad is 8 or 16;
 // lanes whose activation row is beyond mpad read a real row again and drop the result.
-template <int WAVES>
+template <int WAVES, bool ONCE>
 __global__ void __launch_bounds__(WAVES * TS_WAVE)
 gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restrict__ x, long x_stride,
                             const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int mpad,
@@ -82,8 +84,8 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restr
     const int pieces_per_row = stage * (CHUNK / 8);
     const uint16_t* xl = xs_resident + (lane16 % mpad) * x_row + 8 * group;
     WeightChunk wa, wb;
-    load_weights(wa, wrow, first * CHUNK, group, k);
-    if (first + 1 < last) load_weights(wb, wrow, (first + 1) * CHUNK, group, k);
+    load_weights<ONCE>(wa, wrow, first * CHUNK, group, k);
+    if (first + 1 < last) load_weights<ONCE>(wb, wrow, (first + 1) * CHUNK, group, k);
     for (int begin = first; begin < last; begin += stage) {
       const int end = min(begin + stage, last);
       if (begin != first) __syncthreads();  // everyone has read the previous stretch
@@ -107,14 +109,14 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restr
           const u32x4 b = *reinterpret_cast<const u32x4*>(xc + 32 * j);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa.piece[j]), as_bf16x8(b), acc, 0, 0, 0);
         }
-        if (c + 2 < last) load_weights(wa, wrow, (c + 2) * CHUNK, group, k);
+        if (c + 2 < last) load_weights<ONCE>(wa, wrow, (c + 2) * CHUNK, group, k);
         if (c + 1 >= end) break;
 #pragma unroll
         for (int j = 0; j < STEPS; ++j) {
           const u32x4 b = *reinterpret_cast<const u32x4*>(xc + CHUNK + 32 * j);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb.piece[j]), as_bf16x8(b), acc, 0, 0, 0);
         }
-        if (c + 3 < last) load_weights(wb, wrow, (c + 3) * CHUNK, group, k);
+        if (c + 3 < last) load_weights<ONCE>(wb, wrow, (c + 3) * CHUNK, group, k);
       }
     }
   }
@@ -148,9 +150,10 @@ gemm_skinny_resident_kernel(float* __restrict__ partial, const uint16_t* __restr
 // wavefronts (16 weight rows each) per workgroup, 4 or 8.  stage_chunks: chunks staged at a time,
 // an even number unless it covers a whole split; the LDS it needs,
 // mpad * (min(stage_chunks, chunks_per_split) * 256 + 8) * 2 bytes with mpad = 8 or 16, must be <= 64 KiB.
+// once: the weights are read with non-temporal loads.
 extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_stride, const void* w, const void* bias,
                                        int m, int n, int k, int chunks_per_split, int splits, int waves,
-                                       int stage_chunks, hipStream_t stream) {
+                                       int stage_chunks, int once, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!partial || !x || !w || m < 0 || n < 0 || k < 8) return TS_ERR_ARG;
   if (m > 16 || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
@@ -165,13 +168,14 @@ extern "C" int ts_gemm_skinny_resident(float* partial, const void* x, long x_str
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
   dim3 grid((n + 16 * waves - 1) / (16 * waves), splits), block(waves * TS_WAVE);
-  if (waves == 4)
-    hipLaunchKernelGGL((gemm_skinny_resident_kernel<4>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m,
-                       mpad, n, k, chunks_per_split, stage_chunks);
-  else if (waves == 8)
-    hipLaunchKernelGGL((gemm_skinny_resident_kernel<8>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m,
-                       mpad, n, k, chunks_per_split, stage_chunks);
-  else
-    return TS_ERR_SHAPE;
+  if (waves != 4 && waves != 8) return TS_ERR_SHAPE;
+#define TS_LAUNCH_RESIDENT(W, O)                                                                                      \
+  hipLaunchKernelGGL((gemm_skinny_resident_kernel<W, O>), grid, block, lds, stream, partial, xp, x_stride, wp, bp, m, \
+                     mpad, n, k, chunks_per_split, stage_chunks)
+  if (waves == 4 && once) TS_LAUNCH_RESIDENT(4, true);
+  else if (waves == 4) TS_LAUNCH_RESIDENT(4, false);
+  else if (once) TS_LAUNCH_RESIDENT(8, true);
+  else TS_LAUNCH_RESIDENT(8, false);
+#undef TS_LAUNCH_RESIDENT
   return ts_launch_status();
 }

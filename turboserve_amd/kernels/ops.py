@@ -56,7 +56,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                    c_int, c_int, c_void_p],
+                                    c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_hbm_read": [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_long, c_long, c_int, c_long, c_long, c_int,
                         c_void_p],
@@ -698,6 +698,8 @@ class Ops:
     skinny_resident_rows = 16
     #: Wavefronts per workgroup of the resident variant (4 or 8); 0 chooses by the grid's size.
     skinny_resident_wg = 0
+    #: Whether the resident product reads its weights with non-temporal loads.
+    skinny_resident_once = False
     #: Chunks of 256 staged in LDS at a time for up to 8 rows and for up to 16 rows (even numbers).
     skinny_stage_chunks = (10, 4)
 
@@ -717,10 +719,6 @@ class Ops:
         waves = self.skinny_resident_wg or (8 if (splits == limit or -(-n // 128) * splits >= 4 * self.compute_units) else 4)
         return per_split, splits, waves, self.skinny_stage_chunks[0 if m <= 8 else 1]
 
-    #: Up to this many rows a product of a wide matrix (at least 200 tiles of 160 rows) stays with
-    #: the resident-activation kernel, which is a little faster there; everything else up to 128
-    #: rows runs the tiled kernel.
-    resident_wide_rows = 8
     #: Matrices smaller than this many bytes stay with the resident kernel up to 16 rows: the product
     #: lasts a few microseconds and the resident kernel's many small workgroups start faster.
     resident_small_bytes = 64 << 20
@@ -827,7 +825,8 @@ class Ops:
         per_split, splits, waves, stage = self._resident_plan(m, n, -(-k // 256), max_splits)
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_skinny_resident(_ptr(partial), _ptr(x), x_stride, _ptr(weight), _ptr(bias),
-                                                 m, n, k, per_split, splits, waves, stage, self.stream()),
+                                                 m, n, k, per_split, splits, waves, stage,
+                                                 1 if self.skinny_resident_once else 0, self.stream()),
                "ts_gemm_skinny_resident")
         return partial
 
@@ -835,19 +834,18 @@ class Ops:
                     *, max_splits: int | None = None) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
         K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``: the
-        tiled kernel, except for a few rows against a wide matrix (the resident kernel is a
-        little faster there)."""
+        tiled kernel, except for up to 16 rows against a small matrix (the resident kernel's
+        many small workgroups start faster)."""
         if self._resident_runs(x.shape[0], weight.shape[0], weight.shape[1]):
             return self.gemm_resident(x, weight, bias, max_splits=max_splits)
         return self.gemm_tiled(x, weight, bias, max_splits=max_splits)
 
     def _resident_runs(self, m: int, n: int, k: int) -> bool:
         """Whether the resident kernel, not the tiled one, runs a decode-sized product: small
-        matrices up to 16 rows, the widest ones up to eight (the head of the 7B shape at eight rows:
-        189 against 197 us)."""
-        if m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes:
-            return True
-        return m <= self.resident_wide_rows and -(-n // 160) >= 200
+        matrices up to 16 rows.  (Before the weights were read with non-temporal loads it also
+        ran the widest matrices at up to eight rows; now the tiled kernel is faster there: the
+        head of the 7B shape at eight rows in 173 against 189 us.)"""
+        return m <= self.skinny_resident_rows and 2 * n * k < self.resident_small_bytes
 
     #: Row counts that steps of more rows than the decode products take are run at by the BLAS
     #: library (ascending; empty: every step at its own size).  The library's choice of kernel is

@@ -14,9 +14,12 @@ weights (N(0, 0.02), norm gains 1) and 8 requests whose prompts of uniform-rando
 are prefilled (chunked, by the engine) to a context of 8,192 tokens; then W untimed and K timed
 decode steps.  One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` times
 one 2,048-token prompt from arrival to its first token; ``roofline`` prices the decode step
-against HBM bandwidth; ``points`` holds decode at batch 1 and 64 at the same context and the
-benchmark's literal workload (prompts of 512 tokens, 256 generated, end-of-sequence ignored,
-greedy) at 1, 8 and 64 requests, with the details of those runs under ``workload``.  The
+against HBM bandwidth (against the published peak, and against what a kernel that only reads
+gets from this device, ``read_probe``); ``points`` holds decode at batch 1 and 64 at the same
+context, the benchmark's literal workload (prompts of 512 tokens, 256 generated,
+end-of-sequence ignored, greedy) at 1, 8 and 64 requests, with the details of those runs under
+``workload``, and further sizes, detailed under ``further``: prompts of 8,192 and 32,767 tokens
+in portions of 2,048, and decode at batch 1 and 8 with about 32 k tokens of context.  The
 prefill's projections are BLAS-library products; which of the library's kernels runs each is
 timed once at the engine's start (``--no-gemm-tuning`` leaves it to the library's heuristic).
 Peaks are the published MI355X figures: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3
@@ -27,7 +30,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -66,6 +69,7 @@ SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, num_hidden_layers=48, num_attention
 SHAPE_32B = dict(SHAPE_14B, num_hidden_layers=64, intermediate_size=27648)
 SHAPES = {"7b": ("Qwen2.5-7B", SHAPE_7B), "14b": ("Qwen2.5-14B", SHAPE_14B), "32b": ("Qwen2.5-32B", SHAPE_32B)}
 CONTEXT = 8192
+LONG_CONTEXT = 32768
 PREFILL_TOKENS = 2048
 PAGE = 16
 #: The benchmark's literal decode workload: prompt length and generated tokens.
@@ -104,6 +108,11 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                    help="with --closed-loop: temperature 0.7, top-p 0.8, top-k 20, repetition penalty 1.05 instead of greedy")
     p.add_argument("--sample-kernel", type=int, default=0, metavar="ROWS",
                    help="time the sampling kernel alone on ROWS rows of logits of the shape's vocabulary, and exit")
+    p.add_argument("--hbm-read", action="store_true",
+                   help="time a kernel that only reads, walking memory in several ways with plain and non-temporal "
+                        "loads (what the memory gives: the practical ceiling of the decode step), and exit")
+    p.add_argument("--no-further", action="store_true",
+                   help="skip the further sizes: prefill of 8,192 and 32,767 tokens, decode at 32 k tokens of context")
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
@@ -243,15 +252,17 @@ def run_workload(model, config, batch: int, prompt_len: int, new_tokens: int, ru
             "total_seconds": total, "total_tokens_per_s": batch * new_tokens / total}
 
 
-def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True) -> float:
+def run_prefill(model, config, tokens: int, repeats: int = 3, tune: bool = True, budget: int | None = None) -> float:
     """Seconds (best of ``repeats``) from the arrival of a ``tokens``-long prompt to its first
-    token on the host, through ``LLMEngine`` with a step budget that takes the prompt whole."""
+    token on the host, through ``LLMEngine`` with a step budget that takes the prompt whole, or
+    with ``budget`` tokens a step (the prompt then runs in portions, as it does in serving)."""
     import torch
 
     from turboserve_amd.sampling.params import SamplingParams
 
-    engine = make_engine(model, config, max_num_seqs=1, budget=tokens, tokens_per_request=tokens + 1,
-                         tune_tokens=(tokens,) if tune else ())
+    budget = min(tokens, budget or tokens)
+    engine = make_engine(model, config, max_num_seqs=1, budget=budget, tokens_per_request=tokens + 1,
+                         tune_tokens=(budget,) if tune else ())
     prompt = random_prompts(config, 1, tokens, 4321)[0]
     best = float("inf")
     for attempt in range(repeats + 1):
@@ -406,6 +417,60 @@ def run_sample_kernel(shape: dict, rows: int, launches: int = 20) -> dict:
     return result
 
 
+def run_hbm_read(launches: int = 12) -> dict:
+    """What the memory gives a kernel that only reads (``csrc/probe.hip``), in GB/s, for a few ways
+    of walking 272 MB (the 7B shape's gate|up matrix; five copies in turn, so that no cache holds
+    them): the rows as a checkpoint stores them in tiles of 160, 64 and 32 rows as the decode
+    products walk them, the same bytes with every workgroup's iteration contiguous, and one long
+    contiguous stream per workgroup; each with plain and with non-temporal loads."""
+    import torch
+
+    from turboserve_amd.kernels.ops import Ops
+
+    ops = Ops("cuda:0")
+    n, k = 37888, 3584
+    row_bytes, iters, copies = 2 * k, k // 128, 5
+    size = (n + 512) * row_bytes
+    buffers = [torch.randint(0, 2 ** 31 - 1, (size // 4,), dtype=torch.int32, device="cuda") for _ in range(copies)]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def rate(iterations: int, **walk) -> float:
+        read = walk["workgroups"] * 16 * walk["pieces"] * iterations * 256
+        for buffer in buffers:
+            ops.hbm_read(buffer, iters=iterations, **walk)
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            start.record()
+            for _ in range(max(1, launches // copies)):
+                for buffer in buffers:
+                    ops.hbm_read(buffer, iters=iterations, **walk)
+            stop.record()
+            stop.synchronize()
+            best = min(best, start.elapsed_time(stop) * 1e-3 / (max(1, launches // copies) * copies))
+        return round(read / best / 1e9, 1)
+
+    table: dict[str, float] = {}
+    for once in (False, True):
+        tag = "non-temporal" if once else "plain"
+        for pieces, ahead in ((10, 2), (4, 2), (2, 1)):
+            rows = 16 * pieces
+            table[f"rows as stored, {rows} a workgroup, {tag}"] = rate(
+                iters, workgroups=-(-n // rows), pieces=pieces, ahead=ahead, wg_stride=rows * row_bytes, it_stride=256,
+                blk_rows=rows, blk_stride=0, row_stride=row_bytes, non_temporal=once)
+            table[f"iteration contiguous, {rows} rows a workgroup, {tag}"] = rate(
+                iters, workgroups=-(-n // rows), pieces=pieces, ahead=ahead, wg_stride=iters * rows * 256,
+                it_stride=rows * 256, blk_rows=rows, blk_stride=0, row_stride=256, non_temporal=once)
+        for workgroups in (256, 1024):
+            chunk = 16 * 4 * 256
+            count = n * row_bytes // (workgroups * chunk)
+            table[f"one contiguous stream a workgroup, {workgroups} workgroups, {tag}"] = rate(
+                count, workgroups=workgroups, pieces=4, ahead=2, wg_stride=count * chunk, it_stride=chunk, blk_rows=64,
+                blk_stride=0, row_stride=256, non_temporal=once)
+    return {"kernel": "read-only probe", "bytes": n * row_bytes, "unit": "GB/s", "rates": table,
+            "best": max(table.values()), "peak": HBM_PEAK_GBS}
+
+
 def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
     """Bytes a decode step has to read: every weight it uses once (all but the embedding
     table, of which it reads one row per request) and the cache of the live requests."""
@@ -436,6 +501,9 @@ def main(argv: list[str] | None = None) -> int:
         return 0
     if args.sample_kernel:
         print(json.dumps(run_sample_kernel(SHAPES[args.shape][1], args.sample_kernel)))
+        return 0
+    if args.hbm_read:
+        print(json.dumps(run_hbm_read()))
         return 0
     if args.attention_prefill:
         sizes = [int(v) for v in args.attention_prefill.split(",")]
@@ -569,6 +637,30 @@ def main(argv: list[str] | None = None) -> int:
             }
         result["points"] = points
         result["workload"] = workload
+    if not args.no_further and not args.no_points and args.shape == "7b" and full_layers == layers:
+        # Further sizes and contexts: long prompts in portions of the step budget, and decode steps
+        # whose requests hold about 32 k tokens (the shape's max_position_embeddings).
+        further = {}
+        for tokens in (8192, LONG_CONTEXT - 1):
+            seconds = run_prefill(model, config, tokens, repeats=2, tune=tune, budget=PREFILL_TOKENS)
+            result.setdefault("points", {})[f"prefill_{tokens}"] = round(tokens / seconds, 1)
+            further[f"prefill_{tokens}"] = {"ms": round(seconds * 1e3, 2), "budget": PREFILL_TOKENS,
+                                            "frac": round(prefill_flops(config, layers, tokens) / seconds / PEAK_FLOPS[dtype_key], 4)}
+        for batch in (1, 8):
+            steps, warmup = 24, 12
+            run = run_decode(model, config, batch, LONG_CONTEXT - 1 - steps - warmup - 16, steps=steps, warmup=warmup,
+                             run_ahead=run_ahead)
+            read = decode_bytes(config, layers, batch, run["mean_context"], itemsize)
+            result["points"][f"decode_b{batch}_ctx{LONG_CONTEXT}"] = round(run["tokens_per_s"], 2)
+            further[f"decode_b{batch}_ctx{LONG_CONTEXT}"] = {
+                "ms_per_step": round(run["step_seconds"] * 1e3, 4), "mean_context": round(run["mean_context"], 1),
+                "hbm_frac": round(read / run["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4)}
+        result["further"] = further
+    if not args.no_points:
+        # What a kernel that only reads gets from this device's memory: the decode step's practical ceiling.
+        probe = run_hbm_read(launches=10)
+        result["roofline"]["read_probe"] = probe["best"]
+        result["roofline"]["frac_of_read_probe"] = round(achieved / probe["best"], 4)
     result["hw"] = brief()
     print(json.dumps(result))
     return 0

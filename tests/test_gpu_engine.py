@@ -301,6 +301,7 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
     from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
 
     ops = Ops("cuda:0")
+    ops.wide_default_rows = 0  # the library's product is the one under test here
     g = torch.Generator().manual_seed(3)
     # A width of its own for every run of this test: a shape that was timed before in this process
     # is not timed again, and nothing would be written.
@@ -322,13 +323,17 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
         torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
 
 
-def test_library_products_at_timed_step_sizes(model, tmp_path):
+def test_library_products_at_timed_step_sizes(model, tmp_path, monkeypatch):
     """An engine told to run the library's products at a few timed sizes: prompts of lengths
     between the sizes, alone and cut into portions beside decoded tokens, give the plain
-    implementation's log-probabilities, and their products did run at the sizes."""
+    implementation's log-probabilities, and their products did run at the sizes.  (The engine's
+    own product for steps of many rows is switched off: the library's is the one under test.)"""
     from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
     from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.kernels.ops import Ops
     from turboserve_amd.sampling.params import SamplingParams
+
+    monkeypatch.setattr(Ops, "wide_default_rows", 0)
 
     prompts = [tiny.random_tokens(model["vocab"], length, 900 + length) for length in (131, 203, 250, 390)]
     sampling = SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True, logprobs=True)

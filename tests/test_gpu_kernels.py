@@ -202,12 +202,84 @@ def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
             x.to(DEV), w.to(DEV), torch.zeros(2 * inter).bfloat16().to(DEV), plan=plan, gated=True)
 
 
-def test_library_product_at_a_larger_size_ignores_the_rows_behind(ops):
+WIDE_GRIDS = [(2, 128, 4), (4, 128, 4), (5, 128, 4), (2, 256, 4), (4, 256, 4), (5, 256, 4),
+              (2, 128, 8), (4, 128, 8), (5, 128, 8), (2, 256, 8), (4, 256, 8), (5, 256, 8), (8, 256, 8)]
+
+
+@pytest.mark.parametrize("tile,x_rows,waves", WIDE_GRIDS)
+@pytest.mark.parametrize("m,n,k", [(130, 97, 72), (300, 500, 200), (257, 322, 136), (513, 640, 1096), (129, 1000, 40)])
+def test_gemm_wide_every_tile_and_grid(ops, tile, x_rows, waves, m, n, k):
+    """The product for steps of many rows with its grid given by hand: every tile of weight rows,
+    both heights of the activation tile, four and eight wavefronts, one range of K (a bfloat16
+    result with the bias) and several (32-bit partial sums), last tiles partly beyond N and M, a K
+    that is no multiple of the 64 an iteration takes and one below it; and the SwiGLU in the
+    product's epilogue against the two-kernel way."""
+    g = torch.Generator().manual_seed(tile * 1000 + n + x_rows + waves)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    b = torch.randn(n, generator=g).bfloat16()
+    want = x.double() @ w.double().T + b.double()
+    iters = -(-k // 64)
+    one = ops.gemm_wide(x.to(DEV), w.to(DEV), b.to(DEV), plan=(iters, 1, tile, x_rows, waves))
+    assert one.shape == (m, n) and one.dtype == torch.bfloat16
+    assert float((one.double().cpu() - want).abs().max()) <= 1e-2 * float(want.abs().max() + 1)
+    for per_split in sorted({1, 2, max(1, iters - 1)}):
+        splits = -(-iters // per_split)
+        if splits == 1:
+            continue
+        partial = ops.gemm_wide(x.to(DEV), w.to(DEV), b.to(DEV), plan=(per_split, splits, tile, x_rows, waves))
+        assert partial.shape == (splits, m, n) and partial.dtype == torch.float32
+        got = partial.double().sum(0).cpu()
+        assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1), per_split
+    if n % 2 == 0:
+        fused = ops.gemm_wide(x.to(DEV), w.to(DEV), plan=(iters, 1, tile, x_rows, waves), gated=True)
+        two_steps = ops.swiglu(ops.gemm_wide(x.to(DEV), w.to(DEV), plan=(iters, 1, tile, x_rows, waves)), paired=True)
+        y = x.double() @ w.double().T
+        gated = torch.nn.functional.silu(y[:, 0::2]) * y[:, 1::2]
+        assert fused.shape == (m, n // 2)
+        assert float((fused.double().cpu() - gated).abs().max()) <= 1e-2 * float(gated.abs().max() + 1)
+        # the fused form rounds once, the two-kernel form twice: equal up to that
+        assert float((fused.double() - two_steps.double()).abs().max()) <= 1e-2 * float(gated.abs().max() + 1)
+    with pytest.raises(Exception, match="one range of K"):
+        ops.gemm_wide(x.to(DEV), w.to(DEV), plan=(1, iters, tile, x_rows, waves), gated=True) if iters > 1 else ops.gemm_wide(
+            x.to(DEV), w.to(DEV), b.to(DEV), plan=(iters, 1, tile, x_rows, waves), gated=True)
+
+
+def test_gemm_wide_rows_do_not_depend_on_the_batch_and_plans_fill_the_device(ops):
+    """A row's result is the same bits whatever rows stand beside it (for one grid), rows behind
+    the step's own reach nothing, and the planner's grids for the 7B shape's matrices give most
+    compute units a workgroup."""
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(300, 264, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(500, 264, generator=g) * 0.1).bfloat16().to(DEV)
+    plan = (5, 1, 4, 128, 8)
+    whole = ops.gemm_wide(x, w, plan=plan)
+    assert torch.equal(ops.gemm_wide(x[100:260], w, plan=plan), whole[100:260])
+    shuffled = torch.randperm(300, generator=g).to(DEV)
+    assert torch.equal(ops.gemm_wide(x[shuffled], w, plan=plan), whole[shuffled])
+    for n, k in ((4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944)):
+        for m in (130, 256, 512, 1000):
+            for one_range in (False, True):
+                per_split, splits, tile, x_rows, waves = ops._wide_plan(m, n, k, one_range)
+                assert splits == -(-(-(-k // 64)) // per_split) and (splits == 1 or not one_range)
+                workgroups = -(-n // (32 * tile)) * -(-m // x_rows) * splits
+                assert one_range or workgroups >= 0.8 * ops.compute_units, (m, n, k, workgroups)
+    # through `linear`: 200 rows take the own kernel by default, and give the library's result up to rounding
+    y = ops.linear(x[:200], w)
+    assert y.dtype == torch.bfloat16 and y.shape == (200, 500)
+    torch.testing.assert_close(y.float(), x[:200].float() @ w.float().t(), rtol=2e-2, atol=2e-2)
+    sums = ops.linear(x[:200], w, for_residual=True)
+    torch.testing.assert_close(ops.dense(sums, torch.bfloat16).float(), x[:200].float() @ w.float().t(), rtol=2e-2, atol=2e-2)
+
+
+def test_library_product_at_a_larger_size_ignores_the_rows_behind(ops, monkeypatch):
     """With sizes set for the library's products, a step's activations are allocated up to the
     next size and the product runs that long; the rows behind the step's own (not-a-numbers
-    here) reach no row of the result, and a buffer without the room runs at its own size."""
+    here) reach no row of the result, and a buffer without the room runs at its own size.
+    (The engine's own product for such steps is switched off here.)"""
     from turboserve_amd.kernels.ops import Ops
 
+    monkeypatch.setattr(Ops, "wide_default_rows", 0)
     sized = Ops(DEV)
     sized.library_buckets = (192, 256)
     g = torch.Generator().manual_seed(12)

@@ -160,9 +160,16 @@ class LLMEngine:
             ops.library_buckets = ops.bucket_sizes(budget)  # until close(): the model may outlive this engine
             sizes.update(size for size in ops.library_buckets if size > ops.skinny_max_rows)
         started = time.perf_counter()
+        ops = self.model.runtime.ops
         with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
-            for tokens in sorted(sizes):
-                self.runner.dry_run(tokens)
+            # Inside, every product of more rows than a decode step has runs both ways once, by the
+            # library's best kernel and by this engine's own, and the faster one is kept.
+            ops.time_wide_choices = True
+            try:
+                for tokens in sorted(sizes):
+                    self.runner.dry_run(tokens)
+            finally:
+                ops.time_wide_choices = False
         logger.info("library products timed for steps of %s tokens in %.1f s (%d choices kept in %s)",
                     sorted(sizes), time.perf_counter() - started, tuning.num_results(), tuning.results_file)
 

@@ -37,6 +37,7 @@ MODULES: dict[str, tuple[str, ...]] = {
         "gemm_plain.hip",
         "gemm_skinny.hip",
         "gemm_tiled.hip",
+        "gemm_wide.hip",
         "sampling.hip",
         "probe.hip",
     ),

@@ -55,6 +55,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                           c_int, c_int, c_void_p],
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
+        "ts_gemm_wide": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -269,6 +271,12 @@ class Ops:
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._tiled_plans: dict[tuple, tuple[int, int, int]] = {}  # (m, n, k, max_splits) -> grid of the tiled product
+        self._wide_plans: dict[tuple, tuple[int, int, int, int, int]] = {}  # (m, n, k, one range) -> grid of the wide product
+        #: (rows a step's products run at, N, K, kind) -> whether this engine's own product was the
+        #: faster one when both were timed (``time_wide_choices``).
+        self.wide_choices: dict[tuple, bool] = {}
+        #: While true, a product of many rows whose choice is not known yet runs both ways, timed.
+        self.time_wide_choices = False
         #: Compute units of the device (256 on an MI355X): the launch plans below size their grids by it.
         self.compute_units = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         #: Wavefronts a decode attention launch aims for (each keeps two windows of loads in
@@ -709,6 +717,12 @@ class Ops:
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= 128
                 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0)
 
+    @staticmethod
+    def skinny_supported_any_rows(x: torch.Tensor, weight: torch.Tensor) -> bool:
+        """bfloat16 and K a multiple of 8: what this engine's matrix-core products take, whatever the rows."""
+        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
+                and x.stride(0) % 8 == 0 and x.stride(1) == 1 and weight.is_contiguous())
+
     def _resident_plan(self, m: int, n: int, chunks: int, max_splits: int | None) -> tuple[int, int, int, int]:
         """(chunks per split, splits, wavefronts per workgroup, chunks staged at a time) of the
         skinny product with resident activations: splits sized for a number of wavefronts."""
@@ -806,6 +820,113 @@ class Ops:
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_tiled(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
                                        per_split, splits, tile, self.stream()), "ts_gemm_tiled")
+        return partial
+
+    #: Up to this many rows a product that was not timed against the BLAS library runs this
+    #: engine's own kernel (more than ``skinny_max_rows``: ``gemm_wide``).  At the 7B shape the own
+    #: kernel is the faster one up to about a thousand rows (down projection at 256 / 512 rows: 47 /
+    #: 75 us against the library's best 75 / 116; gate|up with its SwiGLU 78 / 149 against 89 / 151),
+    #: the library above (2,048 rows: gate|up 516 against 402 + 44 us, down 270 against 241).
+    wide_default_rows = 640
+
+    def _wide_plan(self, m: int, n: int, k: int, one_range: bool) -> tuple[int, int, int, int, int]:
+        """(iterations of 64 per range of K, ranges, tile, activation rows, wavefronts) of the wide
+        product for ``m`` rows: the cheapest grid by a small model of what a compute unit does.
+        A workgroup's time is its iterations times its tile's area over how well that tile feeds
+        the matrix cores (measured at 2,048 rows: tiles of 256 x 256, 160 x 256, 128 x 256,
+        160 x 128 and 128 x 128 reach 1.06, 0.92, 0.87, 0.75 and 0.72 PFLOP/s) plus a start; the
+        workgroups run in rounds of one per compute unit; partial sums of several ranges of K
+        are written here and read by the consumer.  ``one_range``: the consumer wants one
+        bfloat16 result."""
+        key = (m, n, k, one_range)
+        known = self._wide_plans.get(key)
+        if known is not None:
+            return known
+        iters = -(-k // 64)
+        units = self.compute_units
+        unit_flops_per_us = 2.5e9 * 256 / units / 256  # a compute unit's share of the matrix peak, a microsecond
+        best = None
+        for tile, x_rows, rate in ((8, 256, 1.06), (5, 256, 0.92), (4, 256, 0.87), (5, 128, 0.75), (4, 128, 0.72)):
+            if x_rows == 256 and m <= 128:
+                continue
+            per_iteration = 2.0 * 32 * tile * x_rows * 64 / (rate / 2.5 * unit_flops_per_us)  # microseconds
+            for want in range(1, (1 if one_range else min(iters, 24)) + 1):
+                per_split = -(-iters // want)
+                splits = -(-iters // per_split)
+                if splits != want:
+                    continue
+                workgroups = -(-n // (32 * tile)) * -(-m // x_rows) * splits
+                rounds = -(-workgroups // units)
+                cost = rounds * (per_split + 3) * per_iteration
+                if splits > 1:
+                    cost += 2.0 * splits * m * n * 4 / 4e6  # the partial sums' way through memory, 4 TB/s
+                if best is None or cost < best[0]:
+                    best = (cost, per_split, splits, tile, x_rows, 8)
+        self._wide_plans[key] = best[1:]
+        return best[1:]
+
+    def _wide_runs(self, rows: int, n: int, k: int, kind: str, plan, own, library) -> bool:
+        """Whether this engine's own product (with the grid ``plan``), not the BLAS library's, runs
+        a product of ``rows`` rows (more than the decode products take): what a timing found, or,
+        untimed, up to ``wide_default_rows`` rows if the grid gives at least half of the compute
+        units a workgroup.  With ``time_wide_choices`` an unknown product that is worth timing
+        runs both ways here (``own()`` and ``library()``), three times each behind a warm-up, by
+        device events."""
+        key = (self.library_rows(rows), n, k, kind)
+        known = self.wide_choices.get(key)
+        if known is not None:
+            return known
+        if not self.time_wide_choices or rows * n * k < self.library_tuning_min_work:
+            workgroups = -(-n // (32 * plan[2])) * -(-rows // plan[3]) * plan[1]
+            return rows <= self.wide_default_rows and (2 * workgroups >= self.compute_units or rows * n * k < self.library_tuning_min_work)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        times = []
+        for run in (own, library):
+            run()
+            run()
+            start.record()
+            for _ in range(3):
+                run()
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop))
+        self.wide_choices[key] = times[0] <= times[1]
+        return self.wide_choices[key]
+
+    def gemm_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
+                  plan: tuple[int, int, int, int, int], gated: bool = False) -> torch.Tensor:
+        """``x [M, K] @ weight [N, K]^T (+ bias)`` by the LDS-tiled kernel for steps of many rows
+        (``csrc/gemm_wide.hip``): any M, K a multiple of 8.  ``plan`` = (iterations of 64 per range
+        of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup).  One range: bfloat16 ``[M, N]``; several:
+        32-bit partial sums ``[S, M, N]`` (bias in the first).  ``gated``: the weight is a gate|up
+        projection whose rows alternate gate, up, and the result is ``silu(gate) * up`` as
+        bfloat16 ``[M, N / 2]`` (one range of K, no bias)."""
+        _gpu(x, weight, bias)
+        _need(x.dim() == 2 and x.stride(1) == 1 and weight.dim() == 2 and weight.is_contiguous()
+              and x.shape[1] == weight.shape[1], "x must be [M, K] with unit inner stride, weight contiguous [N, K]")
+        _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0,
+              "the wide product takes bfloat16 and K % 8 == 0")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
+        per_split, splits, tile, x_rows, waves = plan
+        x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
+        if gated:
+            _need(splits == 1 and bias is None and n % 2 == 0,
+                  "the gated result needs one range of K, no bias and an even number of weight rows")
+            out = self.rows_buffer(m, n // 2, torch.bfloat16, x.device)
+            _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k, per_split, splits,
+                                          tile, x_rows, waves, 2, self.stream()), "ts_gemm_wide")
+            return out
+        if splits == 1:
+            out = self.rows_buffer(m, n, torch.bfloat16, x.device)
+            _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
+                                          splits, tile, x_rows, waves, 0, self.stream()), "ts_gemm_wide")
+            return out
+        partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+        _check(self.core.ts_gemm_wide(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
+                                      splits, tile, x_rows, waves, 1, self.stream()), "ts_gemm_wide")
         return partial
 
     def gemm_resident(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
@@ -940,6 +1061,15 @@ class Ops:
             plan = self._tiled_plan(x.shape[0], weight.shape[0], weight.shape[1], None)
             if plan[1] == 1 and weight.shape[0] % 2 == 0 and weight.is_contiguous() and x.stride(1) == 1:
                 return self.gemm_tiled(x, weight, plan=plan, gated=True)
+        elif (x.dtype == torch.bfloat16 and self.skinny_supported_any_rows(x, weight) and weight.shape[0] % 2 == 0
+              and weight.is_contiguous() and x.stride(1) == 1):
+            _gpu(x, weight)
+            m, (n, k) = x.shape[0], weight.shape
+            plan = self._wide_plan(m, n, k, True)
+            if self._wide_runs(m, n, k, "gated", plan, lambda: self.gemm_wide(x, weight, plan=plan, gated=True),
+                               lambda: self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True)):
+                return self.gemm_wide(x, weight, plan=plan, gated=True)
+            return self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True)
         return self.swiglu(self.linear(x, weight), x.dtype, paired=True)
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
@@ -949,9 +1079,10 @@ class Ops:
         :meth:`gemm_skinny` and return ``[S, M, N]`` 32-bit partial sums for the consumer to add
         up, or, where K is no multiple of 8 (the matrix-core kernels load 16 bytes at a time),
         :meth:`gemm_plain` on bfloat16 operands: slower, but a kernel of this engine, so a
-        recorded step never holds a library call.  Larger batches use the BLAS library behind
-        torch, as the reference does for every linear layer
-        (src/turboserve/engine/model/layers.py:142).  ``for_residual``: the result is what a
+        recorded step never holds a library call.  Larger batches use :meth:`gemm_wide` or the
+        BLAS library behind torch (as the reference does for every linear layer,
+        src/turboserve/engine/model/layers.py:142), whichever was the faster one when both were
+        timed (``_wide_runs``).  ``for_residual``: the result is what a
         norm adds to the 32-bit residual stream, so the library leaves it in 32-bit too (as
         ``[1, M, N]``, one partial sum): the stream then gets the same unrounded addend from a
         prompt's step as from a decode step's partial sums."""
@@ -962,6 +1093,15 @@ class Ops:
             if self.skinny_supported(x, weight):
                 return self.gemm_skinny(x, weight, bias)
             return self.gemm_plain(x, weight, bias)  # a K that 16-byte loads do not divide
+        if self.skinny_supported_any_rows(x, weight):
+            m, (n, k) = x.shape[0], weight.shape
+            # What goes into the residual stream may stay partial sums (the norm adds them up);
+            # any other consumer of a step this long wants one bfloat16 result.
+            plan = self._wide_plan(m, n, k, not for_residual)
+            if self._wide_runs(m, n, k, "sums" if for_residual else "one", plan,
+                               lambda: self.gemm_wide(x, weight, bias, plan=plan),
+                               lambda: self._library_product(x, weight, bias, None)):
+                return self.gemm_wide(x, weight, bias, plan=plan)
         if for_residual and self.library_residual_float32:
             out = self._library_product(x, weight, None, torch.float32)
             if bias is not None:

@@ -295,8 +295,8 @@ int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long
 // [splits, m, n]; mode 2: out = bfloat16 [m, n / 2] = silu(gate) * up for a w whose rows alternate
 // gate, up (splits 1, no bias, n even).  iters_per_split iterations of 64 of k go to each of
 // `splits` = ceil(ceil(k / 64) / iters_per_split) ranges.  tile: 2, 4, 5 or (with 8 wavefronts and 256 activation rows) 8 (64, 128, 160 or 256
-// weight rows a workgroup); x_rows: 128 or 256 activation rows a workgroup; waves: 4 or 8 wavefronts a
-// workgroup (two, or four, along the activation rows).
+// weight rows a workgroup); x_rows: 128 or 256 (with 8 wavefronts also 64) activation rows a workgroup; waves: 4 or 8
+// wavefronts a workgroup (two, or four, along the activation rows).
 extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_stride, const void* w, const void* bias,
                             int m, int n, int k, int iters_per_split, int splits, int tile, int x_rows, int waves,
                             int mode, hipStream_t stream) {
@@ -322,10 +322,16 @@ extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_str
     if (tile == 2) TS_WIDE(2, 8, 2);
     if (tile == 4) TS_WIDE(4, 8, 2);
     if (tile == 5) TS_WIDE(5, 8, 2);
+  } else if (waves == 8 && x_rows == 64) {
+    if (tile == 2) TS_WIDE(2, 1, 4);
+    if (tile == 4) TS_WIDE(4, 1, 4);
+    if (tile == 5) TS_WIDE(5, 1, 4);
+    if (tile == 8) TS_WIDE(8, 1, 4);
   } else if (waves == 8 && x_rows == 128) {
     if (tile == 2) TS_WIDE(2, 2, 4);
     if (tile == 4) TS_WIDE(4, 2, 4);
     if (tile == 5) TS_WIDE(5, 2, 4);
+    if (tile == 8) TS_WIDE(8, 2, 4);
   } else if (waves == 8 && x_rows == 256) {
     if (tile == 2) TS_WIDE(2, 4, 4);
     if (tile == 4) TS_WIDE(4, 4, 4);

@@ -894,11 +894,11 @@ class Ops:
         return self.wide_choices[key]
 
     def gemm_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
-                  plan: tuple[int, int, int, int, int], gated: bool = False) -> torch.Tensor:
+                  plan: tuple[int, int, int, int, int], gated: bool = False, sums: bool = False) -> torch.Tensor:
         """``x [M, K] @ weight [N, K]^T (+ bias)`` by the LDS-tiled kernel for steps of many rows
         (``csrc/gemm_wide.hip``): any M, K a multiple of 8.  ``plan`` = (iterations of 64 per range
-        of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup).  One range: bfloat16 ``[M, N]``; several:
-        32-bit partial sums ``[S, M, N]`` (bias in the first).  ``gated``: the weight is a gate|up
+        of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup).  One range: bfloat16 ``[M, N]``; several
+        (or, with ``sums``, one as well): 32-bit partial sums ``[S, M, N]`` (bias in the first).  ``gated``: the weight is a gate|up
         projection whose rows alternate gate, up, and the result is ``silu(gate) * up`` as
         bfloat16 ``[M, N / 2]`` (one range of K, no bias)."""
         _gpu(x, weight, bias)
@@ -919,7 +919,7 @@ class Ops:
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k, per_split, splits,
                                           tile, x_rows, waves, 2, self.stream()), "ts_gemm_wide")
             return out
-        if splits == 1:
+        if splits == 1 and not sums:
             out = self.rows_buffer(m, n, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
                                           splits, tile, x_rows, waves, 0, self.stream()), "ts_gemm_wide")
@@ -957,9 +957,36 @@ class Ops:
         K (bias in the first); their sum over ``S`` is the product.  For decode-sized ``M``: the
         tiled kernel, except for up to 16 rows against a small matrix (the resident kernel's
         many small workgroups start faster)."""
-        if self._resident_runs(x.shape[0], weight.shape[0], weight.shape[1]):
+        m, (n, k) = x.shape[0], weight.shape
+        if self._resident_runs(m, n, k):
             return self.gemm_resident(x, weight, bias, max_splits=max_splits)
+        if self._few_rows_wide(m, n, k, max_splits):
+            return self.gemm_wide(x, weight, bias, plan=self._wide_plan_few_rows(m, n, k, max_splits), sums=True)
         return self.gemm_tiled(x, weight, bias, max_splits=max_splits)
+
+    def _few_rows_wide(self, m: int, n: int, k: int, max_splits: int | None) -> bool:
+        """Whether a decode-sized product runs the kernel of the steps of many rows
+        (``gemm_wide``: eight wavefronts, an iteration's staging between the halves of the one
+        before's products) instead of the tiled one: above 64 rows always (7B shape at 128 rows,
+        alone: gate|up 59 against 72 us, down 35 against 39, q|k|v 14 against 16, the head 246
+        against 282), from 33 rows for the small matrices and the head (q|k|v at 64 rows 11.0
+        against 14.6 us, the head 206 against 221)."""
+        if m > 64:
+            return True
+        return m > 32 and (2 * n * k < self.resident_small_bytes or (max_splits == 1 and n >= 128 * self.compute_units))
+
+    def _wide_plan_few_rows(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int, int, int]:
+        """The wide product's grid for up to 128 rows, where reading the weights sets the pace: one
+        tile of 64 or 128 activation rows, tiles of 160 weight rows if those alone give nearly every
+        compute unit a workgroup (one range of K), else tiles of 128 and as many ranges of K as it
+        takes to give every compute unit one."""
+        x_rows = 64 if m <= 64 else 128
+        iters = -(-k // 64)
+        if 10 * -(-n // 160) >= 9 * self.compute_units:
+            return iters, 1, 5, x_rows, 8
+        want = max(1, min(iters, max_splits or iters, self.compute_units // -(-n // 128)))
+        per_split = -(-iters // want)
+        return per_split, -(-iters // per_split), 4, x_rows, 8
 
     def _resident_runs(self, m: int, n: int, k: int) -> bool:
         """Whether the resident kernel, not the tiled one, runs a decode-sized product: small
@@ -1058,6 +1085,10 @@ class Ops:
         case is the projection followed by :meth:`swiglu`."""
         if x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             _gpu(x, weight)
+            if (self._few_rows_wide(x.shape[0], weight.shape[0], weight.shape[1], None) and weight.shape[0] % 2 == 0
+                    and weight.is_contiguous() and x.stride(1) == 1):
+                wide = self._wide_plan_few_rows(x.shape[0], weight.shape[0], weight.shape[1], 1)
+                return self.gemm_wide(x, weight, plan=wide, gated=True)
             plan = self._tiled_plan(x.shape[0], weight.shape[0], weight.shape[1], None)
             if plan[1] == 1 and weight.shape[0] % 2 == 0 and weight.is_contiguous() and x.stride(1) == 1:
                 return self.gemm_tiled(x, weight, plan=plan, gated=True)

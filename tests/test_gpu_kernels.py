@@ -245,6 +245,37 @@ def test_gemm_wide_every_tile_and_grid(ops, tile, x_rows, waves, m, n, k):
             x.to(DEV), w.to(DEV), b.to(DEV), plan=(iters, 1, tile, x_rows, waves), gated=True)
 
 
+@pytest.mark.parametrize("tile,x_rows,depth", [(2, 64, 64), (4, 64, 64), (5, 64, 64), (8, 64, 64), (2, 64, 128), (4, 64, 128),
+                                                (5, 64, 128), (8, 128, 64)])
+@pytest.mark.parametrize("m,n,k", [(40, 97, 72), (64, 500, 200), (33, 322, 1096), (17, 1000, 40), (100, 161, 264)])
+def test_gemm_wide_at_decode_sizes(ops, tile, x_rows, depth, m, n, k):
+    """The same kernel as the product of decode steps of 17 to 128 rows: tiles of 64 activation
+    rows, iterations 64 and 128 deep, always partial sums out (or the SwiGLU), against the exact
+    product; and `gemm_skinny` / `linear_swiglu`, which pick it for these row counts."""
+    if m > x_rows:
+        pytest.skip("one tile of activation rows here")
+    g = torch.Generator().manual_seed(tile * 100 + n + depth)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    b = torch.randn(n, generator=g).bfloat16()
+    want = x.double() @ w.double().T + b.double()
+    iters = -(-k // depth)
+    for per_split in sorted({1, iters}):
+        splits = -(-iters // per_split)
+        partial = ops.gemm_wide(x.to(DEV), w.to(DEV), b.to(DEV), plan=(per_split, splits, tile, x_rows, 8, depth), sums=True)
+        assert partial.shape == (splits, m, n) and partial.dtype == torch.float32
+        assert float((partial.double().sum(0).cpu() - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1)
+    picked = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert float((picked.double().sum(0).cpu() - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1)
+    if n % 2 == 0:
+        y = x.double() @ w.double().T
+        gated = torch.nn.functional.silu(y[:, 0::2]) * y[:, 1::2]
+        fused = ops.gemm_wide(x.to(DEV), w.to(DEV), plan=(iters, 1, tile, x_rows, 8, depth), gated=True)
+        assert float((fused.double().cpu() - gated).abs().max()) <= 1e-2 * float(gated.abs().max() + 1)
+        either = ops.linear_swiglu(x.to(DEV), w.to(DEV))
+        assert float((either.double().cpu() - gated).abs().max()) <= 1e-2 * float(gated.abs().max() + 1)
+
+
 def test_gemm_wide_rows_do_not_depend_on_the_batch_and_plans_fill_the_device(ops):
     """A row's result is the same bits whatever rows stand beside it (for one grid), rows behind
     the step's own reach nothing, and the planner's grids for the 7B shape's matrices give most

@@ -31,18 +31,19 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int W_DEPTH = 64;              // k per iteration
-constexpr int W_LDS_ROW = W_DEPTH + 8;   // LDS row stride in elements
-constexpr int W_ROW_PIECES = W_DEPTH / 8;  // 16-byte pieces of a row of an iteration
 constexpr int DIES = 8;
 
 __device__ __forceinline__ bf16x8 wide_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-// WM: wavefronts along the activation rows (the workgroup has 2 WM wavefronts).
-template <int TN, int MB, int WM>
+// WM: wavefronts along the activation rows (the workgroup has 2 WM wavefronts).  DP: k per
+// iteration, 64, or 128 for tiles small enough that two buffers still fit LDS (the iterations of
+// a few activation rows hold little work, and half as many barriers tell).
+template <int TN, int MB, int WM, int DP>
 struct WideRegs {
   static constexpr int THREADS = 2 * WM * TS_WAVE;
-  static constexpr int PIECE_ROWS = THREADS / W_ROW_PIECES;  // rows one pass of the threads covers: 32 or 64
+  static constexpr int LDS_ROW = DP + 8;      // LDS row stride in elements
+  static constexpr int ROW_PIECES = DP / 8;   // 16-byte pieces of a row of an iteration
+  static constexpr int PIECE_ROWS = THREADS / ROW_PIECES;  // rows one pass of the threads covers
   static constexpr int NT = 32 * TN;
   static constexpr int XROWS = 16 * WM * MB;
   static constexpr int W_PIECES = (NT + PIECE_ROWS - 1) / PIECE_ROWS;
@@ -53,15 +54,18 @@ struct WideRegs {
 };
 
 // out: bfloat16 [m, n] (mode 0), partial: float [splits, m, n] (mode 1), out: bfloat16 [m, n / 2] (mode 2).
-template <int TN, int MB, int WM, int MODE, bool ONCE>
+template <int TN, int MB, int WM, int DP, int MODE, bool ONCE>
 __global__ void __launch_bounds__(2 * WM * TS_WAVE)
 gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const uint16_t* __restrict__ x, long x_stride,
                  const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
                  int iters_per_split, int splits, int n_tiles, int m_tiles) {
-  typedef WideRegs<TN, MB, WM> Regs;
+  typedef WideRegs<TN, MB, WM, DP> Regs;
   constexpr int NT = Regs::NT;
   constexpr int XROWS = Regs::XROWS;
   constexpr int W_PIECE_ROWS = Regs::PIECE_ROWS;
+  constexpr int W_DEPTH = DP;
+  constexpr int W_LDS_ROW = Regs::LDS_ROW;
+  constexpr int W_ROW_PIECES = Regs::ROW_PIECES;
   constexpr int STAGE = (NT + XROWS) * W_LDS_ROW;  // elements of one LDS buffer: weight rows, then activation rows
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [2][STAGE]
   // Workgroup id -> (weight tile and range of K, tile of activation rows): see the head of the file.
@@ -154,7 +158,7 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
         for (int b = 0; b < MB; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wide_bf16x8(wf), wide_bf16x8(xf[b]), acc[a][b], 0, 0, 0);
       }
-      if (step == 0) stage(next, buf ^ 1, it_next);
+      if (step == W_DEPTH / 64 - 1) stage(next, buf ^ 1, it_next);  // between the halves
     }
 #ifndef TS_WIDE_NO_SCHED
     // Order asked of the scheduler for the round (one basic block: the loads of the iteration
@@ -246,16 +250,16 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
   }
 }
 
-template <int TN, int MB, int WM, int MODE, bool ONCE>
+template <int TN, int MB, int WM, int DP, int MODE, bool ONCE>
 int launch_wide_kernel(float* partial, uint16_t* out, const uint16_t* x, long x_stride, const uint16_t* w,
                        const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
-  typedef WideRegs<TN, MB, WM> Regs;
-  constexpr size_t lds_bytes = (size_t)2 * (Regs::NT + Regs::XROWS) * W_LDS_ROW * sizeof(uint16_t);
+  typedef WideRegs<TN, MB, WM, DP> Regs;
+  constexpr size_t lds_bytes = (size_t)2 * (Regs::NT + Regs::XROWS) * Regs::LDS_ROW * sizeof(uint16_t);
   static_assert(lds_bytes <= 160 * 1024, "two buffers must fit the LDS of a compute unit");
   if (lds_bytes > 48 * 1024) {
     static bool raised = false;  // per process; the attribute belongs to the kernel
     if (!raised) {
-      if (hipFuncSetAttribute((const void*)gemm_wide_kernel<TN, MB, WM, MODE, ONCE>,
+      if (hipFuncSetAttribute((const void*)gemm_wide_kernel<TN, MB, WM, DP, MODE, ONCE>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
         return TS_ERR_LAUNCH;
       raised = true;
@@ -266,21 +270,21 @@ int launch_wide_kernel(float* partial, uint16_t* out, const uint16_t* x, long x_
   const long units = (long)n_tiles * splits;
   const long ids = ((units + DIES - 1) / DIES) * DIES * m_tiles;
   if (ids > 0x7fffffffL) return TS_ERR_SHAPE;
-  hipLaunchKernelGGL((gemm_wide_kernel<TN, MB, WM, MODE, ONCE>), dim3((unsigned)ids), dim3(Regs::THREADS), lds_bytes,
+  hipLaunchKernelGGL((gemm_wide_kernel<TN, MB, WM, DP, MODE, ONCE>), dim3((unsigned)ids), dim3(Regs::THREADS), lds_bytes,
                      stream, partial, out, x, x_stride, w, bias, m, n, k, iters_per_split, splits, n_tiles, m_tiles);
   return ts_launch_status();
 }
 
-template <int TN, int MB, int WM>
+template <int TN, int MB, int WM, int DP>
 int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long x_stride, const uint16_t* w,
                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
   // One tile of activation rows: every weight is read once, with non-temporal loads; more: the
   // tiles over a weight tile share it through their die's L2.
-  const bool once = m <= WideRegs<TN, MB, WM>::XROWS;
+  const bool once = m <= WideRegs<TN, MB, WM, DP>::XROWS;
 #define TS_WIDE_MODE(MODE)                                                                                            \
-  return once ? launch_wide_kernel<TN, MB, WM, MODE, true>(partial, out, x, x_stride, w, bias, m, n, k,              \
+  return once ? launch_wide_kernel<TN, MB, WM, DP, MODE, true>(partial, out, x, x_stride, w, bias, m, n, k,              \
                                                            iters_per_split, splits, stream)                           \
-              : launch_wide_kernel<TN, MB, WM, MODE, false>(partial, out, x, x_stride, w, bias, m, n, k,             \
+              : launch_wide_kernel<TN, MB, WM, DP, MODE, false>(partial, out, x, x_stride, w, bias, m, n, k,             \
                                                             iters_per_split, splits, stream)
   if (mode == 0) TS_WIDE_MODE(0);
   if (mode == 1) TS_WIDE_MODE(1);
@@ -293,18 +297,20 @@ int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long
 // x [m, k] bfloat16 with row stride x_stride; w [n, k] bfloat16 contiguous; bias [n] bfloat16 or
 // null; k % 8 == 0.  mode 0: out = bfloat16 [m, n] (splits must be 1); mode 1: partial = float
 // [splits, m, n]; mode 2: out = bfloat16 [m, n / 2] = silu(gate) * up for a w whose rows alternate
-// gate, up (splits 1, no bias, n even).  iters_per_split iterations of 64 of k go to each of
-// `splits` = ceil(ceil(k / 64) / iters_per_split) ranges.  tile: 2, 4, 5 or (with 8 wavefronts and 256 activation rows) 8 (64, 128, 160 or 256
+// gate, up (splits 1, no bias, n even).  depth: k per iteration, 64 or (tiles of 64 activation rows
+// only) 128; iters_per_split iterations of `depth` of k go to each of `splits` =
+// ceil(ceil(k / depth) / iters_per_split) ranges.  tile: 2, 4, 5 or (with 8 wavefronts and 256 activation rows) 8 (64, 128, 160 or 256
 // weight rows a workgroup); x_rows: 128 or 256 (with 8 wavefronts also 64) activation rows a workgroup; waves: 4 or 8
 // wavefronts a workgroup (two, or four, along the activation rows).
 extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_stride, const void* w, const void* bias,
                             int m, int n, int k, int iters_per_split, int splits, int tile, int x_rows, int waves,
-                            int mode, hipStream_t stream) {
+                            int depth, int mode, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || mode < 0 || mode > 2) return TS_ERR_ARG;
   if ((mode == 1) != (partial != nullptr) || (mode != 1) != (out != nullptr)) return TS_ERR_ARG;
   if ((k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
-  const int total = (k + W_DEPTH - 1) / W_DEPTH;
+  if (depth != 64 && depth != 128) return TS_ERR_SHAPE;
+  const int total = (k + depth - 1) / depth;
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split) return TS_ERR_SHAPE;
   if (mode != 1 && splits != 1) return TS_ERR_ARG;
   if (mode == 2 && (bias || (n & 1) != 0)) return TS_ERR_ARG;
@@ -312,31 +318,39 @@ extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_str
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-#define TS_WIDE(TN, MB, WM) \
-  return launch_wide<TN, MB, WM>(mode, partial, op, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream)
+#define TS_WIDE(TN, MB, WM, DP) \
+  return launch_wide<TN, MB, WM, DP>(mode, partial, op, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream)
+  if (depth == 128) {  // tiles of 64 activation rows, eight wavefronts
+    if (waves == 8 && x_rows == 64) {
+      if (tile == 2) TS_WIDE(2, 1, 4, 128);
+      if (tile == 4) TS_WIDE(4, 1, 4, 128);
+      if (tile == 5) TS_WIDE(5, 1, 4, 128);
+    }
+    return TS_ERR_SHAPE;
+  }
   if (waves == 4 && x_rows == 128) {
-    if (tile == 2) TS_WIDE(2, 4, 2);
-    if (tile == 4) TS_WIDE(4, 4, 2);
-    if (tile == 5) TS_WIDE(5, 4, 2);
+    if (tile == 2) TS_WIDE(2, 4, 2, 64);
+    if (tile == 4) TS_WIDE(4, 4, 2, 64);
+    if (tile == 5) TS_WIDE(5, 4, 2, 64);
   } else if (waves == 4 && x_rows == 256) {
-    if (tile == 2) TS_WIDE(2, 8, 2);
-    if (tile == 4) TS_WIDE(4, 8, 2);
-    if (tile == 5) TS_WIDE(5, 8, 2);
+    if (tile == 2) TS_WIDE(2, 8, 2, 64);
+    if (tile == 4) TS_WIDE(4, 8, 2, 64);
+    if (tile == 5) TS_WIDE(5, 8, 2, 64);
   } else if (waves == 8 && x_rows == 64) {
-    if (tile == 2) TS_WIDE(2, 1, 4);
-    if (tile == 4) TS_WIDE(4, 1, 4);
-    if (tile == 5) TS_WIDE(5, 1, 4);
-    if (tile == 8) TS_WIDE(8, 1, 4);
+    if (tile == 2) TS_WIDE(2, 1, 4, 64);
+    if (tile == 4) TS_WIDE(4, 1, 4, 64);
+    if (tile == 5) TS_WIDE(5, 1, 4, 64);
+    if (tile == 8) TS_WIDE(8, 1, 4, 64);
   } else if (waves == 8 && x_rows == 128) {
-    if (tile == 2) TS_WIDE(2, 2, 4);
-    if (tile == 4) TS_WIDE(4, 2, 4);
-    if (tile == 5) TS_WIDE(5, 2, 4);
-    if (tile == 8) TS_WIDE(8, 2, 4);
+    if (tile == 2) TS_WIDE(2, 2, 4, 64);
+    if (tile == 4) TS_WIDE(4, 2, 4, 64);
+    if (tile == 5) TS_WIDE(5, 2, 4, 64);
+    if (tile == 8) TS_WIDE(8, 2, 4, 64);
   } else if (waves == 8 && x_rows == 256) {
-    if (tile == 2) TS_WIDE(2, 4, 4);
-    if (tile == 4) TS_WIDE(4, 4, 4);
-    if (tile == 5) TS_WIDE(5, 4, 4);
-    if (tile == 8) TS_WIDE(8, 4, 4);
+    if (tile == 2) TS_WIDE(2, 4, 4, 64);
+    if (tile == 4) TS_WIDE(4, 4, 4, 64);
+    if (tile == 5) TS_WIDE(5, 4, 4, 64);
+    if (tile == 8) TS_WIDE(8, 4, 4, 64);
   }
 #undef TS_WIDE
   return TS_ERR_SHAPE;

@@ -56,7 +56,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
         "ts_gemm_wide": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_void_p],
+                         c_int, c_int, c_int, c_int, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -896,8 +896,8 @@ class Ops:
     def gemm_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
                   plan: tuple[int, int, int, int, int], gated: bool = False, sums: bool = False) -> torch.Tensor:
         """``x [M, K] @ weight [N, K]^T (+ bias)`` by the LDS-tiled kernel for steps of many rows
-        (``csrc/gemm_wide.hip``): any M, K a multiple of 8.  ``plan`` = (iterations of 64 per range
-        of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup).  One range: bfloat16 ``[M, N]``; several
+        (``csrc/gemm_wide.hip``): any M, K a multiple of 8.  ``plan`` = (iterations per range
+        of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup[, k per iteration: 64 (the default) or 128]).  One range: bfloat16 ``[M, N]``; several
         (or, with ``sums``, one as well): 32-bit partial sums ``[S, M, N]`` (bias in the first).  ``gated``: the weight is a gate|up
         projection whose rows alternate gate, up, and the result is ``silu(gate) * up`` as
         bfloat16 ``[M, N / 2]`` (one range of K, no bias)."""
@@ -910,23 +910,24 @@ class Ops:
         n = weight.shape[0]
         if bias is not None:
             _need(bias.shape == (n,) and bias.dtype == torch.bfloat16 and bias.is_contiguous(), "bias must be bfloat16 [N]")
-        per_split, splits, tile, x_rows, waves = plan
+        per_split, splits, tile, x_rows, waves = plan[:5]
+        depth = plan[5] if len(plan) > 5 else 64
         x_stride = x.stride(0) if m > 1 else max(k, x.stride(0))
         if gated:
             _need(splits == 1 and bias is None and n % 2 == 0,
                   "the gated result needs one range of K, no bias and an even number of weight rows")
             out = self.rows_buffer(m, n // 2, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k, per_split, splits,
-                                          tile, x_rows, waves, 2, self.stream()), "ts_gemm_wide")
+                                          tile, x_rows, waves, depth, 2, self.stream()), "ts_gemm_wide")
             return out
         if splits == 1 and not sums:
             out = self.rows_buffer(m, n, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                          splits, tile, x_rows, waves, 0, self.stream()), "ts_gemm_wide")
+                                          splits, tile, x_rows, waves, depth, 0, self.stream()), "ts_gemm_wide")
             return out
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_wide(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                      splits, tile, x_rows, waves, 1, self.stream()), "ts_gemm_wide")
+                                      splits, tile, x_rows, waves, depth, 1, self.stream()), "ts_gemm_wide")
         return partial
 
     def gemm_resident(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
@@ -967,26 +968,30 @@ class Ops:
     def _few_rows_wide(self, m: int, n: int, k: int, max_splits: int | None) -> bool:
         """Whether a decode-sized product runs the kernel of the steps of many rows
         (``gemm_wide``: eight wavefronts, an iteration's staging between the halves of the one
-        before's products) instead of the tiled one: above 64 rows always (7B shape at 128 rows,
-        alone: gate|up 59 against 72 us, down 35 against 39, q|k|v 14 against 16, the head 246
-        against 282), from 33 rows for the small matrices and the head (q|k|v at 64 rows 11.0
-        against 14.6 us, the head 206 against 221)."""
-        if m > 64:
+        before's products) instead of the tiled one: above 32 rows always (7B shape, alone, at 64
+        rows: gate|up 46.7 against 50.1 us, down 27.6 against 29.3, q|k|v 10.7 against 14.4, o 9.5
+        against 10.6, the head 209 against 221; at 128 rows: 59 against 72, 35 against 39, 14
+        against 16, 246 against 282), from 17 rows for a matrix that fills the device as one range
+        of K and once over (gate|up at 32 rows: 45.3 against 47.8 us)."""
+        if m > 32:
             return True
-        return m > 32 and (2 * n * k < self.resident_small_bytes or (max_splits == 1 and n >= 128 * self.compute_units))
+        tiles = -(-n // 160)
+        return m > 16 and max_splits == 1 and 9 * self.compute_units <= 10 * tiles <= 20 * self.compute_units
 
-    def _wide_plan_few_rows(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int, int, int]:
+    def _wide_plan_few_rows(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int, int, int, int]:
         """The wide product's grid for up to 128 rows, where reading the weights sets the pace: one
-        tile of 64 or 128 activation rows, tiles of 160 weight rows if those alone give nearly every
-        compute unit a workgroup (one range of K), else tiles of 128 and as many ranges of K as it
-        takes to give every compute unit one."""
+        tile of 64 or 128 activation rows; iterations 128 deep under the tiles of 64 rows (half as
+        many barriers; the head, whose grid runs in several rounds, is faster 64 deep); tiles of
+        160 weight rows if those alone give nearly every compute unit a workgroup (one range of
+        K), else tiles of 128 and as many ranges of K as it takes to give every compute unit one."""
         x_rows = 64 if m <= 64 else 128
-        iters = -(-k // 64)
+        depth = 128 if x_rows == 64 and -(-n // 160) <= 2 * self.compute_units else 64
+        iters = -(-k // depth)
         if 10 * -(-n // 160) >= 9 * self.compute_units:
-            return iters, 1, 5, x_rows, 8
+            return iters, 1, 5, x_rows, 8, depth
         want = max(1, min(iters, max_splits or iters, self.compute_units // -(-n // 128)))
         per_split = -(-iters // want)
-        return per_split, -(-iters // per_split), 4, x_rows, 8
+        return per_split, -(-iters // per_split), 4, x_rows, 8, depth
 
     def _resident_runs(self, m: int, n: int, k: int) -> bool:
         """Whether the resident kernel, not the tiled one, runs a decode-sized product: small
@@ -1085,7 +1090,7 @@ class Ops:
         case is the projection followed by :meth:`swiglu`."""
         if x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             _gpu(x, weight)
-            if (self._few_rows_wide(x.shape[0], weight.shape[0], weight.shape[1], None) and weight.shape[0] % 2 == 0
+            if (self._few_rows_wide(x.shape[0], weight.shape[0], weight.shape[1], 1) and weight.shape[0] % 2 == 0
                     and weight.is_contiguous() and x.stride(1) == 1):
                 wide = self._wide_plan_few_rows(x.shape[0], weight.shape[0], weight.shape[1], 1)
                 return self.gemm_wide(x, weight, plan=wide, gated=True)

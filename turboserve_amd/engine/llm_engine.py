@@ -161,15 +161,23 @@ class LLMEngine:
             sizes.update(size for size in ops.library_buckets if size > ops.skinny_max_rows)
         started = time.perf_counter()
         ops = self.model.runtime.ops
-        with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
-            # Inside, every product of more rows than a decode step has runs both ways once, by the
-            # library's best kernel and by this engine's own, and the faster one is kept.
-            ops.time_wide_choices = True
-            try:
+        own_rows = ops.wide_default_rows
+        try:
+            # First the library's kernels for every product (this engine's own product for steps of
+            # many rows stands aside meanwhile) ...
+            ops.wide_default_rows = 0
+            with LibraryGemmTuning(self.config.gemm_tuning_file) as tuning:
                 for tokens in sorted(sizes):
                     self.runner.dry_run(tokens)
-            finally:
-                ops.time_wide_choices = False
+            # ... then, with the library's winners in use and its timing mode off, every such
+            # product runs both ways, by the library and by this engine's own kernel, and the
+            # faster one is kept (``Ops.wide_choices``).
+            ops.time_wide_choices = True
+            for tokens in sorted(sizes):
+                self.runner.dry_run(tokens)
+        finally:
+            ops.time_wide_choices = False
+            ops.wide_default_rows = own_rows
         logger.info("library products timed for steps of %s tokens in %.1f s (%d choices kept in %s)",
                     sorted(sizes), time.perf_counter() - started, tuning.num_results(), tuning.results_file)
 

@@ -275,6 +275,8 @@ class Ops:
         #: (rows a step's products run at, N, K, kind) -> whether this engine's own product was the
         #: faster one when both were timed (``time_wide_choices``).
         self.wide_choices: dict[tuple, bool] = {}
+        #: The same keys -> (milliseconds of the own product, of the library's) as timed.
+        self.wide_timings: dict[tuple, tuple[float, float]] = {}
         #: While true, a product of many rows whose choice is not known yet runs both ways, timed.
         self.time_wide_choices = False
         #: Compute units of the device (256 on an MI355X): the launch plans below size their grids by it.
@@ -870,8 +872,8 @@ class Ops:
         a product of ``rows`` rows (more than the decode products take): what a timing found, or,
         untimed, up to ``wide_default_rows`` rows if the grid gives at least half of the compute
         units a workgroup.  With ``time_wide_choices`` an unknown product that is worth timing
-        runs both ways here (``own()`` and ``library()``), three times each behind a warm-up, by
-        device events."""
+        runs both ways here (``own()`` and ``library()``), four launches each behind a warm-up, each
+        waited for, the best by device events."""
         key = (self.library_rows(rows), n, k, kind)
         known = self.wide_choices.get(key)
         if known is not None:
@@ -879,18 +881,25 @@ class Ops:
         if not self.time_wide_choices or rows * n * k < self.library_tuning_min_work:
             workgroups = -(-n // (32 * plan[2])) * -(-rows // plan[3]) * plan[1]
             return rows <= self.wide_default_rows and (2 * workgroups >= self.compute_units or rows * n * k < self.library_tuning_min_work)
+        # One launch at a time, each waited for: launches that follow one another without a
+        # dependency overlap where a grid leaves compute units idle, and would look faster than
+        # they are inside a step.
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         times = []
         for run in (own, library):
             run()
             run()
-            start.record()
-            for _ in range(3):
+            best = float("inf")
+            for _ in range(4):
+                torch.cuda.synchronize(self.device)
+                start.record()
                 run()
-            stop.record()
-            stop.synchronize()
-            times.append(start.elapsed_time(stop))
+                stop.record()
+                stop.synchronize()
+                best = min(best, start.elapsed_time(stop))
+            times.append(best)
         self.wide_choices[key] = times[0] <= times[1]
+        self.wide_timings[key] = (times[0], times[1])
         return self.wide_choices[key]
 
     def gemm_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,

@@ -1,10 +1,11 @@
-"""Host models of the addresses three kernels form, checked against their buffers' bounds.
+"""Host models of the addresses four kernels form, checked against their buffers' bounds.
 
 A wild address on the GPU can end more than the test that made it, so the index arithmetic of
 the kernels whose launches the host plans most freely is restated here in Python and swept
 over shapes, plans and cache states on the CPU: the tiled product (``csrc/gemm_tiled.hip``:
 what a thread fetches, where it stages it in LDS, which fragments a wavefront reads, where the
-sums go), the decode attention (``csrc/attention_mfma.hip``, ``decode_kernel``: which page and
+sums go), the product of steps of many rows (``csrc/gemm_wide.hip``: the same, with its
+numbering of workgroups over weight tiles, ranges of K and tiles of activation rows), the decode attention (``csrc/attention_mfma.hip``, ``decode_kernel``: which page and
 key every lane reads for every split, with pages given back below a window and table entries
 that are padding) and the 32-row prefill attention (``prefill_wide_kernel``: the block-table
 look-ups of its pipeline, five windows ahead, self-fed and fed, whole blocks and shares of a
@@ -278,3 +279,104 @@ def test_prefill_attention_looks_up_live_pages_only():
         for row, rows, first_slot, shares in combine:
             assert 0 <= row and row + rows <= count and 0 <= first_slot and first_slot + shares <= slots
             assert set(range(first_slot, first_slot + shares)) <= seen
+
+
+def check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, mode, x_stride):
+    """``gemm_wide_kernel`` (``csrc/gemm_wide.hip``): the workgroup numbering covers every (weight
+    tile, range of K, tile of activation rows) exactly once, and every address a thread forms,
+    in global memory and in LDS, lies inside its buffer."""
+    wm = waves // 2
+    threads = 64 * waves
+    lds_row, row_pieces = depth + 8, depth // 8
+    piece_rows = threads // row_pieces
+    nt = 32 * tile
+    mb = x_rows // (16 * wm)
+    assert mb >= 1 and 16 * wm * mb == x_rows and x_rows % piece_rows == 0
+    w_pieces, x_pieces = -(-nt // piece_rows), x_rows // piece_rows
+    stage = (nt + x_rows) * lds_row
+    assert 2 * stage * 2 <= 160 * 1024
+    n_tiles, m_tiles = -(-n // nt), -(-m // x_rows)
+    units = n_tiles * splits
+    ids = -(-units // 8) * 8 * m_tiles
+    total = -(-k // depth)
+    x_size = (m - 1) * x_stride + k
+    seen = set()
+    for block in range(ids):
+        die, turn = block % 8, block // 8
+        m_tile, unit = turn % m_tiles, (turn // m_tiles) * 8 + die
+        if unit >= units:
+            continue
+        assert (unit, m_tile) not in seen
+        seen.add((unit, m_tile))
+    assert len(seen) == units * m_tiles
+    for unit, m_tile in sorted({(0, 0), (units - 1, m_tiles - 1), (units // 2, m_tiles // 2)}):
+        n_base, split, m_base = (unit % n_tiles) * nt, unit // n_tiles, m_tile * x_rows
+        first = split * per_split
+        last = min(first + per_split, total)
+        if first >= last:
+            continue
+        for tid in range(threads):
+            piece_k, piece_row = 8 * (tid % row_pieces), tid // row_pieces
+            for it in sorted({first, last - 1, last, last + 2}):  # loads are issued up to three iterations past the range
+                k0 = min(min(it, last - 1) * depth + piece_k, k - 8)
+                assert k0 >= 0
+                for i in range(w_pieces):
+                    at = min(n_base + min(piece_row + piece_rows * i, nt - 1), n - 1) * k + k0
+                    assert 0 <= at and at + 8 <= n * k
+                for i in range(x_pieces):
+                    at = min(m_base + piece_row + piece_rows * i, m - 1) * x_stride + k0
+                    assert 0 <= at and at + 8 <= x_size
+            dst = piece_row * lds_row + piece_k
+            for buf in (0, 1):
+                for i in range(x_pieces):
+                    at = buf * stage + dst + (nt + piece_rows * i) * lds_row
+                    assert buf * stage + nt * lds_row <= at and at + 8 <= (buf + 1) * stage
+                for i in range(w_pieces):
+                    if nt % piece_rows == 0 or piece_row + piece_rows * i < nt:
+                        at = buf * stage + dst + piece_rows * i * lds_row
+                        assert buf * stage <= at and at + 8 <= buf * stage + nt * lds_row
+            lane, wave = tid % 64, tid // 64
+            lane16, group, wave_n, wave_m = lane % 16, lane // 16, wave // wm, wave % wm
+            base = lane16 * lds_row + 8 * group
+            for step in range(depth // 32):
+                for b in range(mb):
+                    at = base + (nt + 16 * mb * wave_m + 16 * b) * lds_row + 32 * step
+                    assert nt * lds_row <= at and at + 8 <= stage
+                for a in range(tile):
+                    assert base + (wave_n * tile + a) * 16 * lds_row + 32 * step + 8 <= nt * lds_row
+            for a in range(tile):
+                nrow = n_base + (wave_n * tile + a) * 16 + 4 * group
+                if nrow >= n:
+                    continue
+                for b in range(mb):
+                    row = m_base + 16 * mb * wave_m + 16 * b + lane16
+                    if row >= m:
+                        continue
+                    if mode == 2:
+                        width = 2 if nrow + 3 < n else (1 if nrow + 1 < n else 0)
+                        assert row * (n // 2) + nrow // 2 + width <= m * (n // 2)
+                    elif mode == 1:
+                        width = 4 if (nrow + 3 < n and n % 4 == 0) else min(4, n - nrow)
+                        assert (split * m + row) * n + nrow + width <= splits * m * n
+                    else:
+                        width = 4 if (nrow + 3 < n and n % 4 == 0) else min(4, n - nrow)
+                        assert row * n + nrow + width <= m * n
+
+
+WIDE_SHAPES = [(2, 128, 4, 64), (5, 256, 4, 64), (4, 128, 8, 64), (5, 128, 8, 64), (2, 256, 8, 64), (5, 256, 8, 64), (8, 256, 8, 64),
+               (8, 128, 8, 64), (2, 64, 8, 64), (5, 64, 8, 64), (8, 64, 8, 64), (2, 64, 8, 128), (4, 64, 8, 128), (5, 64, 8, 128)]
+
+
+@pytest.mark.parametrize("tile,x_rows,waves,depth", WIDE_SHAPES)
+def test_wide_product_stays_inside_its_buffers(tile, x_rows, waves, depth):
+    rng = random.Random(tile * x_rows + depth)
+    for m, n, k in ((130, 97, 72), (300, 500, 200), (513, 640, 1096), (17, 1000, 40), (64, 161, 264), (257, 6, 16), (1, 48, 8)):
+        iters = -(-k // depth)
+        for want in sorted({1, 2, iters}):
+            per_split = -(-iters // min(want, iters))
+            splits = -(-iters // per_split)
+            check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, 1, k + 8 * rng.randint(0, 3))
+            if splits == 1:
+                check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, 0, k)
+                if n % 2 == 0:
+                    check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, 2, k)

@@ -287,8 +287,23 @@ def check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, mode, x_s
     in global memory and in LDS, lies inside its buffer."""
     wm = waves // 2
     threads = 64 * waves
-    lds_row, row_pieces = depth + 8, depth // 8
+    lds_row, row_pieces = depth, depth // 8  # rows are not padded: the pieces of a row are swizzled
     piece_rows = threads // row_pieces
+
+    def key(row):
+        return (row >> 1) & 7 if row_pieces == 8 else row & 15
+
+    def banks(element):  # the four 4-byte banks (of 64) a 16-byte piece at this element offset lies in
+        return {(element // 2 + i) % 64 for i in range(4)}
+
+    # sixteen lanes of a write (consecutive pieces of one or two rows) and of a read (one piece of
+    # sixteen consecutive rows) touch every bank at most once
+    for first in range(0, threads, 16):
+        touched = [banks((t // row_pieces) * lds_row + 8 * ((t % row_pieces) ^ key(t // row_pieces))) for t in range(first, first + 16)]
+        assert sum(len(b) for b in touched) == len(set().union(*touched)) == 64
+    for piece in range(row_pieces):
+        touched = [banks(r * lds_row + 8 * (piece ^ key(r))) for r in range(16)]
+        assert sum(len(b) for b in touched) == len(set().union(*touched)) == 64
     nt = 32 * tile
     mb = x_rows // (16 * wm)
     assert mb >= 1 and 16 * wm * mb == x_rows and x_rows % piece_rows == 0
@@ -326,7 +341,7 @@ def check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, mode, x_s
                 for i in range(x_pieces):
                     at = min(m_base + piece_row + piece_rows * i, m - 1) * x_stride + k0
                     assert 0 <= at and at + 8 <= x_size
-            dst = piece_row * lds_row + piece_k
+            dst = piece_row * lds_row + 8 * ((tid % row_pieces) ^ key(piece_row))
             for buf in (0, 1):
                 for i in range(x_pieces):
                     at = buf * stage + dst + (nt + piece_rows * i) * lds_row
@@ -337,13 +352,15 @@ def check_wide(m, n, k, tile, x_rows, waves, depth, per_split, splits, mode, x_s
                         assert buf * stage <= at and at + 8 <= buf * stage + nt * lds_row
             lane, wave = tid % 64, tid // 64
             lane16, group, wave_n, wave_m = lane % 16, lane // 16, wave // wm, wave % wm
-            base = lane16 * lds_row + 8 * group
+            base = lane16 * lds_row
             for step in range(depth // 32):
+                piece = 8 * ((4 * step + group) ^ key(lane16))
+                assert 0 <= piece and piece + 8 <= lds_row
                 for b in range(mb):
-                    at = base + (nt + 16 * mb * wave_m + 16 * b) * lds_row + 32 * step
+                    at = base + (nt + 16 * mb * wave_m + 16 * b) * lds_row + piece
                     assert nt * lds_row <= at and at + 8 <= stage
                 for a in range(tile):
-                    assert base + (wave_n * tile + a) * 16 * lds_row + 32 * step + 8 <= nt * lds_row
+                    assert base + (wave_n * tile + a) * 16 * lds_row + piece + 8 <= nt * lds_row
             for a in range(tile):
                 nrow = n_base + (wave_n * tile + a) * 16 + 4 * group
                 if nrow >= n:

@@ -6,7 +6,8 @@
 //   * a workgroup of 2 x WM wavefronts (WM = 2 or 4) owns NT = 32 TN weight rows (TN = 2, 4 or
 //     5) by XROWS = 16 WM MB activation rows (128 or 256) and one range of K, walked 64 deep: both
 //     operands travel global memory -> registers (16-byte pieces, eight consecutive threads a
-//     row's 128 bytes) -> LDS (two buffers, rows padded by 16 bytes) -> matrix cores.  The loads
+//     row's 128 bytes) -> LDS (two buffers, the pieces of a row swizzled against bank conflicts) ->
+//     matrix cores.  The loads
 //     of an iteration are issued two iterations ahead into one of two sets of registers, and an
 //     iteration's registers go to LDS between the two halves of the iteration before's products,
 //     so that a wavefront's LDS writes, LDS reads and matrix instructions overlap; every load is
@@ -41,7 +42,7 @@ __device__ __forceinline__ bf16x8 wide_bf16x8(u32x4 v) { return __builtin_bit_ca
 template <int TN, int MB, int WM, int DP>
 struct WideRegs {
   static constexpr int THREADS = 2 * WM * TS_WAVE;
-  static constexpr int LDS_ROW = DP + 8;      // LDS row stride in elements
+  static constexpr int LDS_ROW = DP;          // LDS row stride in elements: no padding, the pieces of a row are swizzled
   static constexpr int ROW_PIECES = DP / 8;   // 16-byte pieces of a row of an iteration
   static constexpr int PIECE_ROWS = THREADS / ROW_PIECES;  // rows one pass of the threads covers
   static constexpr int NT = 32 * TN;
@@ -102,7 +103,15 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
 #pragma unroll
   for (int i = 0; i < Regs::X_PIECES; ++i)
     xsrc[i] = x + (size_t)min(m_base + piece_row + W_PIECE_ROWS * i, m - 1) * x_stride;
-  const int dst = piece_row * W_LDS_ROW + piece_k;
+  // Where a piece lies in its LDS row: piece p of row r at p ^ key(r), key = (r / 2) % 8 for rows of
+  // eight pieces (128 bytes: two rows span the 64 banks) and r % 16 for rows of sixteen.  Sixteen
+  // lanes that write a row's (or two rows') consecutive pieces, and sixteen lanes that read the
+  // same piece of sixteen consecutive rows, then each touch every bank once; with padded rows
+  // instead the writes of neighbouring rows overlapped (a third of the LDS cycles of the 256 x 256
+  // tile were bank conflicts).  Tiles start at multiples of 16 rows, so a thread's key is constant.
+  auto swizzle_key = [](int row) { return W_ROW_PIECES == 8 ? (row >> 1) & 7 : row & 15; };
+  const int dst = piece_row * W_LDS_ROW + 8 * ((tid % W_ROW_PIECES) ^ swizzle_key(piece_row));
+  static_assert(W_PIECE_ROWS % 16 == 0 && NT % 16 == 0, "a thread's rows differ by multiples of 16");
 
   auto fetch = [&](Regs& r, int it) {
     const int k0 = min(min(it, last - 1) * W_DEPTH + piece_k, k - 8);
@@ -144,16 +153,18 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
   // The products of the iteration staged in buffer `buf`; between its two halves the registers
   // `next` (iteration `it_next`) go to the other buffer.
   auto multiply = [&](int buf, const Regs& next, int it_next) {
-    const uint16_t* base = lds + buf * STAGE + lane16 * W_LDS_ROW + 8 * group;
+    const uint16_t* base = lds + buf * STAGE + lane16 * W_LDS_ROW;
+    const int key = swizzle_key(lane16);
 #pragma unroll
     for (int step = 0; step < W_DEPTH / 32; ++step) {
+      const int piece = 8 * ((4 * step + group) ^ key);  // this lane's piece of the step, in every row it reads
       u32x4 xf[MB];
 #pragma unroll
       for (int b = 0; b < MB; ++b)
-        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 16 * MB * wave_m + 16 * b) * W_LDS_ROW + 32 * step);
+        xf[b] = *reinterpret_cast<const u32x4*>(base + (NT + 16 * MB * wave_m + 16 * b) * W_LDS_ROW + piece);
 #pragma unroll
       for (int a = 0; a < TN; ++a) {
-        const u32x4 wf = *reinterpret_cast<const u32x4*>(base + (wave_n * TN + a) * 16 * W_LDS_ROW + 32 * step);
+        const u32x4 wf = *reinterpret_cast<const u32x4*>(base + (wave_n * TN + a) * 16 * W_LDS_ROW + piece);
 #pragma unroll
         for (int b = 0; b < MB; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wide_bf16x8(wf), wide_bf16x8(xf[b]), acc[a][b], 0, 0, 0);
@@ -336,6 +347,8 @@ extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_str
     if (tile == 2) TS_WIDE(2, 8, 2, 64);
     if (tile == 4) TS_WIDE(4, 8, 2, 64);
     if (tile == 5) TS_WIDE(5, 8, 2, 64);
+    // (tiles of 256 x 256 on four wavefronts, 128 x 128 outputs each, do not fit the registers
+    // beside two sets of staging registers: the compiler spills)
   } else if (waves == 8 && x_rows == 64) {
     if (tile == 2) TS_WIDE(2, 1, 4, 64);
     if (tile == 4) TS_WIDE(4, 1, 4, 64);

@@ -128,6 +128,43 @@ def test_tied_checkpoint_may_carry_the_head(tmp_path):
     assert model.head.weight is model.embedding.weight  # one tensor, as a tied head shares the table
 
 
+def test_a_model_never_holds_its_weights_twice(tmp_path):
+    """Nothing is read before the checks have passed; each tensor is read once, when its part asks
+    for it, and what a part has fused into a layout of its own is gone when the load returns."""
+    import weakref
+
+    from turboserve_amd.weights import loader
+
+    config, seed, _ = tiny.TINY["A"]  # tied: the head asks for the embedding's table again
+    folder = write_random_model(config, tmp_path, seed=seed)
+    reads: list[str] = []
+    handed_out: dict[str, weakref.ref] = {}
+    entries = []
+    for name, entry in loader.iter_checkpoint_entries(safetensors_files(folder)):
+        def read(name=name, entry=entry):
+            reads.append(name)
+            return entry.read()
+        entries.append((name, loader.StoredTensor(entry.shape, entry.dtype, read)))
+    model = cpu_model(config)
+    supply, report = load_tensors(model.tensor_specs(), iter(entries), dtype=torch.float32, device="cpu",
+                                  ignorable=model.ignorable_names())
+    assert report.ok and reads == []  # headers only so far
+    assert report.num_bytes == 4 * model.num_parameters()
+
+    class Watched(dict):
+        def __getitem__(self, name):
+            tensor = supply[name]
+            handed_out[name] = weakref.ref(tensor)
+            return tensor
+
+    model.load(Watched())
+    assert sorted(reads) == sorted(model.tensor_specs())  # each once; the tied table not a second time
+    assert model.head.weight is model.embedding.weight
+    fused = [n for n in handed_out if any(k in n for k in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj"))]
+    assert fused and all(handed_out[n]() is None for n in fused)
+    assert handed_out["model.layers.0.self_attn.o_proj.weight"]() is model.blocks[0].mixer.o_weight
+
+
 def test_random_model_is_a_function_of_config_and_seed(tmp_path):
     config, _, _ = tiny.TINY["B"]
     a = load_file(str(write_random_model(config, tmp_path / "a", seed=3) / "model.safetensors"))

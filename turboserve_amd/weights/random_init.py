@@ -79,18 +79,26 @@ def write_random_model(
 
 def random_tensors_on_device(model, seed: int, *, std: float = 0.02) -> None:
     """Fill ``model`` with N(0, std) weights drawn on its device (norm gains 1).  The values
-    differ from the folder mode's; the distributions are the same."""
+    differ from the folder mode's; the distributions are the same.  A tensor is drawn when a part
+    asks for it, from a generator seeded with ``seed`` and the tensor's place among the model's
+    tensors: the values do not depend on the order of asking, and the model never holds a
+    second copy of what its parts have fused."""
+    from turboserve_amd.weights.loader import TensorSupply
+
     runtime = model.runtime
-    generator = torch.Generator(device=runtime.device)
-    generator.manual_seed(int(seed))
-    tensors: dict[str, torch.Tensor] = {}
-    for name, spec in model.tensor_specs().items():
+    specs = model.tensor_specs()
+    places = {name: place for place, name in enumerate(specs)}
+
+    def make(name: str) -> torch.Tensor:
+        spec = specs[name]
         if spec.init == "ones":
-            tensors[name] = torch.ones(spec.shape, dtype=runtime.dtype, device=runtime.device)
-        elif spec.init == "zeros":
-            tensors[name] = torch.zeros(spec.shape, dtype=runtime.dtype, device=runtime.device)
-        else:
-            values = torch.empty(spec.shape, dtype=runtime.dtype, device=runtime.device)
-            values.normal_(0.0, std, generator=generator)
-            tensors[name] = values
-    model.load(tensors)
+            return torch.ones(spec.shape, dtype=runtime.dtype, device=runtime.device)
+        if spec.init == "zeros":
+            return torch.zeros(spec.shape, dtype=runtime.dtype, device=runtime.device)
+        generator = torch.Generator(device=runtime.device)
+        generator.manual_seed(int(seed) * 1_000_003 + places[name])
+        values = torch.empty(spec.shape, dtype=runtime.dtype, device=runtime.device)
+        values.normal_(0.0, std, generator=generator)
+        return values
+
+    model.load(TensorSupply(specs, make))

@@ -540,9 +540,14 @@ def main(argv: list[str] | None = None) -> int:
         return 0
     if args.only_prefill:
         seconds = run_prefill(model, config, args.only_prefill, tune=tune)
+        ops = model.runtime.ops
+        # What the start-up timing found for the step's products (device time of one launch).
+        products = {f"{n}x{k} at {rows} rows, {kind}": {"own_us": round(own * 1e3, 1), "library_us": round(library * 1e3, 1)}
+                    for (rows, n, k, kind), (own, library) in sorted(ops.wide_timings.items())}
         print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": args.only_prefill, "layers": layers,
                           "tokens_per_s": round(args.only_prefill / seconds, 1),
-                          "frac": round(prefill_flops(config, layers, args.only_prefill) / seconds / PEAK_FLOPS[dtype_key], 4)}))
+                          "frac": round(prefill_flops(config, layers, args.only_prefill) / seconds / PEAK_FLOPS[dtype_key], 4),
+                          "products": products}))
         return 0
 
     main_run = run_decode(model, config, args.batch, args.context - 1, steps=args.steps, warmup=args.warmup,

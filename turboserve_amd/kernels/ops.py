@@ -846,7 +846,7 @@ class Ops:
             return known
         iters = -(-k // 64)
         units = self.compute_units
-        unit_flops_per_us = 2.5e9 * 256 / units / 256  # a compute unit's share of the matrix peak, a microsecond
+        unit_flops_per_us = 2.5e9 / units  # a compute unit's share of the matrix peak (2.5 PFLOP/s), per microsecond
         best = None
         for tile, x_rows, rate in ((8, 256, 1.06), (5, 256, 0.92), (4, 256, 0.87), (5, 128, 0.75), (4, 128, 0.72)):
             if x_rows == 256 and m <= 128:
@@ -873,7 +873,7 @@ class Ops:
         untimed, up to ``wide_default_rows`` rows if the grid gives at least half of the compute
         units a workgroup.  With ``time_wide_choices`` an unknown product that is worth timing
         runs both ways here (``own()`` and ``library()``), four launches each behind a warm-up, each
-        waited for, the best by device events."""
+        waited for, the best by device events that see the device's time alone."""
         key = (self.library_rows(rows), n, k, kind)
         known = self.wide_choices.get(key)
         if known is not None:
@@ -883,8 +883,13 @@ class Ops:
             return rows <= self.wide_default_rows and (2 * workgroups >= self.compute_units or rows * n * k < self.library_tuning_min_work)
         # One launch at a time, each waited for: launches that follow one another without a
         # dependency overlap where a grid leaves compute units idle, and would look faster than
-        # they are inside a step.
+        # they are inside a step.  Each timed launch follows a kernel that keeps the device busy
+        # for longer than the host needs to issue it (clearing 256 MB: some 80 us), so that the
+        # events see the device's time alone: the host's own time per launch differs between a
+        # library call and this engine's (by more than a short product lasts) and is hidden
+        # inside a step, where the host runs ahead.
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        busy = torch.empty(1 << 26, dtype=torch.float32, device=self.device)
         times = []
         for run in (own, library):
             run()
@@ -892,12 +897,14 @@ class Ops:
             best = float("inf")
             for _ in range(4):
                 torch.cuda.synchronize(self.device)
+                busy.zero_()
                 start.record()
                 run()
                 stop.record()
                 stop.synchronize()
                 best = min(best, start.elapsed_time(stop))
             times.append(best)
+        del busy
         self.wide_choices[key] = times[0] <= times[1]
         self.wide_timings[key] = (times[0], times[1])
         return self.wide_choices[key]

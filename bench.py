@@ -543,7 +543,8 @@ def main(argv: list[str] | None = None) -> int:
         ops = model.runtime.ops
         # What the start-up timing found for the step's products (device time of one launch).
         products = {f"{n}x{k} at {rows} rows, {kind}": {"own_us": round(own * 1e3, 1), "library_us": round(library * 1e3, 1)}
-                    for (rows, n, k, kind), (own, library) in sorted(ops.wide_timings.items())}
+                    for (rows, n, k, kind), (own, library) in sorted(ops.wide_timings.items())
+                    if rows == ops.library_rows(args.only_prefill)}
         print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": args.only_prefill, "layers": layers,
                           "tokens_per_s": round(args.only_prefill / seconds, 1),
                           "frac": round(prefill_flops(config, layers, args.only_prefill) / seconds / PEAK_FLOPS[dtype_key], 4),

@@ -323,6 +323,49 @@ def test_timed_library_products_and_the_dry_step(model, tmp_path):
         torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
 
 
+def test_own_product_against_the_librarys_is_timed_once_and_remembered(tmp_path):
+    """A product of many rows that is worth timing runs both ways when asked to, the faster one
+    is kept, both give the product, and the next process (another ``Ops``) adopts the choice
+    from the file unless the file is of another state of the sources."""
+    import json
+
+    from turboserve_amd.kernels.gemm_tuning import OwnProductChoices
+    from turboserve_amd.kernels.ops import Ops
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(300, 1024, generator=g).bfloat16().to("cuda:0")
+    w = (torch.randn(1152, 1024, generator=g) / 32).bfloat16().to("cuda:0")
+    bias = torch.randn(1152, generator=g).bfloat16().to("cuda:0")
+    want = x.float() @ w.float().t() + bias.float()
+    ops = Ops("cuda:0")
+    ops.time_wide_choices = True
+    first = ops.linear(x, w, bias)
+    key = (300, 1152, 1024, "one")
+    assert set(ops.wide_timings) == {key} and all(0 < t < 50 for t in ops.wide_timings[key])
+    assert ops.wide_choices[key] == (ops.wide_timings[key][0] <= ops.wide_timings[key][1])
+    timings = dict(ops.wide_timings)
+    results = [first]
+    for forced in (True, False):
+        ops.wide_choices[key] = forced
+        results.append(ops.linear(x, w, bias))
+    assert ops.wide_timings == timings, "a known product is not timed again"
+    for got in results:
+        assert got.shape == want.shape and got.dtype == torch.bfloat16
+        torch.testing.assert_close(got.float().cpu(), want.cpu(), rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    ops.wide_choices[key] = timings[key][0] <= timings[key][1]
+    kept = OwnProductChoices(str(tmp_path / "choices.csv"), ops)
+    kept.save()
+    other = Ops("cuda:0")
+    assert OwnProductChoices(str(tmp_path / "choices.csv"), other).load() == 1
+    assert other.wide_choices == ops.wide_choices and other.wide_timings == ops.wide_timings
+    assert OwnProductChoices(str(tmp_path / "choices.csv"), other).load() == 0  # nothing new the second time
+    data = json.loads((tmp_path / "choices.csv.own.json").read_text())
+    data["stamp"]["source"] = "another state of the sources"
+    (tmp_path / "choices.csv.own.json").write_text(json.dumps(data))
+    assert OwnProductChoices(str(tmp_path / "choices.csv"), Ops("cuda:0")).load() == 0
+    assert OwnProductChoices(str(tmp_path / "absent.csv"), Ops("cuda:0")).load() == 0
+
+
 def test_library_products_at_timed_step_sizes(model, tmp_path, monkeypatch):
     """An engine told to run the library's products at a few timed sizes: prompts of lengths
     between the sizes, alone and cut into portions beside decoded tokens, give the plain

@@ -151,7 +151,7 @@ class LLMEngine:
         sizes (dry steps that leave the cache alone) and keep the fastest."""
         if self.model.runtime.dtype != torch.bfloat16:
             return  # the 32-bit path uses this engine's own product kernel
-        from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning
+        from turboserve_amd.kernels.gemm_tuning import LibraryGemmTuning, OwnProductChoices
 
         budget = self.config.scheduler.max_num_batched_tokens
         sizes = {min(t, budget) for t in self.config.tune_gemm_tokens}
@@ -171,10 +171,14 @@ class LLMEngine:
                     self.runner.dry_run(tokens)
             # ... then, with the library's winners in use and its timing mode off, every such
             # product runs both ways, by the library and by this engine's own kernel, and the
-            # faster one is kept (``Ops.wide_choices``).
+            # faster one is kept (``Ops.wide_choices``; what an earlier process found is read
+            # from a file beside the library's results and not timed again).
+            choices = OwnProductChoices(tuning.results_file, ops)
+            choices.load()
             ops.time_wide_choices = True
             for tokens in sorted(sizes):
                 self.runner.dry_run(tokens)
+            choices.save()
         finally:
             ops.time_wide_choices = False
             ops.wide_default_rows = own_rows

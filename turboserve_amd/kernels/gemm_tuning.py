@@ -23,6 +23,7 @@ never its precision: bfloat16 operands, 32-bit accumulation.
 
 from __future__ import annotations
 
+import json
 import os
 import tempfile
 
@@ -83,3 +84,54 @@ class LibraryGemmTuning:
     @staticmethod
     def num_results() -> int:
         return len(torch.cuda.tunable.get_results())
+
+
+class OwnProductChoices:
+    """What timing this engine's own product against the library's best kernel found
+    (``Ops.wide_choices``, ``Ops.wide_timings``), kept in a file beside the library's results so
+    that the next process starts from it: it decides as the one before did (a run under a
+    profiler, whose clock is not to be trusted, too) and spends no time on what is known.  The
+    file holds for one device and one state of the sources; anything else is ignored and
+    replaced."""
+
+    def __init__(self, results_file: str, ops) -> None:
+        self.path = results_file + ".own.json"
+        self.ops = ops
+
+    def _stamp(self) -> dict[str, str]:
+        from turboserve_amd.hwinfo import source_digest
+
+        return {"device": torch.cuda.get_device_name(self.ops.device), "torch": torch.__version__,
+                "source": source_digest()}
+
+    def load(self) -> int:
+        """Adopt the file's choices for products this process has not timed; how many."""
+        try:
+            with open(self.path, encoding="utf-8") as handle:
+                data = json.load(handle)
+        except (OSError, ValueError):
+            return 0
+        if not isinstance(data, dict) or data.get("stamp") != self._stamp():
+            return 0
+        adopted = 0
+        for entry in data.get("products", []):
+            try:
+                key = (int(entry["rows"]), int(entry["n"]), int(entry["k"]), str(entry["kind"]))
+                own, library = float(entry["own_ms"]), float(entry["library_ms"])
+            except (KeyError, TypeError, ValueError):
+                continue
+            if key not in self.ops.wide_choices:
+                self.ops.wide_choices[key] = own <= library
+                self.ops.wide_timings[key] = (own, library)
+                adopted += 1
+        return adopted
+
+    def save(self) -> None:
+        products = [{"rows": rows, "n": n, "k": k, "kind": kind, "own_ms": own, "library_ms": library}
+                    for (rows, n, k, kind), (own, library) in sorted(self.ops.wide_timings.items())]
+        try:
+            with open(self.path + ".tmp", "w", encoding="utf-8") as handle:
+                json.dump({"stamp": self._stamp(), "products": products}, handle)
+            os.replace(self.path + ".tmp", self.path)
+        except OSError:
+            pass  # a folder that cannot be written: the next process times again

@@ -884,12 +884,15 @@ class Ops:
         # One launch at a time, each waited for: launches that follow one another without a
         # dependency overlap where a grid leaves compute units idle, and would look faster than
         # they are inside a step.  Each timed launch follows a kernel that keeps the device busy
-        # for longer than the host needs to issue it (clearing 256 MB: some 80 us), so that the
-        # events see the device's time alone: the host's own time per launch differs between a
-        # library call and this engine's (by more than a short product lasts) and is hidden
-        # inside a step, where the host runs ahead.
+        # for longer than the host needs to issue it (reading 512 MB: some 80 us; reading, because
+        # a kernel that writes leaves the caches full of lines that go back to memory under the
+        # product), so that the events see the device's time alone: the host's own time per
+        # launch differs between a library call and this engine's (by more than a short
+        # product lasts) and is hidden inside a step, where the host runs ahead.
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        busy = torch.empty(1 << 26, dtype=torch.float32, device=self.device)
+        busy = torch.empty(1 << 27, dtype=torch.int32, device=self.device)
+        chunk = 16 * 4 * 256  # bytes a workgroup of the read-only kernel takes per iteration
+        count = busy.numel() * 4 // (1024 * chunk)
         times = []
         for run in (own, library):
             run()
@@ -897,7 +900,8 @@ class Ops:
             best = float("inf")
             for _ in range(4):
                 torch.cuda.synchronize(self.device)
-                busy.zero_()
+                self.hbm_read(busy, workgroups=1024, iters=count, pieces=4, ahead=2, wg_stride=count * chunk,
+                              it_stride=chunk, blk_rows=64, blk_stride=0, row_stride=256)
                 start.record()
                 run()
                 stop.record()

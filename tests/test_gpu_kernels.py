@@ -99,7 +99,8 @@ def test_embed_swiglu_gather(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 100), (16, 50, 64), (32, 33, 130), (33, 17, 65), (70, 65, 33), (130, 320, 96)])
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 100), (16, 50, 64), (32, 33, 130), (33, 17, 65), (70, 65, 33), (130, 320, 96),
+                                   (97, 129, 17), (300, 257, 200)])
 def test_gemm_plain(ops, dtype, m, n, k):
     g = torch.Generator().manual_seed(m * n)
     x = torch.randn(m, k, generator=g).to(dtype)
@@ -123,11 +124,12 @@ def test_gemm_plain_rows_do_not_depend_on_the_batch(ops, dtype, k):
     32 rows, one output a thread), among many (tiles of 64 x 64): every output is the same chain
     of fused multiply-adds in the order of k in both layouts."""
     g = torch.Generator().manual_seed(9)
-    x = torch.randn(77, k, generator=g).to(dtype)
+    x = torch.randn(300, k, generator=g).to(dtype)
     w = torch.randn(150, k, generator=g).to(dtype)
     b = torch.randn(150, generator=g).to(dtype)
     full = ops.gemm_plain(x.to(DEV), w.to(DEV), b.to(DEV)).cpu()
-    for rows in (slice(40, 41), slice(0, 8), slice(20, 45), slice(3, 35), slice(10, 43), slice(0, 64)):
+    for rows in (slice(40, 41), slice(0, 8), slice(20, 45), slice(3, 35), slice(10, 43), slice(0, 64), slice(100, 196),
+                 slice(7, 104), slice(150, 300)):
         part = ops.gemm_plain(x[rows].to(DEV), w.to(DEV), b.to(DEV)).cpu()
         assert torch.equal(full[rows], part), rows
 

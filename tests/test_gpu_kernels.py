@@ -162,13 +162,19 @@ def test_gemm_skinny(ops, m, n, k):
     torch.testing.assert_close(none, b.float().expand(m, n), rtol=0, atol=0)  # the bias, once
 
 
-@pytest.mark.parametrize("tile", [2, 4, 5])
+@pytest.mark.parametrize("tile", [2, 4, 5, 8])
 @pytest.mark.parametrize("m,n,k", [(64, 500, 1096), (3, 161, 128), (16, 200, 392), (17, 333, 264), (32, 96, 1096), (40, 64, 40),
                                    (128, 330, 520), (77, 1000, 264)])
 def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
     """The tiled product with its grid given by hand: every tile size, ranges of K of one
     iteration and of several, a last range that is shorter, a last tile of rows that is partly
-    beyond N, a K below one iteration."""
+    beyond N, a K below one iteration.  Tiles of 256 weight rows take up to 32 rows and refuse
+    more."""
+    if tile == 8 and m > 32:
+        x = torch.zeros(m, k).bfloat16().to(DEV)
+        with pytest.raises(Exception, match="ts_gemm_tiled"):
+            ops.gemm_tiled(x, torch.zeros(n, k).bfloat16().to(DEV), plan=(-(-k // 128), 1, tile))
+        return
     g = torch.Generator().manual_seed(tile * 1000 + n)
     x = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
@@ -182,9 +188,8 @@ def test_gemm_tiled_every_tile_and_grid(ops, tile, m, n, k):
         assert float((got - want).abs().max()) <= 2e-5 * math.sqrt(k) * float(want.abs().max() + 1), per_split
 
 
-@pytest.mark.parametrize("tile", [2, 4, 5])
-@pytest.mark.parametrize("m,inter,k", [(64, 250, 264), (5, 81, 128), (16, 81, 392), (24, 250, 264), (33, 1000, 40), (128, 250, 264),
-                                       (90, 81, 128)])
+@pytest.mark.parametrize("tile,m,inter,k", [(t, *c) for t in (2, 4, 5, 8) for c in (
+    (64, 250, 264), (5, 81, 128), (16, 81, 392), (24, 250, 264), (33, 1000, 40), (128, 250, 264), (90, 81, 128)) if t != 8 or c[0] <= 32])
 def test_gemm_tiled_applies_swiglu_itself(ops, tile, m, inter, k):
     """A gate|up matrix with alternating rows through the tiled product with the activation in
     its epilogue gives, bit for bit, what the product's partial sums followed by the SwiGLU

@@ -7,7 +7,7 @@
 // The product is bound by reading W once from HBM, and what decides its rate is how the reading
 // is spread over the device, not how much of it is in flight:
 //   * a workgroup of four wavefronts (2 x 2) owns a tile of NT = 32 TN weight rows (TN = 2, 4
-//     or 5) by all activation rows (16 of them, 32 when M > 16, 64 when M > 32, 128 when M > 64: rows beyond M
+//     or 5; 8 for up to 32 activation rows) by all activation rows (16 of them, 32 when M > 16, 64 when M > 32, 128 when M > 64: rows beyond M
 //     are repeats that cost loads and LDS writes, so the tile is no larger than it must be) and
 //     one range of K; the host
 //     sizes tiles and ranges so that
@@ -237,12 +237,27 @@ int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stri
   return launch_tiled_rows<TN, 4>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
 }
 
+// Tiles of 256 weight rows (TN = 8): with more than 32 activation rows two buffers no longer fit
+// the LDS of a compute unit.
+constexpr int M_MAX_TALL = 32;
+
+template <int TN>
+int launch_tiled_tall(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
+                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+  if (m <= 16)
+    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+  if (m <= M_MAX_TALL)
+    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+  return TS_ERR_SHAPE;
+}
+
 }  // namespace
 
 // partial [splits, m, n] float (contiguous); x [m, k] bfloat16 with row stride x_stride;
 // w [n, k] bfloat16 contiguous; bias [n] bfloat16 or null.  Needs m <= 128, k % 8 == 0.
 // iters_per_split iterations of 128 of k go to each of `splits` = ceil(ceil(k / 128) / iters_per_split).
-// tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows).
+// tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows),
+// or, for m <= 32, 8 (256 rows).
 // gated (bfloat16 [m, n / 2], contiguous) instead of partial: w is a gate|up projection whose rows
 // alternate gate, up, and the kernel writes silu(gate) * up; needs splits == 1, no bias, n even.
 extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_stride, const void* w,
@@ -262,5 +277,6 @@ extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_
   if (tile == 2) return launch_tiled<2>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
   if (tile == 4) return launch_tiled<4>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
   if (tile == 5) return launch_tiled<5>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 8) return launch_tiled_tall<8>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
   return TS_ERR_SHAPE;
 }

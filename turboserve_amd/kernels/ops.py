@@ -749,8 +749,13 @@ class Ops:
         iters = -(-k // 128)
         limit = min(iters, max_splits or 32)
         best = None
-        for tile in (5, 4, 2):
-            for want in range(1, limit + 1):
+        for tile in (8, 5, 4, 2):
+            # Tiles of 256 weight rows leave LDS for 32 activation rows, and pay where one range
+            # of K as one round of them replaces nearly two rounds of smaller tiles; in grids of
+            # several rounds or ranges they measured slower than the others.
+            if tile == 8 and (m > 32 or -(-n // 256) > self.compute_units):
+                continue
+            for want in range(1, (1 if tile == 8 else limit) + 1):
                 per_split = -(-iters // want)
                 splits = -(-iters // per_split)
                 if splits != want:
@@ -766,13 +771,17 @@ class Ops:
         compute unit one after the other.  A compute unit holds one workgroup of the larger tiles
         (their LDS fills it) or, up to 64 activation rows, two of the smallest, and streams the
         faster the more weight rows it has in flight: 64 rows (one small workgroup) count as 1,
-        two small workgroups as 1.25, a tile of 128 as 1.21, of 160 as 1.27.  With more than 32
+        two small workgroups as 1.25, a tile of 128 as 1.21, of 160 as 1.27, of 256 (one range of
+        K in one round only) as 1.26 (the 72B shape's gate|up, 59,136 rows by 8,192, at eight rows:
+        231 tiles of 256 rows 152 us, 462 of 128 169 us, 924 of 64 211 us; the 32B shape's, 55,296
+        by 5,120: 216 of 256 93 us, 432 of 128 90 us).  With more than 32
         distinct activation rows two workgroups on a unit get in each other's way (at 64 rows the
         pair is slower than one after the other).  Workgroups beyond what the device holds at
         once wait for a later round, which starts on a busy device, unevenly.  Every workgroup
         pays one more iteration for starting up; partial sums are written here and read by the
         consumer.  Fitted to steps of the 7B and 14B shapes at 8, 32 and 64 rows, measured
-        through the engine with each product's grid varied in turn, and to kernel traces of them."""
+        through the engine with each product's grid varied in turn, and to kernel traces of them;
+        the 32B shape's widest matrix added the rule for a later round that is not full."""
         rows = 32 * tile
         units = self.compute_units
         workgroups = -(-n // rows) * splits
@@ -784,11 +793,17 @@ class Ops:
             if tile == 2:
                 doubled = max(0, count - units) / units if pairs else 0.0  # share of the units that hold two
                 return stretch * (1.0 + pair_extra * doubled)
-            return stretch / (1.21 if tile == 4 else 1.27)
+            return stretch / {4: 1.21, 5: 1.27, 8: 1.26}[tile]
 
         held = units * (2 if pairs else 1)
         full, rest = divmod(workgroups, held)
         cost = full * round_cost(held) + (round_cost(rest) if rest else 0.0)
+        if tile != 2 and full >= 1 and rest:
+            # A later round of the larger tiles that does not fill the device: its workgroups share
+            # the memory among fewer and finish sooner, down to about 0.7 of the units busy, which
+            # is what it takes to saturate the memory (the 32B shape's gate|up, 432 tiles of 128
+            # rows: 90 us at eight rows, as if it were 1.7 rounds; 346 tiles of 160: 112 us).
+            cost = full * round_cost(held) + round_cost(rest) * max(rest / held, 0.7)
         rounds = full + (1 if rest else 0)
         cost *= 1.0 + 0.1 * (rounds - 1)
         cost *= 1.0 + 3.0 * splits * m / k
@@ -991,24 +1006,56 @@ class Ops:
         before's products) instead of the tiled one: above 32 rows always (7B shape, alone, at 64
         rows: gate|up 46.7 against 50.1 us, down 27.6 against 29.3, q|k|v 10.7 against 14.4, o 9.5
         against 10.6, the head 209 against 221; at 128 rows: 59 against 72, 35 against 39, 14
-        against 16, 246 against 282), from 17 rows for a matrix that fills the device as one range
-        of K and once over (gate|up at 32 rows: 45.3 against 47.8 us)."""
+        against 16, 246 against 282), from 17 rows for a matrix that runs as one range of K and
+        whose best grid is at most two rounds of workgroups (gate|up at 24 to 32 rows, 7B / 14B /
+        32B shape: 47.4 / 50.4 / 97.4 us against the tiled kernel's 48.7 / 51.7 / 99.9)."""
         if m > 32:
             return True
-        tiles = -(-n // 160)
-        return m > 16 and max_splits == 1 and 9 * self.compute_units <= 10 * tiles <= 20 * self.compute_units
+        if m <= 16 or max_splits != 1:
+            return False
+        tile = self._one_range_tile(n, 64)
+        return 8 * self.compute_units <= 10 * -(-n // (32 * tile)) <= 20 * self.compute_units * (2 if tile == 2 else 1)
+
+    #: Weight rows a compute unit streams per microsecond through the wide kernel at up to 128
+    #: activation rows and K = 5,120, by tile (tiles of 64 rows: two workgroups a unit).  Larger
+    #: tiles have more in flight and stream faster.  From the gate|up matrices of the 7B, 14B, 32B
+    #: and 72B shapes at 64 rows, each timed with every tile.
+    _ONE_RANGE_RATES = {2: 1.7, 4: 2.04, 5: 2.28, 8: 2.62}
+
+    def _one_range_tile(self, n: int, x_rows: int) -> int:
+        """The tile (in 32 weight rows) with which the wide kernel streams ``n`` weight rows as one
+        range of K soonest: what a unit streams per round at that tile's rate, times the rounds
+        of workgroups, a later round that is not full counting for what is in it but for no less
+        than 0.7 (about that share of the units busy saturates the memory).  Measured against
+        it at 64 rows (us, model / kernel): 7B shape, 37,888 rows: tile 5 49 / 49, tile 8 68 / 62,
+        tile 4 75 / 67; 14B, 27,648: tile 4 63 / 54, 5 70 / 60, 8 98 / 99; 32B, 55,296: 8 98 / 98,
+        4 107 / 106, 5 119 / 119, 2 128 / 126; 72B, 59,136 by 8,192: 8 156 / 157, 4 180 / 189, 5 191 / 196."""
+        units = self.compute_units
+        best = None
+        for tile, rate in self._ONE_RANGE_RATES.items():
+            held = units * (2 if tile == 2 else 1)
+            full, rest = divmod(-(-n // (32 * tile)), held)
+            rounds = 1.0 if full == 0 else full + (max(rest / held, 0.7) if rest else 0.0)
+            cost = rounds * 32 * tile * (2 if tile == 2 else 1) / rate
+            if best is None or cost < best[0]:
+                best = (cost, tile)
+        return best[1]
 
     def _wide_plan_few_rows(self, m: int, n: int, k: int, max_splits: int | None) -> tuple[int, int, int, int, int, int]:
         """The wide product's grid for up to 128 rows, where reading the weights sets the pace: one
-        tile of 64 or 128 activation rows; iterations 128 deep under the tiles of 64 rows (half as
-        many barriers; the head, whose grid runs in several rounds, is faster 64 deep); tiles of
-        160 weight rows if those alone give nearly every compute unit a workgroup (one range of
-        K), else tiles of 128 and as many ranges of K as it takes to give every compute unit one."""
+        tile of 64 or 128 activation rows; as one range of K (a consumer that wants one result:
+        the gated product, the head) the tile of weight rows that fills the device's rounds best
+        (``_one_range_tile``), iterations 128 deep under the tiles of 64 activation rows (half as
+        many barriers; the head, whose grid runs in several rounds, and tiles of 256 weight rows,
+        whose LDS it would not fit, are 64 deep); else tiles of 128 and as many ranges of K as it
+        takes to give every compute unit one."""
         x_rows = 64 if m <= 64 else 128
-        depth = 128 if x_rows == 64 and -(-n // 160) <= 2 * self.compute_units else 64
+        if max_splits == 1 or 10 * -(-n // 160) >= 9 * self.compute_units:
+            tile = self._one_range_tile(n, x_rows)
+            depth = 128 if x_rows == 64 and tile != 8 and -(-n // 160) <= 2 * self.compute_units else 64
+            return -(-k // depth), 1, tile, x_rows, 8, depth
+        depth = 128 if x_rows == 64 else 64
         iters = -(-k // depth)
-        if 10 * -(-n // 160) >= 9 * self.compute_units:
-            return iters, 1, 5, x_rows, 8, depth
         want = max(1, min(iters, max_splits or iters, self.compute_units // -(-n // 128)))
         per_split = -(-iters // want)
         return per_split, -(-iters // per_split), 4, x_rows, 8, depth

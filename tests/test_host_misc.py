@@ -426,6 +426,19 @@ def test_tiled_product_plans_are_the_ones_measured_best():
     assert plan(8, 7168, h14, None) == (10, 4, 2)         # 14B qkv: four ranges, two workgroups a unit
     assert plan(8, 2 * i14, h14, None) == (40, 1, 2)      # 14B gate+up: 432 small workgroups
     assert plan(128, h7, i7, None)[2] != 2                # above 64 rows LDS holds one workgroup: no pairs to count on
+    assert plan(8, 2 * 27648, 5120, None) == (40, 1, 4)   # 32B gate+up: 432 tiles of 128 (1.7 rounds), not 864 of 64
+    assert plan(8, 2 * 29568, 8192, None) == (64, 1, 8)   # 72B gate+up: 231 tiles of 256, one round
+    assert plan(8, 152064, 8192, 1)[2] != 8 and plan(8, h7, i7, None)[2] != 8  # tiles of 256: one range in one round only
+    assert plan(40, 2 * 29568, 8192, None)[2] != 8        # and up to 32 rows
+    # The wide kernel's tile for one range of K at 17 to 128 rows: what was fastest of all tiles
+    # for the gate|up matrices of the 7B, 14B, 32B and 72B shapes.
+    tile = Planner()._one_range_tile
+    assert [tile(n, 64) for n in (2 * i7, 2 * i14, 2 * 27648, 2 * 29568)] == [5, 4, 8, 8]
+    wide = Planner()._wide_plan_few_rows
+    assert wide(64, 2 * i7, h7, 1) == (28, 1, 5, 64, 8, 128) and wide(128, 2 * i7, h7, 1) == (56, 1, 5, 128, 8, 64)
+    assert wide(64, 2 * 27648, 5120, 1) == (80, 1, 8, 64, 8, 64)  # tiles of 256 weight rows are 64 deep
+    assert wide(64, 152064, h7, 1)[2:] == (5, 64, 8, 64)          # the head: several rounds, 64 deep
+    assert wide(64, h7, i7, None) == (17, 9, 4, 64, 8, 128)       # down: ranges of K, tiles of 128
 
 
 def test_library_products_run_at_a_few_sizes():

@@ -79,8 +79,9 @@ gemm_plain_kernel(TOut* __restrict__ y, const TIn* __restrict__ x, const TIn* __
 // owns 16 x 16 outputs, one per thread, and walks K in slices of 64 that travel global ->
 // registers -> LDS (two buffers, one barrier a slice); a thread fetches four consecutive k of one
 // row (one 16-byte load where K allows), so a row's slice is 256 contiguous bytes, and its loads
-// are GF_AHEAD slices ahead of the arithmetic (a ring of registers).  Every load is unconditional (addresses clamped into the tensor, what lies
-// outside replaced by zero afterwards), so that the compiler can count the loads in flight.
+// are GF_AHEAD slices ahead of the arithmetic (a ring of registers).  Every load is unconditional
+// (addresses clamped into the tensor, what lies outside replaced by zero afterwards), so that
+// the compiler can count the loads in flight.
 #define GF_BM 16
 #define GF_BN 16
 #define GF_BK 64

@@ -19,9 +19,11 @@ gets from this device, ``read_probe``); ``points`` holds decode at batch 1 and 6
 context, the benchmark's literal workload (prompts of 512 tokens, 256 generated,
 end-of-sequence ignored, greedy) at 1, 8 and 64 requests, with the details of those runs under
 ``workload``, and further sizes, detailed under ``further``: prompts of 8,192 and 32,767 tokens
-in portions of 2,048, and decode at batch 1 and 8 with about 32 k tokens of context.  The
-prefill's projections are BLAS-library products; which of the library's kernels runs each is
-timed once at the engine's start (``--no-gemm-tuning`` leaves it to the library's heuristic).
+in portions of 2,048, decode at batch 1 and 8 with about 32 k tokens of context, and the
+default decode step at the 14B and 32B shapes (all of their layers).  A prefill's projections
+are this engine's own product or the BLAS library's, whichever is the faster one for the shape:
+both are timed once at the engine's start (``--no-gemm-tuning`` leaves the library's kernels to
+its heuristic and the choice to a rule).
 Peaks are the published MI355X figures: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3
 TFLOP/s.
 
@@ -112,7 +114,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                    help="time a kernel that only reads, walking memory in several ways with plain and non-temporal "
                         "loads (what the memory gives: the practical ceiling of the decode step), and exit")
     p.add_argument("--no-further", action="store_true",
-                   help="skip the further sizes: prefill of 8,192 and 32,767 tokens, decode at 32 k tokens of context")
+                   help="skip the further sizes: prefill of 8,192 and 32,767 tokens, decode at 32 k tokens of context, "
+                        "the decode step at the 14B and 32B shapes")
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
@@ -661,6 +664,24 @@ def main(argv: list[str] | None = None) -> int:
             further[f"decode_b{batch}_ctx{LONG_CONTEXT}"] = {
                 "ms_per_step": round(run["step_seconds"] * 1e3, 4), "mean_context": round(run["mean_context"], 1),
                 "hbm_frac": round(read / run["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4)}
+        # The same decode step at the two wider shapes of the family (all of their layers), so that
+        # their figures are taken by whoever runs this, not only quoted.
+        del model
+        for other in ("14b", "32b"):
+            other_name, other_shape = SHAPES[other]
+            torch.cuda.empty_cache()
+            other_config, other_model = build_model(dict(other_shape), runtime)
+            random_tensors_on_device(other_model, seed=0)
+            steps, warmup = 16, 8
+            run = run_decode(other_model, other_config, args.batch, args.context - 1, steps=steps, warmup=warmup,
+                             run_ahead=run_ahead)
+            read = decode_bytes(other_config, other_config.num_hidden_layers, args.batch, run["mean_context"], itemsize)
+            result["points"][f"decode_b{args.batch}_{other}"] = round(run["tokens_per_s"], 2)
+            further[f"decode_b{args.batch}_{other}"] = {
+                "model": f"{other_name} shape", "layers": other_config.num_hidden_layers,
+                "ms_per_step": round(run["step_seconds"] * 1e3, 4), "mean_context": round(run["mean_context"], 1),
+                "hbm_frac": round(read / run["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4)}
+            del other_model
         result["further"] = further
     if not args.no_points:
         # What a kernel that only reads gets from this device's memory: the decode step's practical ceiling.

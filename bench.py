@@ -20,7 +20,8 @@ context, the benchmark's literal workload (prompts of 512 tokens, 256 generated,
 end-of-sequence ignored, greedy) at 1, 8 and 64 requests, with the details of those runs under
 ``workload``, and further sizes, detailed under ``further``: prompts of 8,192 and 32,767 tokens
 in portions of 2,048, decode at batch 1 and 8 with about 32 k tokens of context, and the
-default decode step at the 14B and 32B shapes (all of their layers).  A prefill's projections
+default decode step at the 14B and 32B shapes (all of their layers) and the 14B shape's mixed
+step (32 decode tokens and one 2,048-token prompt).  A prefill's projections
 are this engine's own product or the BLAS library's, whichever is the faster one for the shape:
 both are timed once at the engine's start (``--no-gemm-tuning`` leaves the library's kernels to
 its heuristic and the choice to a rule).
@@ -681,6 +682,21 @@ def main(argv: list[str] | None = None) -> int:
                 "model": f"{other_name} shape", "layers": other_config.num_hidden_layers,
                 "ms_per_step": round(run["step_seconds"] * 1e3, 4), "mean_context": round(run["mean_context"], 1),
                 "hbm_frac": round(read / run["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4)}
+            if other == "14b":
+                # The 14B shape's mixed step: 32 decode tokens (context as above) and one whole
+                # 2,048-token prompt in every step.
+                mixed_batch = 32
+                run = run_decode(other_model, other_config, mixed_batch, args.context - 1, steps=12, warmup=4,
+                                 mixed_prefill=PREFILL_TOKENS, tune=tune, run_ahead=run_ahead)
+                other_layers = other_config.num_hidden_layers
+                flops = (prefill_flops(other_config, other_layers, PREFILL_TOKENS)
+                         + 2.0 * mixed_batch * decode_bytes(other_config, other_layers, 0, 0, 1)
+                         + 4.0 * mixed_batch * other_layers * other_config.q_proj_size * args.context)
+                result["points"][f"mixed_b{mixed_batch}_prompt{PREFILL_TOKENS}_{other}"] = round(
+                    (mixed_batch + PREFILL_TOKENS) / run["step_seconds"], 1)
+                further[f"mixed_b{mixed_batch}_prompt{PREFILL_TOKENS}_{other}"] = {
+                    "model": f"{other_name} shape", "ms_per_step": round(run["step_seconds"] * 1e3, 3),
+                    "flops_frac": round(flops / run["step_seconds"] / PEAK_FLOPS[dtype_key], 4)}
             del other_model
         result["further"] = further
     if not args.no_points:
